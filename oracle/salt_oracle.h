@@ -1,0 +1,144 @@
+/* salt_oracle.h -- CPU restatement of SALT's quantized decode arithmetic.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing in the shipped library links, loads or
+ * calls this code: it exists so that the parity tests, the smoke check and
+ * the CPU-baseline leg of the benchmark have an independent statement of the
+ * reference algorithm to compare the HIP kernels against.
+ *
+ * Every function names the reference lines it restates.  All arithmetic is
+ * IEEE binary32 with one rounding per operator; build with
+ * -ffp-contract=off (the Makefile next to this file does).
+ */
+#ifndef SALT_ORACLE_H
+#define SALT_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- affine Q4 ("mlx4"): u32 words of 8 nibbles, bf16 scale+bias per 64 */
+
+/* reference src/kernels.c:118-123 */
+float orc_bf16(uint16_t half);
+/* reference src/kernels.c:188-208 (salt_q4_decode) */
+void orc_q4_decode(const void *vals, const void *scales, const void *biases,
+                   size_t n, float *out);
+/* reference src/kernels.c:220-250 (q4_canonical_row) */
+float orc_q4_row(const void *vals, const void *scales, const void *biases,
+                 int C, const float *x, int row);
+/* reference src/kernels.c:252-274, 283-335 (validation + row loop) */
+int orc_q4_matvec(const void *vals, const void *scales, const void *biases,
+                  int R, int C, const float *x, float *y);
+int orc_q4_matvec_rows(const void *vals, const void *scales,
+                       const void *biases, int R, int C, const float *x,
+                       float *y, int r0, int r1);
+/* reference src/kernels.c:1252-1306: ys[t*R+r] = row r against xs[t*C..] */
+int orc_q4_matvec_batch(const void *vals, const void *scales,
+                        const void *biases, int R, int C, int B,
+                        const float *xs, float *ys);
+/* Row-split over `threads` pthreads by the reference's rule
+ * (chunk = ceil(R/threads), src/kernels.c:291-323).  Same bits as the
+ * single-thread call; used for the timed CPU baseline. */
+int orc_q4_matvec_threads(const void *vals, const void *scales,
+                          const void *biases, int R, int C, const float *x,
+                          float *y, int threads);
+
+/* ---- NVFP4: packed E2M1 codes, E4M3FN block scale per 16, fp32 divisor */
+
+/* reference src/nvfp4.c:19-23 */
+float orc_e2m1(uint8_t code);
+/* reference src/nvfp4.c:25-39 */
+float orc_e4m3fn(uint8_t code);
+/* reference src/nvfp4.c:41-63 (argmin scan, ties to even code) */
+int orc_e4m3fn_encode(float value, uint8_t *code);
+/* reference src/nvfp4.c:65-80 */
+uint8_t orc_e2m1_encode(float value);
+/* Closed-form round-to-nearest-even encoders; the HIP kernels use the same
+ * closed forms, and the tests prove them equal to the scans above. */
+uint8_t orc_e4m3fn_encode_rne(float value);
+uint8_t orc_e2m1_encode_rne(float value);
+/* reference src/nvfp4.c:82-130 */
+int orc_nvfp4_qdq(const float *input, int C, float input_global_scale,
+                  uint8_t *packed, uint8_t *scales, float *dequant);
+/* reference src/nvfp4.c:132-155 */
+int orc_nvfp4_dequant_weights(const uint8_t *packed, const uint8_t *scales,
+                              float stored_divisor, int R, int C, float *out);
+/* reference src/nvfp4.c:157-192 (row with a given dequantised activation) */
+float orc_nvfp4_row(const uint8_t *packed, const uint8_t *scales,
+                    float weight_global_scale, int row, int C,
+                    const float *x_dq);
+/* reference src/nvfp4.c:228-256 */
+int orc_nvfp4_matvec(const uint8_t *packed, const uint8_t *scales,
+                     float stored_divisor, float input_global_scale,
+                     int R, int C, const float *input, float *output,
+                     uint8_t *x_packed, uint8_t *x_scales, float *x_dq);
+/* Rows against an activation that is used as given (no Q/DQ pre-pass). */
+int orc_nvfp4_matvec_weights_only(const uint8_t *packed,
+                                  const uint8_t *scales, float stored_divisor,
+                                  int R, int C, const float *x, float *output);
+
+/* ---- deterministic transcendentals */
+
+/* reference src/bitmath.c:44-63 */
+float orc_expf(float x);
+/* reference src/bitmath.c:144-153 */
+float orc_tanhf(float x);
+/* reference models/gemma4-26b-a4b/src/gemma4.c:80-83 */
+float orc_gelu_tanh(float x);
+
+/* ---- routers */
+
+/* reference models/gemma4-26b-a4b/src/gemma4.c:132-186 */
+int orc_router_topk(const float *logits, const float *per_expert_scale,
+                    int n_experts, int topk, int *selected, float *weights);
+/* reference models/gemma4-26b-a4b/src/gemma4_text.c:7923-7930 */
+void orc_sort_selection(int *selected, float *weights, int topk);
+/* reference src/router.c:11-20 */
+uint64_t orc_mix64(uint64_t x);
+/* reference src/router.c:22-57 (fixture router) */
+int orc_router_fixture(int *idx, float *w, int n_experts, int topk,
+                       uint64_t state, int layer, double locality);
+
+/* ---- routed expert FFN and MoE layer */
+
+/* Byte geometry of one expert in the pool: [gate|up|down], each projection
+ * [vals|scales|biases] (reference gemma4_text.c:73-79, 7608-7612). */
+typedef struct OrcExpertGeometry {
+    int hidden;      /* d_model, columns of gate/up, rows of down   */
+    int routed;      /* d_ff, rows of gate/up, columns of down      */
+} OrcExpertGeometry;
+size_t orc_expert_proj_bytes(const OrcExpertGeometry *g);
+size_t orc_expert_slot_bytes(const OrcExpertGeometry *g);
+
+/* reference gemma4_text.c:7608-7649 (expert_worker): gate, up, gelu*up,
+ * down.  gate/up scratch hold `routed` floats, output `hidden` floats. */
+int orc_expert_ffn(const OrcExpertGeometry *g, const unsigned char *slot,
+                   const float *input, float *gate, float *up, float *output);
+/* One decode layer-step: router top-k, ascending sort, the selected
+ * experts, and the in-order weighted sum (reference gemma4_text.c:8360,
+ * 7923-7930, 7608-7649, 8301-8304).  pool points at expert 0 of the layer;
+ * experts are orc_expert_slot_bytes apart.  expert_out (optional) receives
+ * the topk per-expert outputs [topk][hidden] in sorted order. */
+int orc_moe_decode_step(const OrcExpertGeometry *g, const unsigned char *pool,
+                        int n_experts, int topk, const float *logits,
+                        const float *per_expert_scale, const float *input,
+                        int *selected, float *weights, float *expert_out,
+                        float *output, int threads);
+/* Grouped prefill MoE: validation, ascending-expert / token / rank row
+ * order, per-expert batch FFN, scatter to [token][rank] slots, in-order
+ * weighted reduce (reference src/moe_group.c:83-97, 138-224 with the Gemma
+ * group ops gemma4_text.c:8749-9137 doing gate/up -> gelu*up -> down).
+ * group_rows (optional, n_experts ints) receives each expert's row count. */
+int orc_moe_group(const OrcExpertGeometry *g, const unsigned char *pool,
+                  int n_experts, int topk, int batch, const int *selected,
+                  const float *weights, const float *inputs, float *outputs,
+                  int *group_rows, int threads);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* SALT_ORACLE_H */
