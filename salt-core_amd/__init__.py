@@ -5,4 +5,4 @@ this Python package only loads it through ctypes for tests and the benchmark.
 The directory name carries a hyphen, so it is imported under the module name
 ``salt_core_amd`` (see ``__graft_entry__.load_package``).
 """
-from . import synth  # noqa: F401
+from . import lib, synth  # noqa: F401

@@ -1,0 +1,251 @@
+// Library state, diagnostics, device helpers and the device-resident Q4 entry
+// points of libsalt_gpu_mi355.so.
+#include "backend_state.h"
+
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+namespace mi355 {
+
+State g_state;
+
+void set_error(const char *format, ...) {
+    va_list args;
+    va_start(args, format);
+    vsnprintf(g_state.last_error, sizeof g_state.last_error, format, args);
+    va_end(args);
+    if (getenv("SALT_GPU_DIAG")) fprintf(stderr, "salt-mi355: %s\n", g_state.last_error);
+}
+
+int hip_ok(hipError_t status, const char *what) {
+    if (status == hipSuccess) return 0;
+    set_error("%s: %s", what, hipGetErrorString(status));
+    return -1;
+}
+
+namespace {
+
+// What the kernels assume of the two converters, checked once on the device:
+// a byte 0..15 through the fp8 converter is an exact multiple k * v(1) of the
+// value it gives byte 1 (a power of two), and every fp4 code decodes to the
+// E2M1 magnitude with its sign.
+int verify_converters() {
+    float *device = nullptr;
+    if (hip_ok(hipMalloc((void **)&device, (256 + 512) * sizeof(float)), "hipMalloc probe") != 0) return -1;
+    int rc = probe_converters_launch(device, device + 256, g_state.stream);
+    if (rc == 0) rc = hip_ok(hipStreamSynchronize(g_state.stream), "converter probe");
+    if (rc == 0)
+        rc = hip_ok(hipMemcpy(g_state.fp8_table, device, 256 * sizeof(float), hipMemcpyDeviceToHost), "probe copy");
+    if (rc == 0)
+        rc = hip_ok(hipMemcpy(g_state.fp4_table, device + 256, 512 * sizeof(float), hipMemcpyDeviceToHost),
+                    "probe copy");
+    hipFree(device);
+    if (rc != 0) return -1;
+    const float unit = g_state.fp8_table[1];
+    int exponent = 0;
+    if (!(unit > 0.0f) || frexpf(unit, &exponent) != 0.5f) {
+        set_error("fp8 converter: byte 1 decodes to %g, not a power of two", (double)unit);
+        return -1;
+    }
+    for (int k = 0; k < 16; ++k)
+        if (g_state.fp8_table[k] != (float)k * unit) {
+            set_error("fp8 converter: byte %d decodes to %g, expected %g", k, (double)g_state.fp8_table[k],
+                      (double)((float)k * unit));
+            return -1;
+        }
+    g_state.code_scale = 1.0f / unit;
+    static const float magnitude[8] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
+    for (int byte = 0; byte < 256; ++byte)
+        for (int half = 0; half < 2; ++half) {
+            const int code = half ? byte >> 4 : byte & 15;
+            const float want = (code & 8) ? -magnitude[code & 7] : magnitude[code & 7];
+            if (g_state.fp4_table[2 * byte + half] != want) {   // -0 == +0 here on purpose
+                set_error("fp4 converter: code %d decodes to %g, expected %g", code,
+                          (double)g_state.fp4_table[2 * byte + half], (double)want);
+                return -1;
+            }
+        }
+    return 0;
+}
+
+}  // namespace
+
+// Grows the device copy of a host job table; returns the device pointer.
+void *stage_table(const void *host_table, size_t nbytes, hipStream_t stream) {
+    State &s = g_state;
+    if (nbytes > s.table_capacity) {
+        if (s.table_device) {
+            if (hip_ok(hipDeviceSynchronize(), "sync before table growth") != 0) return nullptr;
+            hipFree(s.table_device);
+            hipHostFree(s.table_pinned);
+            s.table_device = nullptr; s.table_pinned = nullptr; s.table_capacity = 0;
+        }
+        size_t capacity = 64 * 1024;
+        while (capacity < nbytes) capacity *= 2;
+        if (hip_ok(hipMalloc(&s.table_device, capacity), "hipMalloc job table") != 0 ||
+            hip_ok(hipHostMalloc(&s.table_pinned, capacity, hipHostMallocDefault), "hipHostMalloc job table") != 0)
+            return nullptr;
+        s.table_capacity = capacity;
+    }
+    // The pinned staging copy is reused by the next call, so the previous
+    // upload must have been consumed: tables are tiny, wait for the stream.
+    if (hip_ok(hipStreamSynchronize(stream), "job table reuse") != 0) return nullptr;
+    memcpy(s.table_pinned, host_table, nbytes);
+    if (hip_ok(hipMemcpyAsync(s.table_device, s.table_pinned, nbytes, hipMemcpyHostToDevice, stream),
+               "job table upload") != 0)
+        return nullptr;
+    return s.table_device;
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" {
+
+int salt_mi355_init(void) {
+    State &s = g_state;
+    if (s.ready) return 0;
+    int count = 0;
+    if (hip_ok(hipGetDeviceCount(&count), "hipGetDeviceCount") != 0 || count < 1) {
+        if (count < 1) set_error("no HIP device");
+        return -1;
+    }
+    hipDeviceProp_t prop;
+    if (hip_ok(hipSetDevice(0), "hipSetDevice") != 0 ||
+        hip_ok(hipGetDeviceProperties(&prop, 0), "hipGetDeviceProperties") != 0)
+        return -1;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        set_error("device is %s; this library carries gfx950 code only", prop.gcnArchName);
+        return -1;
+    }
+    s.compute_units = prop.multiProcessorCount;
+    if (hip_ok(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking), "hipStreamCreate") != 0) return -1;
+    if (verify_converters() != 0) {
+        hipStreamDestroy(s.stream);
+        s.stream = nullptr;
+        return -1;
+    }
+    s.ready = 1;
+    if (getenv("SALT_GPU_DIAG"))
+        fprintf(stderr, "salt-mi355: ready on %s, %d CUs, fp8 code scale %g\n", prop.gcnArchName,
+                s.compute_units, (double)s.code_scale);
+    return 0;
+}
+
+int salt_mi355_shutdown(void) {
+    State &s = g_state;
+    if (!s.ready) return 0;
+    int failed = hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize at shutdown");
+    if (s.table_device) { hipFree(s.table_device); hipHostFree(s.table_pinned); }
+    if (s.stream) failed |= hip_ok(hipStreamDestroy(s.stream), "hipStreamDestroy");
+    char keep[sizeof s.last_error];
+    memcpy(keep, s.last_error, sizeof keep);
+    s = State();
+    memcpy(s.last_error, keep, sizeof keep);
+    return failed ? -1 : 0;
+}
+
+const char *salt_mi355_last_error(void) { return g_state.last_error; }
+
+int salt_mi355_converter_tables(float *fp8, float *fp4) {
+    if (!g_state.ready || !fp8 || !fp4) return -1;
+    memcpy(fp8, g_state.fp8_table, sizeof g_state.fp8_table);
+    memcpy(fp4, g_state.fp4_table, sizeof g_state.fp4_table);
+    return 0;
+}
+
+void *salt_mi355_dev_alloc(size_t nbytes) {
+    void *p = nullptr;
+    if (!g_state.ready || nbytes == 0) return nullptr;
+    if (hip_ok(hipMalloc(&p, nbytes), "hipMalloc") != 0) return nullptr;
+    return p;
+}
+int salt_mi355_dev_free(void *p) { return p ? hip_ok(hipFree(p), "hipFree") : 0; }
+int salt_mi355_dev_upload(void *dst, const void *src, size_t nbytes) {
+    return hip_ok(hipMemcpy(dst, src, nbytes, hipMemcpyHostToDevice), "hipMemcpy H2D");
+}
+int salt_mi355_dev_download(void *dst, const void *src, size_t nbytes) {
+    return hip_ok(hipMemcpy(dst, src, nbytes, hipMemcpyDeviceToHost), "hipMemcpy D2H");
+}
+int salt_mi355_dev_fill(void *dst, int value, size_t nbytes) {
+    return hip_ok(hipMemset(dst, value, nbytes), "hipMemset");
+}
+void *salt_mi355_stream(void) { return g_state.stream; }
+int salt_mi355_stream_sync(void *stream) {
+    return hip_ok(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
+}
+void *salt_mi355_event_create(void) {
+    hipEvent_t e = nullptr;
+    return hip_ok(hipEventCreate(&e), "hipEventCreate") == 0 ? (void *)e : nullptr;
+}
+int salt_mi355_event_destroy(void *e) { return hip_ok(hipEventDestroy((hipEvent_t)e), "hipEventDestroy"); }
+int salt_mi355_event_record(void *e, void *stream) {
+    return hip_ok(hipEventRecord((hipEvent_t)e, (hipStream_t)stream), "hipEventRecord");
+}
+int salt_mi355_event_elapsed_ms(void *start, void *stop, float *ms) {
+    if (!ms || hip_ok(hipEventSynchronize((hipEvent_t)stop), "hipEventSynchronize") != 0) return -1;
+    return hip_ok(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop), "hipEventElapsedTime");
+}
+
+// ---------------------------------------------------------------- Q4, device-resident
+
+int salt_mi355_q4_jobs_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tokens, int chains,
+                           void *stream_handle) {
+    State &s = g_state;
+    hipStream_t stream = (hipStream_t)stream_handle;
+    if (!s.ready) { set_error("q4: library not initialised"); return -1; }
+    if (!jobs || njobs < 1 || C < 1 || tokens < 1) { set_error("q4: bad arguments"); return -1; }
+    if (chains != 0 && chains != 8 && chains != 4 && chains != 2) { set_error("q4: chains_per_lane %d", chains); return -1; }
+    for (int j = 0; j < njobs; ++j)
+        if (!jobs[j].vals || !jobs[j].scales || !jobs[j].xs || !jobs[j].ys || jobs[j].rows < 1 ||
+            (size_t)jobs[j].rows > SIZE_MAX / (size_t)C) {
+            set_error("q4: job %d is malformed", j);
+            return -1;
+        }
+    std::vector<Q4Job> table((size_t)njobs);
+    for (int first = 0; first < tokens; first += 4) {
+        const int group = tokens - first < 4 ? tokens - first : 4;
+        bool tileable = true;
+        for (int j = 0; j < njobs; ++j) {
+            Q4Job &q = table[(size_t)j];
+            q.vals = (const uint8_t *)jobs[j].vals;
+            q.scales = (const uint8_t *)jobs[j].scales;
+            q.biases = (const uint8_t *)jobs[j].biases;
+            q.x = jobs[j].xs + (size_t)first * (size_t)C;
+            q.y = jobs[j].ys + (size_t)first * (size_t)jobs[j].rows;
+            q.rows = jobs[j].rows;
+            q.x_stride = C;
+            q.y_stride = jobs[j].rows;
+            tileable = tileable && q4_job_is_tileable(q, C);
+        }
+        Q4Launch launch;
+        memset(&launch, 0, sizeof launch);
+        launch.total_tiles = q4_assign_tiles(table.data(), njobs);
+        launch.njobs = njobs;
+        launch.cols = C;
+        launch.tokens = group;
+        launch.code_scale = s.code_scale;
+        if (njobs == 1) {
+            launch.one = table[0];
+        } else {
+            launch.table = (const Q4Job *)stage_table(table.data(), table.size() * sizeof(Q4Job), stream);
+            if (!launch.table) return -1;
+        }
+        const int rc = tileable ? q4_launch(launch, chains, stream) : q4_launch_generic(launch, stream);
+        if (rc != 0) { set_error("q4: kernel launch failed: %s", hipGetErrorString(hipGetLastError())); return -1; }
+    }
+    return 0;
+}
+
+int salt_mi355_q4_matvec_dev(const void *vals, const void *scales, const void *biases, int R, int C, int B,
+                             const float *xs, float *ys, int chains, void *stream) {
+    SaltMi355Q4Job job;
+    job.vals = vals; job.scales = scales; job.biases = biases; job.xs = xs; job.ys = ys; job.rows = R;
+    return salt_mi355_q4_jobs_dev(&job, 1, C, B, chains, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,117 @@
+// Internal declarations shared by the kernel translation units and the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace mi355 {
+
+// ---------------------------------------------------------------- affine Q4
+
+// One weight matrix against `tokens` activation rows.  All pointers are
+// device pointers.  Rows are processed in tiles of 64; tile0 is the index of
+// the job's first tile inside the launch that carries it.
+struct Q4Job {
+    const uint8_t *vals;      // packed nibbles, row-major, C/2 bytes per row
+    const uint8_t *scales;    // bf16 per 64 elements
+    const uint8_t *biases;    // bf16 per 64 elements, may be null (bias 0)
+    const float *x;           // [tokens][x_stride]
+    float *y;                 // [tokens][y_stride]
+    int rows;
+    int tile0;
+    int x_stride;
+    int y_stride;
+};
+
+struct Q4Launch {
+    Q4Job one;                // used when table == nullptr
+    const Q4Job *table;       // device array of njobs jobs sorted by tile0
+    int njobs;
+    int cols;                 // C, shared by every job of the launch
+    int tokens;               // 1..4 activation rows per job
+    int total_tiles;
+    float code_scale;         // 1 / (value the fp8 converter gives byte 1)
+};
+
+// chains_per_lane: 8, 4 or 2; 0 lets the launcher choose from the tile count.
+int q4_launch(const Q4Launch &launch, int chains_per_lane, hipStream_t stream);
+// Any C, any byte alignment: one wave64 computes two rows, lane = chain.
+int q4_launch_generic(const Q4Launch &launch, hipStream_t stream);
+// true when every pointer and the column count meet the tiled kernel's needs
+bool q4_job_is_tileable(const Q4Job &job, int cols);
+
+// fills table[i].tile0 and returns the launch's tile count
+int q4_assign_tiles(Q4Job *table, int njobs);
+
+// ---------------------------------------------------------------- NVFP4
+
+struct Fp4Job {
+    const uint8_t *packed;    // E2M1 codes, two per byte, C/2 bytes per row
+    const uint8_t *scales;    // E4M3FN, one per 16 columns
+    const float *x;           // [tokens][x_stride] activation used as given
+    float *y;                 // [tokens][y_stride]
+    float weight_global_scale;  // 1 / stored divisor
+    int rows;
+    int tile0;
+    int x_stride;
+    int y_stride;
+};
+
+struct Fp4Launch {
+    Fp4Job one;
+    const Fp4Job *table;
+    int njobs;
+    int cols;
+    int tokens;
+    int total_tiles;
+};
+
+int fp4_launch(const Fp4Launch &launch, int chains_per_lane, hipStream_t stream);
+// activation quantise/dequantise per 16-block; any of packed/scales may be null
+int fp4_qdq_launch(const float *input, int cols, int tokens, float input_global_scale,
+                   uint8_t *packed, uint8_t *scales, float *dequant, int *status,
+                   hipStream_t stream);
+
+// ---------------------------------------------------------------- MoE
+
+struct MoeGeometry {
+    int hidden;               // d_model
+    int routed;               // d_ff
+    int n_experts;
+    int topk;
+};
+
+// Device workspace of one decode layer-step; sized by moe_workspace_bytes.
+struct MoeWorkspace {
+    Q4Job *gate_up_jobs;      // 2*topk jobs
+    Q4Job *down_jobs;         // topk jobs
+    float *gate;              // [topk][routed]
+    float *up;                // [topk][routed]
+    float *act;               // [topk][routed]
+    float *expert_out;        // [topk][hidden]
+    int *status;              // 0 ok, -1 router rejected its input
+};
+
+size_t moe_workspace_bytes(const MoeGeometry &g);
+void moe_workspace_carve(const MoeGeometry &g, void *base, MoeWorkspace *ws);
+
+int router_topk_launch(const float *logits, const float *per_expert_scale, int n_experts, int topk,
+                       int *selected, float *weights, int *status, hipStream_t stream);
+
+int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_stride,
+                           const float *logits, const float *per_expert_scale, const float *x,
+                           int *selected, float *weights, float *expert_out, float *out,
+                           const MoeWorkspace &ws, float code_scale, hipStream_t stream);
+
+int moe_activate_launch(const float *gate, const float *up, float *act, size_t n, hipStream_t stream);
+int moe_reduce_launch(const float *expert_out, const float *weights, int topk, int hidden, float *out,
+                      hipStream_t stream);
+
+// ---------------------------------------------------------------- probes
+
+// Decodes all 256 byte values through the fp8 and fp4 converters (device
+// arrays of 256 and 512 floats).
+int probe_converters_launch(float *fp8_values, float *fp4_values, hipStream_t stream);
+
+}  // namespace mi355

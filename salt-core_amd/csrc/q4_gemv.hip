@@ -1,0 +1,448 @@
+// Affine-Q4 matvec for gfx950, bit-identical to the engine's CPU kernel.
+//
+// The arithmetic contract (reference src/kernels.c:220-250): per row, 32
+// independent fp32 chains, chain j owning the columns c with c % 32 == j,
+//     w = fl(fl(q * scale) + bias);  p = fl(w * x[c]);  acc[j] = fl(acc[j] + p)
+// in ascending c, then the fixed fold  part[j] = sum_{a=0..7} acc[4a+j] from +0
+// and y = (part0 + part2) + (part1 + part3).  Nothing may be reassociated, so
+// parallelism comes from rows and from the 32 chains, never from splitting K.
+//
+// How the tiled kernel maps that to CDNA4:
+//  * A workgroup owns a tile of 64 rows; lane l of every wave owns row l.
+//    Wave t owns S of the 32 chains (S = 8, 4 or 2): the t-th S/2-byte slice
+//    of every 16-byte block (32 columns) of the row.  Because the chain set is
+//    wave-uniform, x[c] is a scalar (SGPR) operand fetched with s_load.
+//  * 16 blocks (256 bytes per row, 16 KiB per tile) are staged per step into
+//    LDS with coalesced 128-bit global loads, double-buffered; the row pitch
+//    of 65 dwords makes every lane's slice read conflict-free.
+//  * q -> float costs half an instruction: nibbles are isolated in bytes and
+//    converted two at a time by v_cvt_pk_f32_fp8 (a byte 0..15 decodes to
+//    q * 2^-9 exactly), with the power of two folded into the scale.  q*scale
+//    is exact in fp32 (4-bit times 8-bit significand), so fma(q', scale', bias)
+//    rounds once, exactly where the reference's separate add rounds.
+//  * (scale', bias) pairs are converted once per tile step into LDS, not once
+//    per wave.  A scale so large that scale * 2^9 would overflow flips the
+//    tile to a path that multiplies and adds separately with the raw scale.
+//  * The per-row fold runs in the documented order from LDS.
+#include "mi355_internal.h"
+
+#include <stddef.h>
+#include <stdio.h>
+#include <stdlib.h>
+
+namespace mi355 {
+namespace {
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+// Activations are read-only for the lifetime of a launch and their address is
+// wave-uniform, so they are read through the constant address space: the
+// compiler then fetches them with scalar loads and feeds them to the VALU as
+// SGPR operands.
+typedef const float __attribute__((address_space(4))) *uniform_f32_ptr;
+__device__ __forceinline__ uniform_f32_ptr as_uniform(const float *p) {
+    return (uniform_f32_ptr)(uintptr_t)p;
+}
+
+constexpr int TILE_ROWS = 64;
+constexpr int CHUNK_BLOCKS = 16;                       // 32-column blocks per staged step
+constexpr int CHUNK_GROUPS = CHUNK_BLOCKS / 2;         // 64-column scale groups per step
+constexpr int W_PITCH = 16 * CHUNK_BLOCKS + 4;         // bytes per staged row: odd dword pitch
+constexpr int M_PITCH = 2 * CHUNK_GROUPS + 2;          // floats per staged row of (scale, bias)
+constexpr int W_STAGE = TILE_ROWS * W_PITCH;
+constexpr int M_STAGE = TILE_ROWS * M_PITCH;
+constexpr int FOLD_PITCH = 33;
+constexpr float BIG_SCALE = 0x1p118f;
+
+__device__ __forceinline__ float bf16_to_f32(uint32_t half) { return __uint_as_float(half << 16); }
+
+// Pointers that arrive inside a job record are generic; naming their address
+// space lets the compiler use global_load / s_load instead of flat_load.
+typedef const uint8_t __attribute__((address_space(1))) *global_u8_ptr;
+typedef const uint16_t __attribute__((address_space(1))) *global_u16_ptr;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef const u32x4 __attribute__((address_space(1))) *global_u128_ptr;
+typedef float __attribute__((address_space(1))) *global_f32_out_ptr;
+typedef const uint64_t __attribute__((address_space(4))) *uniform_u64_ptr;
+
+static_assert(sizeof(Q4Job) == 56 && offsetof(Q4Job, rows) == 40 && offsetof(Q4Job, tile0) == 44 &&
+              offsetof(Q4Job, x_stride) == 48 && offsetof(Q4Job, y_stride) == 52,
+              "find_job reads a job record as seven 64-bit words");
+
+__device__ __forceinline__ Q4Job find_job(const Q4Launch &L, int tile) {
+    if (L.table == nullptr) return L.one;
+    const uniform_u64_ptr words = (uniform_u64_ptr)(uintptr_t)L.table;     // 7 words per record
+    int lo = 0, hi = L.njobs - 1;
+    while (lo < hi) {                      // last job whose tile0 <= tile
+        const int mid = (lo + hi + 1) >> 1;
+        if ((int)(words[7 * mid + 5] >> 32) <= tile) lo = mid; else hi = mid - 1;
+    }
+    const uniform_u64_ptr rec = words + 7 * lo;
+    Q4Job job;
+    job.vals = (const uint8_t *)rec[0];
+    job.scales = (const uint8_t *)rec[1];
+    job.biases = (const uint8_t *)rec[2];
+    job.x = (const float *)rec[3];
+    job.y = (float *)rec[4];
+    job.rows = (int)(uint32_t)rec[5];
+    job.tile0 = (int)(rec[5] >> 32);
+    job.x_stride = (int)(uint32_t)rec[6];
+    job.y_stride = (int)(rec[6] >> 32);
+    return job;
+}
+
+// Eight nibbles of w as floats scaled by the converter's constant:
+// q[n] = nibble_n * 2^-9 on gfx950.
+__device__ __forceinline__ void nibbles_to_f32(uint32_t w, float (&q)[8]) {
+    const uint32_t lo = w & 0x0F0F0F0Fu;
+    const uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;
+    const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, false);   // nibbles 0, 2
+    const f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, false);   // nibbles 1, 3
+    const f32x2 c = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, true);    // nibbles 4, 6
+    const f32x2 d = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, true);    // nibbles 5, 7
+    q[0] = a.x; q[1] = b.x; q[2] = a.y; q[3] = b.y;
+    q[4] = c.x; q[5] = d.x; q[6] = c.y; q[7] = d.y;
+}
+
+// One packed word of a lane: nibble n belongs to block (n / S) of the word's
+// span and to the lane's chain (n % S).  xw points at x for the span's first
+// block and the wave's first chain; it is wave-uniform.
+template <int S, int NB, int NNIB, bool SLOW>
+__device__ __forceinline__ void consume_word(uint32_t w, float scale, float bias, float code_scale,
+                                             uniform_f32_ptr xw, int x_stride, float (&acc)[NB][S]) {
+    float q[8];
+    nibbles_to_f32(w, q);
+#pragma unroll
+    for (int n = 0; n < NNIB; ++n) {
+        const int blk = (S == 8) ? 0 : n / S;
+        const int ch = n % S;
+        float wgt;
+        if (!SLOW) {
+            wgt = __builtin_fmaf(q[n], scale, bias);
+        } else {
+            const float qi = q[n] * code_scale;          // back to the integer value, exact
+            wgt = qi * scale;
+            wgt = wgt + bias;
+        }
+#pragma unroll
+        for (int t = 0; t < NB; ++t) {
+            const float p = wgt * xw[(size_t)t * x_stride + blk * 32 + ch];
+            acc[t][ch] = acc[t][ch] + p;
+        }
+    }
+}
+
+template <int S, int NB>
+__global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L) {
+    constexpr int WAVES = 32 / S;
+    constexpr int THREADS = WAVES * 64;
+    constexpr int PIECES = (TILE_ROWS * CHUNK_BLOCKS) / THREADS;              // 16-byte pieces per thread
+    constexpr int META_ITEMS = (TILE_ROWS * CHUNK_GROUPS + THREADS - 1) / THREADS;
+    constexpr int FOLD_BYTES = NB * TILE_ROWS * FOLD_PITCH * 4;
+    constexpr int W_BYTES = 2 * W_STAGE > FOLD_BYTES ? 2 * W_STAGE : FOLD_BYTES;
+    static_assert(THREADS >= NB * TILE_ROWS, "fold needs one thread per (token, row)");
+
+    __shared__ __attribute__((aligned(16))) uint8_t w_lds[W_BYTES];
+    __shared__ __attribute__((aligned(16))) float m_lds[2 * M_STAGE];
+    __shared__ int slow_flag;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    const Q4Job job = find_job(L, blockIdx.x);
+    const int row0 = (blockIdx.x - job.tile0) * TILE_ROWS;
+    const int R = job.rows;
+    const int nblk = L.cols >> 5;
+    const int ngrp = L.cols >> 6;
+    const int nchunk = (nblk + CHUNK_BLOCKS - 1) / CHUNK_BLOCKS;
+    const size_t row_bytes = (size_t)(L.cols >> 1);
+    const global_u8_ptr vals = (global_u8_ptr)(uintptr_t)job.vals;
+    const global_u16_ptr scales16 = (global_u16_ptr)(uintptr_t)job.scales;
+    const global_u16_ptr biases16 = (global_u16_ptr)(uintptr_t)job.biases;
+    const global_f32_out_ptr y = (global_f32_out_ptr)(uintptr_t)job.y;
+
+    u32x4 wreg[PIECES];
+    uint32_t mreg[META_ITEMS];
+
+    auto issue = [&](int ck) {
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int p = tid + i * THREADS;
+            const int row = p >> 4, seg = p & 15;
+            const int blk = ck * CHUNK_BLOCKS + seg;
+            int r = row0 + row;
+            r = r < R ? r : R - 1;
+            if (blk < nblk)
+                wreg[i] = *(global_u128_ptr)(vals + (size_t)r * row_bytes + (size_t)blk * 16);
+            else
+                wreg[i] = u32x4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int i = 0; i < META_ITEMS; ++i) {
+            const int it = tid + i * THREADS;
+            mreg[i] = 0;
+            if (it < TILE_ROWS * CHUNK_GROUPS) {
+                const int row = it >> 3;
+                const int g = ck * CHUNK_GROUPS + (it & 7);
+                int r = row0 + row;
+                r = r < R ? r : R - 1;
+                if (g < ngrp) {
+                    const size_t gi = (size_t)r * ngrp + g;
+                    const uint32_t s = scales16[gi];
+                    const uint32_t b = biases16 ? biases16[gi] : 0u;
+                    mreg[i] = s | (b << 16);
+                }
+            }
+        }
+    };
+
+    auto commit = [&](int stage) {
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int p = tid + i * THREADS;
+            const int row = p >> 4, seg = p & 15;
+            uint32_t *dst = reinterpret_cast<uint32_t *>(w_lds + stage * W_STAGE + row * W_PITCH + seg * 16);
+            dst[0] = wreg[i].x; dst[1] = wreg[i].y; dst[2] = wreg[i].z; dst[3] = wreg[i].w;
+        }
+#pragma unroll
+        for (int i = 0; i < META_ITEMS; ++i) {
+            const int it = tid + i * THREADS;
+            if (it < TILE_ROWS * CHUNK_GROUPS) {
+                const int row = it >> 3;
+                const float s = bf16_to_f32(mreg[i] & 0xFFFFu);
+                const float b = bf16_to_f32(mreg[i] >> 16);
+                if (!(__builtin_fabsf(s) < BIG_SCALE)) slow_flag = 1;
+                float *dst = m_lds + stage * M_STAGE + row * M_PITCH + 2 * (it & 7);
+                dst[0] = s * L.code_scale;
+                dst[1] = b;
+            }
+        }
+    };
+
+    float acc[NB][S];
+#pragma unroll
+    for (int t = 0; t < NB; ++t)
+#pragma unroll
+        for (int c = 0; c < S; ++c) acc[t][c] = 0.0f;
+
+    if (tid == 0) slow_flag = 0;
+    issue(0);
+    __syncthreads();
+
+    int my_row = row0 + lane;
+    my_row = my_row < R ? my_row : R - 1;
+
+    for (int ck = 0; ck < nchunk; ++ck) {
+        const int stage = ck & 1;
+        commit(stage);
+        __syncthreads();
+        if (ck + 1 < nchunk) issue(ck + 1);
+
+        const int slow = __builtin_amdgcn_readfirstlane(slow_flag);
+        const int remaining = ngrp - ck * CHUNK_GROUPS;
+        const int gcount = remaining < CHUNK_GROUPS ? remaining : CHUNK_GROUPS;
+        const uint8_t *wrow = w_lds + stage * W_STAGE + lane * W_PITCH + wave * (S / 2);
+        const float *mrow = m_lds + stage * M_STAGE + lane * M_PITCH;
+
+        for (int g = 0; g < gcount; ++g) {
+            float scale = mrow[2 * g];
+            const float bias = mrow[2 * g + 1];
+            const int blk = ck * CHUNK_BLOCKS + 2 * g;
+            uniform_f32_ptr xg = as_uniform(job.x) + (size_t)blk * 32 + S * wave;
+            uint32_t w0, w1 = 0;
+            if (S == 8) {
+                w0 = *reinterpret_cast<const uint32_t *>(wrow + (2 * g) * 16);
+                w1 = *reinterpret_cast<const uint32_t *>(wrow + (2 * g + 1) * 16);
+            } else if (S == 4) {
+                const uint32_t a = *reinterpret_cast<const uint16_t *>(wrow + (2 * g) * 16);
+                const uint32_t b = *reinterpret_cast<const uint16_t *>(wrow + (2 * g + 1) * 16);
+                w0 = a | (b << 16);
+            } else {
+                const uint32_t a = wrow[(2 * g) * 16];
+                const uint32_t b = wrow[(2 * g + 1) * 16];
+                w0 = a | (b << 8);
+            }
+            if (__builtin_expect(slow, 0)) {
+                scale = bf16_to_f32(scales16[(size_t)my_row * ngrp + ck * CHUNK_GROUPS + g]);
+                if (S == 8) {
+                    consume_word<S, NB, 8, true>(w0, scale, bias, L.code_scale, xg, job.x_stride, acc);
+                    consume_word<S, NB, 8, true>(w1, scale, bias, L.code_scale, xg + 32, job.x_stride, acc);
+                } else {
+                    consume_word<S, NB, (S == 4 ? 8 : 4), true>(w0, scale, bias, L.code_scale, xg, job.x_stride, acc);
+                }
+            } else {
+                if (S == 8) {
+                    consume_word<S, NB, 8, false>(w0, scale, bias, L.code_scale, xg, job.x_stride, acc);
+                    consume_word<S, NB, 8, false>(w1, scale, bias, L.code_scale, xg + 32, job.x_stride, acc);
+                } else {
+                    consume_word<S, NB, (S == 4 ? 8 : 4), false>(w0, scale, bias, L.code_scale, xg, job.x_stride, acc);
+                }
+            }
+        }
+    }
+
+    // Fold the 32 chains of each (token, row) in the reference's order.
+    __syncthreads();
+    float *fold = reinterpret_cast<float *>(w_lds);
+#pragma unroll
+    for (int t = 0; t < NB; ++t)
+#pragma unroll
+        for (int c = 0; c < S; ++c) fold[(t * TILE_ROWS + lane) * FOLD_PITCH + S * wave + c] = acc[t][c];
+    __syncthreads();
+    if (tid < NB * TILE_ROWS) {
+        const int t = tid >> 6;
+        const float *f = fold + (t * TILE_ROWS + lane) * FOLD_PITCH;
+        float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int a = 0; a < 8; ++a)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) part[j] = part[j] + f[4 * a + j];
+        const float even = part[0] + part[2];
+        const float odd = part[1] + part[3];
+        const int row = row0 + lane;
+        if (row < R) y[(size_t)t * job.y_stride + row] = even + odd;
+    }
+}
+
+// ---------------------------------------------------------------- generic
+// Any column count and any byte alignment: lane = chain, 32 lanes per row, two
+// rows per wave, byte loads.  Follows the flat element index k = r*C + c for
+// the nibble and the scale group exactly as the reference does.
+__device__ __forceinline__ uint32_t load_u16_bytes(global_u8_ptr p) { return (uint32_t)p[0] | ((uint32_t)p[1] << 8); }
+
+template <int NB>
+__global__ __launch_bounds__(256) void q4_generic_kernel(const Q4Launch L) {
+    const Q4Job job = find_job(L, blockIdx.x);
+    const int row0 = (blockIdx.x - job.tile0) * TILE_ROWS;
+    const int chain = threadIdx.x & 31;
+    const int sub = threadIdx.x >> 5;                    // 8 rows in flight per workgroup
+    const int C = L.cols;
+    const global_u8_ptr vals = (global_u8_ptr)(uintptr_t)job.vals;
+    const global_u8_ptr scales = (global_u8_ptr)(uintptr_t)job.scales;
+    const global_u8_ptr biases = (global_u8_ptr)(uintptr_t)job.biases;
+    const float __attribute__((address_space(1))) *x = (const float __attribute__((address_space(1))) *)(uintptr_t)job.x;
+    const global_f32_out_ptr y = (global_f32_out_ptr)(uintptr_t)job.y;
+    for (int pass = 0; pass < TILE_ROWS / 8; ++pass) {
+        const int row = row0 + pass * 8 + sub;
+        const bool live = row < job.rows;
+        const int r = live ? row : job.rows - 1;
+        float acc[NB];
+#pragma unroll
+        for (int t = 0; t < NB; ++t) acc[t] = 0.0f;
+        for (int c = chain; c < C; c += 32) {
+            const size_t k = (size_t)r * (size_t)C + (size_t)c;
+            const uint32_t byte = vals[k >> 1];
+            const uint32_t q = (k & 1) ? (byte >> 4) : (byte & 15u);
+            const size_t g = k >> 6;
+            const float s = bf16_to_f32(load_u16_bytes(scales + 2 * g));
+            const float b = biases ? bf16_to_f32(load_u16_bytes(biases + 2 * g)) : 0.0f;
+            float wgt = (float)q * s;
+            wgt = wgt + b;
+#pragma unroll
+            for (int t = 0; t < NB; ++t) {
+                const float p = wgt * x[(size_t)t * job.x_stride + c];
+                acc[t] = acc[t] + p;
+            }
+        }
+        const int base = threadIdx.x & 32;               // first lane of this row's half-wave
+#pragma unroll
+        for (int t = 0; t < NB; ++t) {
+            float part = 0.0f;
+#pragma unroll
+            for (int a = 0; a < 8; ++a) part = part + __shfl(acc[t], base + 4 * a + (chain & 3), 64);
+            const float p0 = __shfl(part, base + 0, 64), p1 = __shfl(part, base + 1, 64);
+            const float p2 = __shfl(part, base + 2, 64), p3 = __shfl(part, base + 3, 64);
+            const float even = p0 + p2;
+            const float odd = p1 + p3;
+            if (live && chain == 0) y[(size_t)t * job.y_stride + row] = even + odd;
+        }
+    }
+}
+
+template <int S>
+int launch_tiles(const Q4Launch &L, hipStream_t stream) {
+    const dim3 grid(L.total_tiles), block((32 / S) * 64);
+    switch (L.tokens) {
+        case 1: hipLaunchKernelGGL((q4_tile_kernel<S, 1>), grid, block, 0, stream, L); break;
+        case 2: hipLaunchKernelGGL((q4_tile_kernel<S, 2>), grid, block, 0, stream, L); break;
+        case 3: hipLaunchKernelGGL((q4_tile_kernel<S, 3>), grid, block, 0, stream, L); break;
+        case 4: hipLaunchKernelGGL((q4_tile_kernel<S, 4>), grid, block, 0, stream, L); break;
+        default: return -1;
+    }
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int env_chains() {
+    static int cached = -1;
+    if (cached < 0) {
+        const char *e = getenv("SALT_MI355_Q4_CHAINS");
+        const int v = e ? atoi(e) : 0;
+        cached = (v == 8 || v == 4 || v == 2) ? v : 0;
+    }
+    return cached;
+}
+
+}  // namespace
+
+bool q4_job_is_tileable(const Q4Job &job, int cols) {
+    return cols >= 64 && (cols & 63) == 0 && ((uintptr_t)job.vals & 15) == 0 && ((uintptr_t)job.scales & 1) == 0 &&
+           ((uintptr_t)job.biases & 1) == 0 && ((uintptr_t)job.x & 3) == 0 && ((uintptr_t)job.y & 3) == 0;
+}
+
+int q4_assign_tiles(Q4Job *table, int njobs) {
+    int tiles = 0;
+    for (int i = 0; i < njobs; ++i) {
+        table[i].tile0 = tiles;
+        tiles += (table[i].rows + TILE_ROWS - 1) / TILE_ROWS;
+    }
+    return tiles;
+}
+
+int q4_launch(const Q4Launch &L, int chains_per_lane, hipStream_t stream) {
+    if (L.total_tiles < 1 || L.tokens < 1 || L.tokens > 4 || L.cols < 64 || (L.cols & 63)) return -1;
+    int S = chains_per_lane ? chains_per_lane : env_chains();
+    if (S == 0) {
+        // enough waves to give every SIMD of the 256 CUs at least two
+        if (L.total_tiles * 4 >= 2048) S = 8;
+        else if (L.total_tiles * 8 >= 2048) S = 4;
+        else S = 2;
+    }
+    switch (S) {
+        case 8: return launch_tiles<8>(L, stream);
+        case 4: return launch_tiles<4>(L, stream);
+        case 2: return launch_tiles<2>(L, stream);
+        default: return -1;
+    }
+}
+
+int q4_launch_generic(const Q4Launch &L, hipStream_t stream) {
+    if (L.total_tiles < 1 || L.tokens < 1 || L.tokens > 4 || L.cols < 1) return -1;
+    const dim3 grid(L.total_tiles), block(256);
+    switch (L.tokens) {
+        case 1: hipLaunchKernelGGL((q4_generic_kernel<1>), grid, block, 0, stream, L); break;
+        case 2: hipLaunchKernelGGL((q4_generic_kernel<2>), grid, block, 0, stream, L); break;
+        case 3: hipLaunchKernelGGL((q4_generic_kernel<3>), grid, block, 0, stream, L); break;
+        case 4: hipLaunchKernelGGL((q4_generic_kernel<4>), grid, block, 0, stream, L); break;
+        default: return -1;
+    }
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// ---------------------------------------------------------------- converter probe
+namespace {
+__global__ void probe_converters_kernel(float *fp8_values, float *fp4_values) {
+    const uint32_t byte = threadIdx.x;                   // 256 threads
+    const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)byte, false);
+    fp8_values[byte] = a.x;
+    const f32x2 b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(byte, 1.0f, 0);
+    fp4_values[2 * byte] = b.x;                          // low nibble
+    fp4_values[2 * byte + 1] = b.y;                      // high nibble
+}
+}  // namespace
+
+int probe_converters_launch(float *fp8_values, float *fp4_values, hipStream_t stream) {
+    hipLaunchKernelGGL(probe_converters_kernel, dim3(1), dim3(256), 0, stream, fp8_values, fp4_values);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+}  // namespace mi355

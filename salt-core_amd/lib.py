@@ -1,0 +1,133 @@
+"""ctypes loader of libsalt_gpu_mi355.so and small host-side conveniences
+(device buffers as numpy-in / numpy-out).  No computation happens here: every
+call goes through the C ABI declared in include/salt_gpu_mi355.h."""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+import numpy as np
+
+LIB_PATH = Path(__file__).resolve().parent / "libsalt_gpu_mi355.so"
+vp = C.c_void_p
+
+
+class Q4Job(C.Structure):
+    _fields_ = [("vals", vp), ("scales", vp), ("biases", vp), ("xs", vp), ("ys", vp), ("rows", C.c_int)]
+
+
+_lib = None
+
+
+def _sig(fn, restype, *argtypes):
+    fn.restype = restype
+    fn.argtypes = list(argtypes)
+
+
+def load() -> C.CDLL:
+    """Loads the shared library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise RuntimeError(f"{LIB_PATH} is missing: build it with `make -C salt-core_amd/csrc` "
+                           "(or __graft_entry__.build())")
+    lib = C.CDLL(str(LIB_PATH))
+    i, sz, f = C.c_int, C.c_size_t, C.c_float
+    _sig(lib.salt_mi355_init, i)
+    _sig(lib.salt_mi355_shutdown, i)
+    _sig(lib.salt_mi355_last_error, C.c_char_p)
+    _sig(lib.salt_mi355_converter_tables, i, vp, vp)
+    _sig(lib.salt_mi355_dev_alloc, vp, sz)
+    _sig(lib.salt_mi355_dev_free, i, vp)
+    _sig(lib.salt_mi355_dev_upload, i, vp, vp, sz)
+    _sig(lib.salt_mi355_dev_download, i, vp, vp, sz)
+    _sig(lib.salt_mi355_dev_fill, i, vp, i, sz)
+    _sig(lib.salt_mi355_stream, vp)
+    _sig(lib.salt_mi355_stream_sync, i, vp)
+    _sig(lib.salt_mi355_event_create, vp)
+    _sig(lib.salt_mi355_event_destroy, i, vp)
+    _sig(lib.salt_mi355_event_record, i, vp, vp)
+    _sig(lib.salt_mi355_event_elapsed_ms, i, vp, vp, C.POINTER(f))
+    _sig(lib.salt_mi355_q4_matvec_dev, i, vp, vp, vp, i, i, i, vp, vp, i, vp)
+    _sig(lib.salt_mi355_q4_jobs_dev, i, C.POINTER(Q4Job), i, i, i, i, vp)
+    _lib = lib
+    return lib
+
+
+def init() -> C.CDLL:
+    """Loads the library and initialises the device; raises with the library's
+    own message when there is no usable MI355X."""
+    lib = load()
+    if lib.salt_mi355_init() != 0:
+        raise RuntimeError("salt_mi355_init failed: " + lib.salt_mi355_last_error().decode())
+    return lib
+
+
+def check(rc: int, what: str = "call"):
+    if rc != 0:
+        raise RuntimeError(f"{what} failed: " + load().salt_mi355_last_error().decode())
+
+
+class DeviceBuffer:
+    """A hipMalloc'd region owned by this object."""
+
+    def __init__(self, nbytes: int, fill: int | None = None):
+        self.lib = load()
+        self.nbytes = int(nbytes)
+        self.ptr = self.lib.salt_mi355_dev_alloc(max(self.nbytes, 1))
+        if not self.ptr:
+            raise MemoryError("salt_mi355_dev_alloc: " + self.lib.salt_mi355_last_error().decode())
+        if fill is not None:
+            check(self.lib.salt_mi355_dev_fill(self.ptr, fill, self.nbytes), "fill")
+
+    @classmethod
+    def from_host(cls, array: np.ndarray) -> "DeviceBuffer":
+        array = np.ascontiguousarray(array)
+        buf = cls(array.nbytes)
+        check(buf.lib.salt_mi355_dev_upload(buf.ptr, array.ctypes.data_as(vp), array.nbytes), "upload")
+        return buf
+
+    def upload(self, array: np.ndarray, offset: int = 0):
+        array = np.ascontiguousarray(array)
+        assert offset + array.nbytes <= self.nbytes
+        check(self.lib.salt_mi355_dev_upload(self.ptr + offset, array.ctypes.data_as(vp), array.nbytes), "upload")
+
+    def to_host(self, dtype, count: int | None = None, offset: int = 0) -> np.ndarray:
+        dtype = np.dtype(dtype)
+        count = (self.nbytes - offset) // dtype.itemsize if count is None else count
+        out = np.empty(count, dtype)
+        check(self.lib.salt_mi355_dev_download(out.ctypes.data_as(vp), self.ptr + offset, out.nbytes), "download")
+        return out
+
+    def at(self, offset: int) -> int:
+        return self.ptr + offset
+
+    def free(self):
+        if self.ptr:
+            self.lib.salt_mi355_dev_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def q4_matvec(vals: np.ndarray, scales: np.ndarray, biases: np.ndarray | None, R: int, C_: int,
+              xs: np.ndarray, chains: int = 0) -> np.ndarray:
+    """Host-array convenience around salt_mi355_q4_matvec_dev: uploads, runs on
+    the library stream, downloads ys[B, R]."""
+    lib = init()
+    xs = np.ascontiguousarray(xs, np.float32).reshape(-1, C_)
+    B = xs.shape[0]
+    dv, ds = DeviceBuffer.from_host(vals), DeviceBuffer.from_host(scales)
+    db = DeviceBuffer.from_host(biases) if biases is not None else None
+    dx = DeviceBuffer.from_host(xs)
+    dy = DeviceBuffer(B * R * 4, fill=0xFF)
+    stream = lib.salt_mi355_stream()
+    check(lib.salt_mi355_q4_matvec_dev(dv.ptr, ds.ptr, db.ptr if db else None, R, C_, B, dx.ptr, dy.ptr,
+                                       chains, stream), "q4_matvec_dev")
+    check(lib.salt_mi355_stream_sync(stream), "sync")
+    return dy.to_host(np.float32).reshape(B, R)
