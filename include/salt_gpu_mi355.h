@@ -91,6 +91,60 @@ typedef struct SaltMi355Q4Job {
 int salt_mi355_q4_jobs_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tokens,
                            int chains_per_lane, void *stream);
 
+/* ---- NVFP4, device-resident ---------------------------------------------
+ * Layout as the reference's nvfp4.h:37-46: packed E2M1 codes, low nibble =
+ * even element; E4M3FN scales [R][C/16]; one fp32 stored divisor per tensor
+ * (weight_global_scale = 1 / divisor). */
+
+/* Dynamic group-16 activation quantise/dequantise of B rows of C floats
+ * (reference salt_nvfp4_quantize_input_reference, nvfp4.c:82-130).  packed
+ * (B*C/2 bytes) and scales (B*C/16 bytes) may be NULL when only the
+ * dequantised activation is wanted.  *status_dev (device int, cleared by the
+ * caller) is set to -1 when an input is not finite; the reference rejects the
+ * call in that case and so must the caller. */
+int salt_mi355_nvfp4_qdq_dev(const float *input, int C, int B, float input_global_scale,
+                             uint8_t *packed, uint8_t *scales, float *dequant,
+                             int *status_dev, void *stream);
+/* Rows against an activation that is used as given: pass the dequantised
+ * output of salt_mi355_nvfp4_qdq_dev to reproduce the reference matvec
+ * (nvfp4.c:228-256), or the raw activation for the weights-only variant. */
+int salt_mi355_nvfp4_matvec_dev(const void *packed, const void *scales, float stored_divisor,
+                                int R, int C, int B, const float *xs, float *ys,
+                                int chains_per_lane, void *stream);
+
+/* ---- MoE decode layer-step, device-resident ----------------------------- */
+
+/* reference salt_gemma4_router_topk (gemma4.c:132-186).  sorted_by_id = 0
+ * keeps the reference function's descending-logit order, 1 applies its
+ * callers' ascending-expert sort (gemma4_text.c:7923-7930).  *status_dev is
+ * set to 0, or to -1 when the reference would return -1 (outputs untouched). */
+int salt_mi355_router_topk_dev(const float *logits, const float *per_expert_scale,
+                               int n_experts, int topk, int sorted_by_id,
+                               int *selected, float *weights, int *status_dev, void *stream);
+
+/* One token through one MoE layer: router top-k, ascending sort, the selected
+ * experts (gate, up, gelu*up, down; all affine-Q4 group 64) and the in-order
+ * weighted sum (reference gemma4_text.c:8360, 7923-7930, 7608-7649,
+ * 8301-8304).  pool = expert 0 of the layer in the engine's slot layout
+ * [gate|up|down] x [vals|scales|biases] (gemma4_text.c:73-79), experts
+ * expert_stride bytes apart.  selected/weights: topk entries; expert_out
+ * (optional): [topk][hidden]; out: [hidden].  workspace: device memory of
+ * salt_mi355_moe_workspace_bytes(); its first int receives the router status
+ * (0 / -1) and must be read after the stream has drained. */
+size_t salt_mi355_moe_workspace_bytes(int hidden, int routed, int n_experts, int topk);
+int salt_mi355_moe_decode_step_dev(const void *pool, size_t expert_stride,
+                                   int hidden, int routed, int n_experts, int topk,
+                                   const float *logits, const float *per_expert_scale,
+                                   const float *x, int *selected, float *weights,
+                                   float *expert_out, float *out,
+                                   void *workspace, void *stream);
+/* The pieces of the step on their own: act = gelu_tanh(gate) * up over n
+ * floats (gemma4.c:80-83, gemma4_text.c:7635), and out[d] = sum_i
+ * expert_out[i][d] * weights[i] from +0 in ascending i (gemma4_text.c:8301-8304). */
+int salt_mi355_moe_activate_dev(const float *gate, const float *up, float *act, size_t n, void *stream);
+int salt_mi355_moe_reduce_dev(const float *expert_out, const float *weights, int topk, int hidden,
+                              float *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -42,7 +42,7 @@ int verify_converters() {
     if (rc == 0)
         rc = hip_ok(hipMemcpy(g_state.fp4_table, device + 256, 512 * sizeof(float), hipMemcpyDeviceToHost),
                     "probe copy");
-    hipFree(device);
+    (void)hipFree(device);
     if (rc != 0) return -1;
     const float unit = g_state.fp8_table[1];
     int exponent = 0;
@@ -57,6 +57,17 @@ int verify_converters() {
             return -1;
         }
     g_state.code_scale = 1.0f / unit;
+    // NVFP4 block scales are OCP E4M3FN (bias 7, 0x7f / 0xff = NaN, no infinities)
+    int ocp = 1;
+    for (int code = 0; code < 256 && ocp; ++code) {
+        const int e = (code >> 3) & 15, m = code & 7;
+        const float got = g_state.fp8_table[code];
+        if (e == 15 && m == 7) { ocp = got != got; continue; }
+        float want = e == 0 ? (float)m * 0.001953125f : (1.0f + (float)m * 0.125f) * ldexpf(1.0f, e - 7);
+        if (code & 0x80) want = -want;
+        ocp = got == want;
+    }
+    g_state.fp8_is_ocp = ocp;
     static const float magnitude[8] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
     for (int byte = 0; byte < 256; ++byte)
         for (int half = 0; half < 2; ++half) {
@@ -79,8 +90,8 @@ void *stage_table(const void *host_table, size_t nbytes, hipStream_t stream) {
     if (nbytes > s.table_capacity) {
         if (s.table_device) {
             if (hip_ok(hipDeviceSynchronize(), "sync before table growth") != 0) return nullptr;
-            hipFree(s.table_device);
-            hipHostFree(s.table_pinned);
+            (void)hipFree(s.table_device);
+            (void)hipHostFree(s.table_pinned);
             s.table_device = nullptr; s.table_pinned = nullptr; s.table_capacity = 0;
         }
         size_t capacity = 64 * 1024;
@@ -125,7 +136,7 @@ int salt_mi355_init(void) {
     s.compute_units = prop.multiProcessorCount;
     if (hip_ok(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking), "hipStreamCreate") != 0) return -1;
     if (verify_converters() != 0) {
-        hipStreamDestroy(s.stream);
+        (void)hipStreamDestroy(s.stream);
         s.stream = nullptr;
         return -1;
     }
@@ -140,7 +151,7 @@ int salt_mi355_shutdown(void) {
     State &s = g_state;
     if (!s.ready) return 0;
     int failed = hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize at shutdown");
-    if (s.table_device) { hipFree(s.table_device); hipHostFree(s.table_pinned); }
+    if (s.table_device) { (void)hipFree(s.table_device); (void)hipHostFree(s.table_pinned); }
     if (s.stream) failed |= hip_ok(hipStreamDestroy(s.stream), "hipStreamDestroy");
     char keep[sizeof s.last_error];
     memcpy(keep, s.last_error, sizeof keep);

@@ -1,0 +1,116 @@
+// Device-resident NVFP4, router and MoE entry points of libsalt_gpu_mi355.so.
+#include "backend_state.h"
+
+#include <math.h>
+#include <string.h>
+
+using namespace mi355;
+
+extern "C" {
+
+int salt_mi355_nvfp4_qdq_dev(const float *input, int C, int B, float input_global_scale, uint8_t *packed,
+                             uint8_t *scales, float *dequant, int *status_dev, void *stream) {
+    if (!g_state.ready) { set_error("nvfp4 qdq: library not initialised"); return -1; }
+    if (!g_state.fp8_is_ocp) { set_error("nvfp4: this device's fp8 converter is not OCP E4M3FN"); return -1; }
+    if (!input || !dequant || !status_dev || C < 16 || (C & 15) || B < 1 || !isfinite(input_global_scale) ||
+        input_global_scale <= 0.0f || ((uintptr_t)input & 15) || ((uintptr_t)dequant & 15) ||
+        ((uintptr_t)packed & 7)) {
+        set_error("nvfp4 qdq: bad arguments");
+        return -1;
+    }
+    if (fp4_qdq_launch(input, C, B, input_global_scale, packed, scales, dequant, status_dev, (hipStream_t)stream) != 0) {
+        set_error("nvfp4 qdq: launch failed");
+        return -1;
+    }
+    return 0;
+}
+
+int salt_mi355_nvfp4_matvec_dev(const void *packed, const void *scales, float stored_divisor, int R, int C, int B,
+                                const float *xs, float *ys, int chains, void *stream) {
+    if (!g_state.ready) { set_error("nvfp4 matvec: library not initialised"); return -1; }
+    if (!g_state.fp8_is_ocp) { set_error("nvfp4: this device's fp8 converter is not OCP E4M3FN"); return -1; }
+    if (!packed || !scales || !xs || !ys || R < 1 || C < 32 || (C & 31) || B < 1 || !isfinite(stored_divisor) ||
+        stored_divisor == 0.0f || ((uintptr_t)packed & 15) || ((uintptr_t)scales & 1) || ((uintptr_t)xs & 3) ||
+        ((uintptr_t)ys & 3) || (chains != 0 && chains != 8 && chains != 4 && chains != 2)) {
+        set_error("nvfp4 matvec: bad arguments (C must be a multiple of 32, packed 16-byte aligned)");
+        return -1;
+    }
+    for (int first = 0; first < B; first += 4) {
+        Fp4Launch launch;
+        memset(&launch, 0, sizeof launch);
+        launch.one.packed = (const uint8_t *)packed;
+        launch.one.scales = (const uint8_t *)scales;
+        launch.one.x = xs + (size_t)first * C;
+        launch.one.y = ys + (size_t)first * R;
+        launch.one.weight_global_scale = 1.0f / stored_divisor;
+        launch.one.rows = R;
+        launch.one.tile0 = 0;
+        launch.one.x_stride = C;
+        launch.njobs = 1;
+        launch.cols = C;
+        launch.tokens = B - first < 4 ? B - first : 4;
+        launch.total_tiles = (R + 63) / 64;
+        if (fp4_launch(launch, chains, (hipStream_t)stream) != 0) { set_error("nvfp4 matvec: launch failed"); return -1; }
+    }
+    return 0;
+}
+
+int salt_mi355_router_topk_dev(const float *logits, const float *per_expert_scale, int n_experts, int topk,
+                               int sorted_by_id, int *selected, float *weights, int *status_dev, void *stream) {
+    if (!g_state.ready) { set_error("router: library not initialised"); return -1; }
+    if (!logits || !per_expert_scale || !selected || !weights || !status_dev) { set_error("router: null argument"); return -1; }
+    if (router_topk_launch(logits, per_expert_scale, n_experts, topk, sorted_by_id, selected, weights, status_dev,
+                           (hipStream_t)stream) != 0) {
+        set_error("router: unsupported geometry (experts %d, topk %d) or launch failure", n_experts, topk);
+        return -1;
+    }
+    return 0;
+}
+
+size_t salt_mi355_moe_workspace_bytes(int hidden, int routed, int n_experts, int topk) {
+    if (hidden < 1 || routed < 1 || n_experts < 1 || topk < 1) return 0;
+    const MoeGeometry g = {hidden, routed, n_experts, topk};
+    return moe_workspace_bytes(g);
+}
+
+int salt_mi355_moe_decode_step_dev(const void *pool, size_t expert_stride, int hidden, int routed, int n_experts,
+                                   int topk, const float *logits, const float *per_expert_scale, const float *x,
+                                   int *selected, float *weights, float *expert_out, float *out, void *workspace,
+                                   void *stream) {
+    if (!g_state.ready) { set_error("moe step: library not initialised"); return -1; }
+    if (!pool || !logits || !per_expert_scale || !x || !selected || !weights || !out || !workspace ||
+        ((uintptr_t)pool & 15) || (expert_stride & 15) || ((uintptr_t)workspace & 255)) {
+        set_error("moe step: bad arguments (pool and expert stride 16-byte aligned, workspace 256-byte aligned)");
+        return -1;
+    }
+    const MoeGeometry g = {hidden, routed, n_experts, topk};
+    const size_t n = (size_t)hidden * (size_t)routed;
+    if (hidden < 64 || (hidden & 63) || routed < 64 || (routed & 63) || expert_stride < 3 * (n / 2 + 4 * (n / 64))) {
+        set_error("moe step: hidden and routed must be multiples of 64 and the stride must cover a slot");
+        return -1;
+    }
+    MoeWorkspace ws;
+    moe_workspace_carve(g, workspace, &ws);
+    if (moe_decode_step_launch(g, (const uint8_t *)pool, expert_stride, logits, per_expert_scale, x, selected, weights,
+                               expert_out, out, ws, g_state.code_scale, (hipStream_t)stream) != 0) {
+        set_error("moe step: unsupported geometry or launch failure");
+        return -1;
+    }
+    return 0;
+}
+
+int salt_mi355_moe_activate_dev(const float *gate, const float *up, float *act, size_t n, void *stream) {
+    if (!g_state.ready || !gate || !up || !act || n < 1) { set_error("moe activate: bad arguments"); return -1; }
+    return moe_activate_launch(gate, up, act, n, (hipStream_t)stream);
+}
+
+int salt_mi355_moe_reduce_dev(const float *expert_out, const float *weights, int topk, int hidden, float *out,
+                              void *stream) {
+    if (!g_state.ready || !expert_out || !weights || !out || topk < 1 || hidden < 1) {
+        set_error("moe reduce: bad arguments");
+        return -1;
+    }
+    return moe_reduce_launch(expert_out, weights, topk, hidden, out, (hipStream_t)stream);
+}
+
+}  // extern "C"

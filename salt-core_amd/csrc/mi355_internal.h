@@ -32,6 +32,7 @@ struct Q4Launch {
     int tokens;               // 1..4 activation rows per job
     int total_tiles;
     float code_scale;         // 1 / (value the fp8 converter gives byte 1)
+    int fused;                // 0: separately rounded multiply and add (bit-exact); 1: fma accumulate
 };
 
 // chains_per_lane: 8, 4 or 2; 0 lets the launcher choose from the tile count.
@@ -50,12 +51,11 @@ struct Fp4Job {
     const uint8_t *packed;    // E2M1 codes, two per byte, C/2 bytes per row
     const uint8_t *scales;    // E4M3FN, one per 16 columns
     const float *x;           // [tokens][x_stride] activation used as given
-    float *y;                 // [tokens][y_stride]
+    float *y;                 // [tokens][rows]
     float weight_global_scale;  // 1 / stored divisor
     int rows;
     int tile0;
     int x_stride;
-    int y_stride;
 };
 
 struct Fp4Launch {
@@ -96,8 +96,10 @@ struct MoeWorkspace {
 size_t moe_workspace_bytes(const MoeGeometry &g);
 void moe_workspace_carve(const MoeGeometry &g, void *base, MoeWorkspace *ws);
 
+// sorted_by_id = 0: descending logit order (what the reference function returns);
+// 1: ascending expert id (what its callers turn that into before running experts)
 int router_topk_launch(const float *logits, const float *per_expert_scale, int n_experts, int topk,
-                       int *selected, float *weights, int *status, hipStream_t stream);
+                       int sorted_by_id, int *selected, float *weights, int *status, hipStream_t stream);
 
 int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_stride,
                            const float *logits, const float *per_expert_scale, const float *x,

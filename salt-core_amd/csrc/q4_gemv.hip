@@ -103,17 +103,17 @@ __device__ __forceinline__ void nibbles_to_f32(uint32_t w, float (&q)[8]) {
     q[4] = c.x; q[5] = d.x; q[6] = c.y; q[7] = d.y;
 }
 
-// One packed word of a lane: nibble n belongs to block (n / S) of the word's
-// span and to the lane's chain (n % S).  xw points at x for the span's first
-// block and the wave's first chain; it is wave-uniform.
-template <int S, int NB, int NNIB, bool SLOW>
-__device__ __forceinline__ void consume_word(uint32_t w, float scale, float bias, float code_scale,
-                                             uniform_f32_ptr xw, int x_stride, float (&acc)[NB][S]) {
+// One packed word of a lane.  Nibble n belongs to block (first_block + n / S)
+// of its scale group and to the lane's chain (n % S).  x holds the wave's
+// activations in SGPRs: x[token][xbase + block * S + chain].
+template <int S, int NB, int XN, int NNIB, bool SLOW, bool FUSED>
+__device__ __forceinline__ void consume_word(uint32_t w, int first_block, int xbase, float scale, float bias,
+                                             const float (&x)[NB][XN], float code_scale, float (&acc)[NB][S]) {
     float q[8];
     nibbles_to_f32(w, q);
 #pragma unroll
     for (int n = 0; n < NNIB; ++n) {
-        const int blk = (S == 8) ? 0 : n / S;
+        const int blk = first_block + ((S == 8) ? 0 : n / S);
         const int ch = n % S;
         float wgt;
         if (!SLOW) {
@@ -125,13 +125,24 @@ __device__ __forceinline__ void consume_word(uint32_t w, float scale, float bias
         }
 #pragma unroll
         for (int t = 0; t < NB; ++t) {
-            const float p = wgt * xw[(size_t)t * x_stride + blk * 32 + ch];
-            acc[t][ch] = acc[t][ch] + p;
+            const float xv = x[t][xbase + blk * S + ch];
+            if (FUSED) {
+                acc[t][ch] = __builtin_fmaf(wgt, xv, acc[t][ch]);
+            } else {
+                const float p = wgt * xv;
+                acc[t][ch] = acc[t][ch] + p;
+            }
         }
     }
 }
 
-template <int S, int NB>
+// How many 64-column groups of activations are fetched into SGPRs at once.
+constexpr int x_batch_groups(int S, int NB) {
+    const int fit = (S == 8 ? 32 : 64) / (2 * S * NB);     // SGPR budget for activations
+    return fit >= 8 ? 8 : fit >= 4 ? 4 : fit >= 2 ? 2 : 1;
+}
+
+template <int S, int NB, bool FUSED>
 __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L) {
     constexpr int WAVES = 32 / S;
     constexpr int THREADS = WAVES * 64;
@@ -139,6 +150,8 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
     constexpr int META_ITEMS = (TILE_ROWS * CHUNK_GROUPS + THREADS - 1) / THREADS;
     constexpr int FOLD_BYTES = NB * TILE_ROWS * FOLD_PITCH * 4;
     constexpr int W_BYTES = 2 * W_STAGE > FOLD_BYTES ? 2 * W_STAGE : FOLD_BYTES;
+    constexpr int XG = x_batch_groups(S, NB);
+    constexpr int XN = XG * 2 * S;
     static_assert(THREADS >= NB * TILE_ROWS, "fold needs one thread per (token, row)");
 
     __shared__ __attribute__((aligned(16))) uint8_t w_lds[W_BYTES];
@@ -152,69 +165,80 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
     const Q4Job job = find_job(L, blockIdx.x);
     const int row0 = (blockIdx.x - job.tile0) * TILE_ROWS;
     const int R = job.rows;
+    const int rows_here = R - row0 < TILE_ROWS ? R - row0 : TILE_ROWS;
     const int nblk = L.cols >> 5;
     const int ngrp = L.cols >> 6;
     const int nchunk = (nblk + CHUNK_BLOCKS - 1) / CHUNK_BLOCKS;
-    const size_t row_bytes = (size_t)(L.cols >> 1);
-    const global_u8_ptr vals = (global_u8_ptr)(uintptr_t)job.vals;
-    const global_u16_ptr scales16 = (global_u16_ptr)(uintptr_t)job.scales;
-    const global_u16_ptr biases16 = (global_u16_ptr)(uintptr_t)job.biases;
+    const uint32_t row_bytes = (uint32_t)(L.cols >> 1);
+    // wave-uniform bases of this tile; per-thread parts are 32-bit offsets
+    const global_u8_ptr vals = (global_u8_ptr)(uintptr_t)job.vals + (size_t)row0 * row_bytes;
+    const global_u16_ptr scales16 = (global_u16_ptr)(uintptr_t)job.scales + (size_t)row0 * ngrp;
+    const global_u16_ptr biases16 =
+        job.biases ? (global_u16_ptr)(uintptr_t)job.biases + (size_t)row0 * ngrp : (global_u16_ptr)0;
     const global_f32_out_ptr y = (global_f32_out_ptr)(uintptr_t)job.y;
+    const uniform_f32_ptr xbase = as_uniform(job.x) + S * wave;
+
+    // Per-thread staging geometry, fixed for the whole tile.  Piece i of a
+    // thread lies (THREADS / 16) rows below piece 0 in the same 16-byte column,
+    // so only the clamped source row offsets need registers.
+    constexpr int W_ROW_STEP = THREADS / 16, M_ROW_STEP = THREADS / 8;
+    const uint32_t w_seg = tid & 15;
+    const uint32_t w_dst0 = (tid >> 4) * W_PITCH + w_seg * 16;
+    uint32_t w_src[PIECES];
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i) {
+        const int row = (tid >> 4) + i * W_ROW_STEP;
+        w_src[i] = (uint32_t)(row < rows_here ? row : rows_here - 1) * row_bytes;
+    }
+    const bool has_meta = tid < TILE_ROWS * CHUNK_GROUPS;    // only narrower than the block when THREADS == 1024
+    const uint32_t m_grp = tid & 7;
+    const uint32_t m_dst0 = ((tid >> 3) & (TILE_ROWS - 1)) * M_PITCH + 2 * m_grp;
+    uint32_t m_src[META_ITEMS];
+#pragma unroll
+    for (int i = 0; i < META_ITEMS; ++i) {
+        const int row = ((tid >> 3) + i * M_ROW_STEP) & (TILE_ROWS - 1);
+        m_src[i] = (uint32_t)(row < rows_here ? row : rows_here - 1) * ngrp;
+    }
 
     u32x4 wreg[PIECES];
     uint32_t mreg[META_ITEMS];
 
+    // Loads of step ck into registers.  Block and group indices past the end
+    // of the row (last step only) are clamped: the data is staged but never
+    // consumed.
     auto issue = [&](int ck) {
 #pragma unroll
         for (int i = 0; i < PIECES; ++i) {
-            const int p = tid + i * THREADS;
-            const int row = p >> 4, seg = p & 15;
-            const int blk = ck * CHUNK_BLOCKS + seg;
-            int r = row0 + row;
-            r = r < R ? r : R - 1;
-            if (blk < nblk)
-                wreg[i] = *(global_u128_ptr)(vals + (size_t)r * row_bytes + (size_t)blk * 16);
-            else
-                wreg[i] = u32x4{0, 0, 0, 0};
+            int blk = ck * CHUNK_BLOCKS + (int)w_seg;
+            blk = blk < nblk ? blk : nblk - 1;
+            wreg[i] = *(global_u128_ptr)(vals + (w_src[i] + (uint32_t)blk * 16u));
         }
 #pragma unroll
         for (int i = 0; i < META_ITEMS; ++i) {
-            const int it = tid + i * THREADS;
-            mreg[i] = 0;
-            if (it < TILE_ROWS * CHUNK_GROUPS) {
-                const int row = it >> 3;
-                const int g = ck * CHUNK_GROUPS + (it & 7);
-                int r = row0 + row;
-                r = r < R ? r : R - 1;
-                if (g < ngrp) {
-                    const size_t gi = (size_t)r * ngrp + g;
-                    const uint32_t s = scales16[gi];
-                    const uint32_t b = biases16 ? biases16[gi] : 0u;
-                    mreg[i] = s | (b << 16);
-                }
-            }
+            int g = ck * CHUNK_GROUPS + (int)m_grp;
+            g = g < ngrp ? g : ngrp - 1;
+            const uint32_t at = m_src[i] + (uint32_t)g;
+            const uint32_t sbits = scales16[at];
+            const uint32_t bbits = biases16 ? (uint32_t)biases16[at] : 0u;
+            mreg[i] = sbits | (bbits << 16);
         }
     };
 
     auto commit = [&](int stage) {
 #pragma unroll
         for (int i = 0; i < PIECES; ++i) {
-            const int p = tid + i * THREADS;
-            const int row = p >> 4, seg = p & 15;
-            uint32_t *dst = reinterpret_cast<uint32_t *>(w_lds + stage * W_STAGE + row * W_PITCH + seg * 16);
+            uint32_t *dst = reinterpret_cast<uint32_t *>(w_lds + stage * W_STAGE + w_dst0 + i * W_ROW_STEP * W_PITCH);
             dst[0] = wreg[i].x; dst[1] = wreg[i].y; dst[2] = wreg[i].z; dst[3] = wreg[i].w;
         }
+        if (has_meta) {
 #pragma unroll
-        for (int i = 0; i < META_ITEMS; ++i) {
-            const int it = tid + i * THREADS;
-            if (it < TILE_ROWS * CHUNK_GROUPS) {
-                const int row = it >> 3;
-                const float s = bf16_to_f32(mreg[i] & 0xFFFFu);
-                const float b = bf16_to_f32(mreg[i] >> 16);
-                if (!(__builtin_fabsf(s) < BIG_SCALE)) slow_flag = 1;
-                float *dst = m_lds + stage * M_STAGE + row * M_PITCH + 2 * (it & 7);
-                dst[0] = s * L.code_scale;
-                dst[1] = b;
+            for (int i = 0; i < META_ITEMS; ++i) {
+                const float sc = bf16_to_f32(mreg[i] & 0xFFFFu);
+                const float bi = __uint_as_float(mreg[i] & 0xFFFF0000u);
+                if (!(__builtin_fabsf(sc) < BIG_SCALE)) slow_flag = 1;
+                float *dst = m_lds + stage * M_STAGE + m_dst0 + i * M_ROW_STEP * M_PITCH;
+                dst[0] = sc * L.code_scale;
+                dst[1] = bi;
             }
         }
     };
@@ -229,27 +253,42 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
     issue(0);
     __syncthreads();
 
-    int my_row = row0 + lane;
-    my_row = my_row < R ? my_row : R - 1;
+    const int my_row = lane < rows_here ? lane : rows_here - 1;
+
+    // x of `groups` consecutive scale groups starting at group g0 of the row
+    auto load_x = [&](int g0, float (&xq)[NB][XN], int groups) {
+        const uniform_f32_ptr xg = xbase + (size_t)g0 * 64;
+#pragma unroll
+        for (int t = 0; t < NB; ++t)
+#pragma unroll
+            for (int k = 0; k < XN; ++k)
+                if (k < groups * 2 * S) xq[t][k] = xg[(size_t)t * job.x_stride + (k / S) * 32 + (k % S)];
+    };
 
     for (int ck = 0; ck < nchunk; ++ck) {
         const int stage = ck & 1;
+        const int remaining = ngrp - ck * CHUNK_GROUPS;
+        const bool full = remaining >= CHUNK_GROUPS;
+        const int gcount = full ? CHUNK_GROUPS : remaining;
+
+        // The first batch of activations is requested before the barrier so
+        // that its latency overlaps the staging writes and the wait.
+        float xq[NB][XN];
+        if (full) load_x(ck * CHUNK_GROUPS, xq, XG);
+
         commit(stage);
         __syncthreads();
         if (ck + 1 < nchunk) issue(ck + 1);
 
         const int slow = __builtin_amdgcn_readfirstlane(slow_flag);
-        const int remaining = ngrp - ck * CHUNK_GROUPS;
-        const int gcount = remaining < CHUNK_GROUPS ? remaining : CHUNK_GROUPS;
         const uint8_t *wrow = w_lds + stage * W_STAGE + lane * W_PITCH + wave * (S / 2);
         const float *mrow = m_lds + stage * M_STAGE + lane * M_PITCH;
 
-        for (int g = 0; g < gcount; ++g) {
-            float scale = mrow[2 * g];
-            const float bias = mrow[2 * g + 1];
-            const int blk = ck * CHUNK_BLOCKS + 2 * g;
-            uniform_f32_ptr xg = as_uniform(job.x) + (size_t)blk * 32 + S * wave;
-            uint32_t w0, w1 = 0;
+        // LDS operands of group g of this step: the lane's nibbles and (scale', bias)
+        auto fetch = [&](int g, uint32_t &w0, uint32_t &w1, float &scale, float &bias) {
+            scale = mrow[2 * g];
+            bias = mrow[2 * g + 1];
+            w1 = 0;
             if (S == 8) {
                 w0 = *reinterpret_cast<const uint32_t *>(wrow + (2 * g) * 16);
                 w1 = *reinterpret_cast<const uint32_t *>(wrow + (2 * g + 1) * 16);
@@ -262,20 +301,51 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
                 const uint32_t b = wrow[(2 * g + 1) * 16];
                 w0 = a | (b << 8);
             }
-            if (__builtin_expect(slow, 0)) {
-                scale = bf16_to_f32(scales16[(size_t)my_row * ngrp + ck * CHUNK_GROUPS + g]);
-                if (S == 8) {
-                    consume_word<S, NB, 8, true>(w0, scale, bias, L.code_scale, xg, job.x_stride, acc);
-                    consume_word<S, NB, 8, true>(w1, scale, bias, L.code_scale, xg + 32, job.x_stride, acc);
-                } else {
-                    consume_word<S, NB, (S == 4 ? 8 : 4), true>(w0, scale, bias, L.code_scale, xg, job.x_stride, acc);
+        };
+
+        if (full && !slow) {
+            // Straight-line code over the eight groups of a full step.
+#pragma unroll
+            for (int batch = 0; batch < CHUNK_GROUPS / XG; ++batch) {
+                if (batch > 0) load_x(ck * CHUNK_GROUPS + batch * XG, xq, XG);
+#pragma unroll
+                for (int gl = 0; gl < XG; ++gl) {
+                    uint32_t w0, w1;
+                    float scale, bias;
+                    fetch(batch * XG + gl, w0, w1, scale, bias);
+                    if (S == 8) {
+                        consume_word<S, NB, XN, 8, false, FUSED>(w0, 0, gl * 2 * S, scale, bias, xq, L.code_scale, acc);
+                        consume_word<S, NB, XN, 8, false, FUSED>(w1, 1, gl * 2 * S, scale, bias, xq, L.code_scale, acc);
+                    } else {
+                        consume_word<S, NB, XN, (S == 4 ? 8 : 4), false, FUSED>(w0, 0, gl * 2 * S, scale, bias, xq,
+                                                                                 L.code_scale, acc);
+                    }
                 }
-            } else {
-                if (S == 8) {
-                    consume_word<S, NB, 8, false>(w0, scale, bias, L.code_scale, xg, job.x_stride, acc);
-                    consume_word<S, NB, 8, false>(w1, scale, bias, L.code_scale, xg + 32, job.x_stride, acc);
+            }
+        } else {
+            // Partial last step, or a tile that met an out-of-range scale.
+            for (int g = 0; g < gcount; ++g) {
+                uint32_t w0, w1;
+                float scale, bias;
+                fetch(g, w0, w1, scale, bias);
+                load_x(ck * CHUNK_GROUPS + g, xq, 1);
+                if (slow) {
+                    scale = bf16_to_f32(scales16[(uint32_t)my_row * ngrp + ck * CHUNK_GROUPS + g]);
+                    if (S == 8) {
+                        consume_word<S, NB, XN, 8, true, FUSED>(w0, 0, 0, scale, bias, xq, L.code_scale, acc);
+                        consume_word<S, NB, XN, 8, true, FUSED>(w1, 1, 0, scale, bias, xq, L.code_scale, acc);
+                    } else {
+                        consume_word<S, NB, XN, (S == 4 ? 8 : 4), true, FUSED>(w0, 0, 0, scale, bias, xq,
+                                                                                L.code_scale, acc);
+                    }
                 } else {
-                    consume_word<S, NB, (S == 4 ? 8 : 4), false>(w0, scale, bias, L.code_scale, xg, job.x_stride, acc);
+                    if (S == 8) {
+                        consume_word<S, NB, XN, 8, false, FUSED>(w0, 0, 0, scale, bias, xq, L.code_scale, acc);
+                        consume_word<S, NB, XN, 8, false, FUSED>(w1, 1, 0, scale, bias, xq, L.code_scale, acc);
+                    } else {
+                        consume_word<S, NB, XN, (S == 4 ? 8 : 4), false, FUSED>(w0, 0, 0, scale, bias, xq,
+                                                                                 L.code_scale, acc);
+                    }
                 }
             }
         }
@@ -299,8 +369,7 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
             for (int j = 0; j < 4; ++j) part[j] = part[j] + f[4 * a + j];
         const float even = part[0] + part[2];
         const float odd = part[1] + part[3];
-        const int row = row0 + lane;
-        if (row < R) y[(size_t)t * job.y_stride + row] = even + odd;
+        if (lane < rows_here) y[(size_t)t * job.y_stride + row0 + lane] = even + odd;
     }
 }
 
@@ -359,14 +428,14 @@ __global__ __launch_bounds__(256) void q4_generic_kernel(const Q4Launch L) {
     }
 }
 
-template <int S>
+template <int S, bool FUSED>
 int launch_tiles(const Q4Launch &L, hipStream_t stream) {
     const dim3 grid(L.total_tiles), block((32 / S) * 64);
     switch (L.tokens) {
-        case 1: hipLaunchKernelGGL((q4_tile_kernel<S, 1>), grid, block, 0, stream, L); break;
-        case 2: hipLaunchKernelGGL((q4_tile_kernel<S, 2>), grid, block, 0, stream, L); break;
-        case 3: hipLaunchKernelGGL((q4_tile_kernel<S, 3>), grid, block, 0, stream, L); break;
-        case 4: hipLaunchKernelGGL((q4_tile_kernel<S, 4>), grid, block, 0, stream, L); break;
+        case 1: hipLaunchKernelGGL((q4_tile_kernel<S, 1, FUSED>), grid, block, 0, stream, L); break;
+        case 2: hipLaunchKernelGGL((q4_tile_kernel<S, 2, FUSED>), grid, block, 0, stream, L); break;
+        case 3: hipLaunchKernelGGL((q4_tile_kernel<S, 3, FUSED>), grid, block, 0, stream, L); break;
+        case 4: hipLaunchKernelGGL((q4_tile_kernel<S, 4, FUSED>), grid, block, 0, stream, L); break;
         default: return -1;
     }
     return hipGetLastError() == hipSuccess ? 0 : -1;
@@ -407,10 +476,18 @@ int q4_launch(const Q4Launch &L, int chains_per_lane, hipStream_t stream) {
         else if (L.total_tiles * 8 >= 2048) S = 4;
         else S = 2;
     }
+    if (L.fused) {
+        switch (S) {
+            case 8: return launch_tiles<8, true>(L, stream);
+            case 4: return launch_tiles<4, true>(L, stream);
+            case 2: return launch_tiles<2, true>(L, stream);
+            default: return -1;
+        }
+    }
     switch (S) {
-        case 8: return launch_tiles<8>(L, stream);
-        case 4: return launch_tiles<4>(L, stream);
-        case 2: return launch_tiles<2>(L, stream);
+        case 8: return launch_tiles<8, false>(L, stream);
+        case 4: return launch_tiles<4, false>(L, stream);
+        case 2: return launch_tiles<2, false>(L, stream);
         default: return -1;
     }
 }

@@ -51,6 +51,13 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_event_elapsed_ms, i, vp, vp, C.POINTER(f))
     _sig(lib.salt_mi355_q4_matvec_dev, i, vp, vp, vp, i, i, i, vp, vp, i, vp)
     _sig(lib.salt_mi355_q4_jobs_dev, i, C.POINTER(Q4Job), i, i, i, i, vp)
+    _sig(lib.salt_mi355_nvfp4_qdq_dev, i, vp, i, i, f, vp, vp, vp, vp, vp)
+    _sig(lib.salt_mi355_nvfp4_matvec_dev, i, vp, vp, f, i, i, i, vp, vp, i, vp)
+    _sig(lib.salt_mi355_router_topk_dev, i, vp, vp, i, i, i, vp, vp, vp, vp)
+    _sig(lib.salt_mi355_moe_workspace_bytes, sz, i, i, i, i)
+    _sig(lib.salt_mi355_moe_decode_step_dev, i, vp, sz, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, vp, vp)
+    _sig(lib.salt_mi355_moe_activate_dev, i, vp, vp, vp, sz, vp)
+    _sig(lib.salt_mi355_moe_reduce_dev, i, vp, vp, i, i, vp, vp)
     _lib = lib
     return lib
 
@@ -131,3 +138,84 @@ def q4_matvec(vals: np.ndarray, scales: np.ndarray, biases: np.ndarray | None, R
                                        chains, stream), "q4_matvec_dev")
     check(lib.salt_mi355_stream_sync(stream), "sync")
     return dy.to_host(np.float32).reshape(B, R)
+
+
+def nvfp4_qdq(x: np.ndarray, g: float):
+    """Host-array convenience around salt_mi355_nvfp4_qdq_dev.  Returns
+    (status, packed, scales, dequant)."""
+    lib = init()
+    x = np.ascontiguousarray(x, np.float32)
+    B, C_ = (1, x.shape[0]) if x.ndim == 1 else x.shape
+    dx = DeviceBuffer.from_host(x)
+    dp, ds, dd = DeviceBuffer(B * C_ // 2, fill=0), DeviceBuffer(B * C_ // 16, fill=0), DeviceBuffer(B * C_ * 4, fill=0)
+    st = DeviceBuffer(4, fill=0)
+    stream = lib.salt_mi355_stream()
+    check(lib.salt_mi355_nvfp4_qdq_dev(dx.ptr, C_, B, g, dp.ptr, ds.ptr, dd.ptr, st.ptr, stream), "nvfp4_qdq_dev")
+    check(lib.salt_mi355_stream_sync(stream), "sync")
+    return (int(st.to_host(np.int32)[0]), dp.to_host(np.uint8), ds.to_host(np.uint8),
+            dd.to_host(np.float32).reshape(x.shape))
+
+
+def nvfp4_matvec(packed: np.ndarray, scales: np.ndarray, divisor: float, R: int, C_: int, xs: np.ndarray,
+                 input_global_scale: float | None = 64.0, chains: int = 0):
+    """The reference matvec: activation Q/DQ (skipped when input_global_scale
+    is None) followed by the rows.  Returns (status, ys[B, R])."""
+    lib = init()
+    xs = np.ascontiguousarray(xs, np.float32).reshape(-1, C_)
+    B = xs.shape[0]
+    dw, ds, dx = DeviceBuffer.from_host(packed), DeviceBuffer.from_host(scales), DeviceBuffer.from_host(xs)
+    dq = DeviceBuffer(B * C_ * 4)
+    dy = DeviceBuffer(B * R * 4, fill=0xFF)
+    st = DeviceBuffer(4, fill=0)
+    stream = lib.salt_mi355_stream()
+    src = dx
+    if input_global_scale is not None:
+        check(lib.salt_mi355_nvfp4_qdq_dev(dx.ptr, C_, B, input_global_scale, None, None, dq.ptr, st.ptr, stream),
+              "nvfp4_qdq_dev")
+        src = dq
+    check(lib.salt_mi355_nvfp4_matvec_dev(dw.ptr, ds.ptr, divisor, R, C_, B, src.ptr, dy.ptr, chains, stream),
+          "nvfp4_matvec_dev")
+    check(lib.salt_mi355_stream_sync(stream), "sync")
+    return int(st.to_host(np.int32)[0]), dy.to_host(np.float32).reshape(B, R)
+
+
+def router_topk(logits: np.ndarray, scale: np.ndarray, topk: int, sorted_by_id: bool = False):
+    lib = init()
+    E = logits.shape[0]
+    dl, dsc = DeviceBuffer.from_host(logits.astype(np.float32)), DeviceBuffer.from_host(scale.astype(np.float32))
+    sel, w, st = DeviceBuffer(topk * 4, fill=0xEE), DeviceBuffer(topk * 4, fill=0xEE), DeviceBuffer(4, fill=0x7F)
+    stream = lib.salt_mi355_stream()
+    check(lib.salt_mi355_router_topk_dev(dl.ptr, dsc.ptr, E, topk, int(sorted_by_id), sel.ptr, w.ptr, st.ptr, stream),
+          "router_topk_dev")
+    check(lib.salt_mi355_stream_sync(stream), "sync")
+    return int(st.to_host(np.int32)[0]), sel.to_host(np.int32), w.to_host(np.float32)
+
+
+class MoeLayer:
+    """One layer's expert pool resident in HBM plus the step workspace."""
+
+    def __init__(self, pool: np.ndarray, n_experts: int, hidden: int, routed: int, topk: int):
+        self.lib = init()
+        self.E, self.H, self.F, self.K = n_experts, hidden, routed, topk
+        self.stride = pool.nbytes // n_experts
+        self.pool = DeviceBuffer.from_host(pool)
+        self.ws = DeviceBuffer(self.lib.salt_mi355_moe_workspace_bytes(hidden, routed, n_experts, topk), fill=0)
+        self.logits, self.scale = DeviceBuffer(n_experts * 4), DeviceBuffer(n_experts * 4)
+        self.x, self.out = DeviceBuffer(hidden * 4), DeviceBuffer(hidden * 4)
+        self.sel, self.w = DeviceBuffer(topk * 4), DeviceBuffer(topk * 4)
+        self.eo = DeviceBuffer(topk * hidden * 4)
+
+    def enqueue(self, stream):
+        return self.lib.salt_mi355_moe_decode_step_dev(
+            self.pool.ptr, self.stride, self.H, self.F, self.E, self.K, self.logits.ptr, self.scale.ptr, self.x.ptr,
+            self.sel.ptr, self.w.ptr, self.eo.ptr, self.out.ptr, self.ws.ptr, stream)
+
+    def step(self, logits, scale, x):
+        self.logits.upload(logits.astype(np.float32)); self.scale.upload(scale.astype(np.float32))
+        self.x.upload(x.astype(np.float32))
+        stream = self.lib.salt_mi355_stream()
+        check(self.enqueue(stream), "moe_decode_step_dev")
+        check(self.lib.salt_mi355_stream_sync(stream), "sync")
+        status = int(self.ws.to_host(np.int32, 1)[0])
+        return (status, self.sel.to_host(np.int32), self.w.to_host(np.float32),
+                self.eo.to_host(np.float32).reshape(self.K, self.H), self.out.to_host(np.float32))
