@@ -1,0 +1,243 @@
+#!/usr/bin/env python3
+"""Throughput of the affine-Q4 decode matvec path on one MI355X.
+
+A step is one pass of the decode-shape sweep (BASELINE.json configs[1], batch
+1): for each (K, N) in {(2816, 2816), (2816, 16384), (8192, 2816)} one launch
+of the bit-exact Q4 kernel over G distinct weight instances resident in HBM
+(G chosen so that every launch streams more than the 256 MB Infinity Cache can
+hold), the way the engine's batched entry point dispatches many matrices at
+once (reference salt_gpu_q4_batch, include/salt/gpu.h:83).  `value` is the
+algorithmic bytes of a step (0.5625 B per weight element plus activations and
+outputs) divided by the step time, weights already resident when the timed
+region starts.
+
+The JSON line also carries the roofline of the dominant kernel (achieved HBM
+GB/s against 8 TB/s), the same sweep timed on the host cores with the
+reference's own C kernel when oracle/_ref is present (else the checker's
+port), and, under "extra", the MoE decode layer-step, the NVFP4 matvec and the
+batch-4 sweep.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path[:0] = [str(ROOT), str(ROOT / "tests")]
+
+HBM_PEAK_GBS = 8000.0
+SWEEP = [(2816, 2816), (16384, 2816), (2816, 8192)]        # (R, C) = (N, K)
+INSTANCE_BYTES = 640e6                                      # distinct weight bytes per launch
+
+
+class Events:
+    def __init__(self, lib, stream):
+        self.lib, self.stream = lib, stream
+        self.a, self.b = lib.salt_mi355_event_create(), lib.salt_mi355_event_create()
+
+    def start(self):
+        self.lib.salt_mi355_event_record(self.a, self.stream)
+
+    def stop_ms(self) -> float:
+        self.lib.salt_mi355_event_record(self.b, self.stream)
+        ms = C.c_float()
+        assert self.lib.salt_mi355_event_elapsed_ms(self.a, self.b, C.byref(ms)) == 0
+        return float(ms.value)
+
+
+class Q4Sweep:
+    """The three decode shapes, G instances each, one multi-job launch per shape."""
+
+    def __init__(self, gpu, synth, tokens: int):
+        self.gpu, self.lib, self.tokens = gpu, gpu.load(), tokens
+        self.launches, self.keep = [], []
+        self.bytes_per_step = 0
+        for seed, (R, Cc) in enumerate(SWEEP):
+            vals, scales, biases = synth.q4_tensor(R, Cc, 100 + seed)
+            per = vals.nbytes + scales.nbytes + biases.nbytes
+            G = max(2, int(INSTANCE_BYTES // per))
+            weights = gpu.DeviceBuffer(per * G)
+            for g in range(G):
+                weights.upload(vals, g * per)
+                weights.upload(scales, g * per + vals.nbytes)
+                weights.upload(biases, g * per + vals.nbytes + scales.nbytes)
+            xs = gpu.DeviceBuffer.from_host(synth.activations(Cc, tokens, 200 + seed))
+            ys = gpu.DeviceBuffer(G * tokens * R * 4)
+            jobs = (gpu.Q4Job * G)()
+            for g in range(G):
+                jobs[g] = gpu.Q4Job(weights.at(g * per), weights.at(g * per + vals.nbytes),
+                                    weights.at(g * per + vals.nbytes + scales.nbytes), xs.ptr,
+                                    ys.at(g * tokens * R * 4), R)
+            self.keep += [weights, xs, ys]
+            self.launches.append((jobs, G, Cc))
+            self.bytes_per_step += G * synth.q4_bytes(R, Cc, tokens)
+
+    def step(self, stream):
+        for jobs, G, Cc in self.launches:
+            rc = self.lib.salt_mi355_q4_jobs_dev(jobs, G, Cc, self.tokens, 0, stream)
+            if rc != 0:
+                raise RuntimeError(self.lib.salt_mi355_last_error().decode())
+
+
+def timed(lib, stream, events, fn, warmup, steps):
+    for _ in range(warmup):
+        fn(stream)
+    assert lib.salt_mi355_stream_sync(stream) == 0
+    events.start()
+    for _ in range(steps):
+        fn(stream)
+    ms = events.stop_ms()
+    assert lib.salt_mi355_stream_sync(stream) == 0
+    return ms / steps
+
+
+def cpu_baseline(synth, budget_s: float = 12.0):
+    """The same sweep (one instance per shape, batch 1) on the host cores."""
+    from oracle_lib import load_oracle, load_reference, ptr
+    cores = max(1, min(16, len(os.sched_getaffinity(0))))
+    os.environ.setdefault("SALT_ATTN_THREADS", str(cores))
+    ref = load_reference()
+    oracle = load_oracle()
+    cases = []
+    for seed, (R, Cc) in enumerate(SWEEP):
+        vals, scales, biases = synth.q4_tensor(R, Cc, 100 + seed)
+        x = synth.activations(Cc, 1, 200 + seed)[0]
+        cases.append((R, Cc, vals, scales, biases, x, np.zeros(R, np.float32)))
+
+    def one_pass():
+        for R, Cc, vals, scales, biases, x, y in cases:
+            if ref is not None:
+                ref.salt_q4_matvec(ptr(vals), ptr(scales), ptr(biases), R, Cc, ptr(x), ptr(y))
+            else:
+                oracle.orc_q4_matvec_threads(ptr(vals), ptr(scales), ptr(biases), R, Cc, ptr(x), ptr(y), cores)
+
+    one_pass()
+    t0 = time.perf_counter()
+    one_pass()
+    once = time.perf_counter() - t0
+    reps = max(3, min(20000, int(budget_s / max(once, 1e-6))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        one_pass()
+    elapsed = time.perf_counter() - t0
+    nbytes = sum(synth.q4_bytes(R, Cc, 1) for R, Cc in SWEEP)
+    threads = int(os.environ["SALT_ATTN_THREADS"]) if ref is not None else cores
+    return {
+        "value": round(nbytes * reps / elapsed / 1e9, 3), "unit": "GB/s", "cores": threads,
+        "kind": "reference" if ref is not None else "port",
+        "sample": f"{reps} passes of the 3-shape sweep, one weight instance per shape, batch 1, "
+                  f"{elapsed:.1f} s; the reference row-splits over {threads} threads when R >= 2048",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the MoE / NVFP4 / batch-4 legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path has no multi-GPU mode (run with --gpus 1)")
+
+    from __graft_entry__ import load_package
+    pkg = load_package()
+    gpu, synth = pkg.lib, pkg.synth
+    lib = gpu.init()
+    stream = lib.salt_mi355_stream()
+    events = Events(lib, stream)
+
+    sweep = Q4Sweep(gpu, synth, tokens=1)
+    ms = timed(lib, stream, events, sweep.step, args.warmup, args.steps)
+    gbs = sweep.bytes_per_step / (ms * 1e-3) / 1e9
+    launches = len(sweep.launches)
+    bytes_per_launch = sweep.bytes_per_step / launches
+    launch_us = ms * 1e3 / launches
+    result = {
+        "metric": "q4_decode_matvec_hbm_gbps", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {
+            "workload": "BASELINE configs[1]: affine-Q4 group-64 decode matvec sweep, batch 1, "
+                        "(K,N) in {(2816,2816),(2816,16384),(8192,2816)}, bit-exact kernel",
+            "instances_per_shape": [g for _, g, _ in sweep.launches],
+            "launches_per_step": launches,
+            "weights": "one seeded instance per shape replicated at distinct HBM addresses",
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": round(bytes_per_launch / (launch_us * 1e-6) / 1e9, 1),
+            "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(bytes_per_launch / (launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            "traffic": None, "kernel": "q4_tile_kernel<4,1,false>",
+            "bytes_per_launch": int(bytes_per_launch), "launch_us": round(launch_us, 2),
+        },
+    }
+    keep_sweep = sweep
+
+    if not args.no_extra:
+        extra = {}
+        del keep_sweep, sweep
+        # batch 4 of the same sweep
+        s4 = Q4Sweep(gpu, synth, tokens=4)
+        ms4 = timed(lib, stream, events, s4.step, 2, max(5, args.steps // 5))
+        extra["q4_sweep_batch4_gbps"] = round(s4.bytes_per_step / (ms4 * 1e-3) / 1e9, 1)
+        del s4
+        # MoE decode layer-step, E = 128 top-8, d_model 2816, d_ff 704; fresh logits per layer instance
+        E, K, H, F = 128, 8, 2816, 704
+        pool = synth.expert_pool(E, H, F, 7)
+        layers = [gpu.MoeLayer(pool, E, H, F, K) for _ in range(2)]
+        for i, layer in enumerate(layers):
+            layer.logits.upload(synth.router_logits(E, 900 + i))
+            layer.scale.upload(np.ones(E, np.float32))
+            layer.x.upload(synth.activations(H, 1, 950 + i)[0])
+
+        def moe_step(st):
+            for layer in layers:
+                if layer.enqueue(st) != 0:
+                    raise RuntimeError(lib.salt_mi355_last_error().decode())
+
+        ms_moe = timed(lib, stream, events, moe_step, 5, 100) / len(layers)
+        step_bytes = synth.moe_step_bytes(H, F, E, K)
+        extra["moe_decode_step_us"] = round(ms_moe * 1e3, 2)
+        extra["moe_layer_tokens_per_s"] = round(1e3 / ms_moe, 1)
+        extra["moe_decode_step_gbps"] = round(step_bytes / (ms_moe * 1e-3) / 1e9, 1)
+        extra["moe_decode_step_hbm_frac"] = round(step_bytes / (ms_moe * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        del layers
+        # NVFP4 8192 x 8192, batch 1, reference semantics (activation Q/DQ + rows), 16 instances
+        R = Cc = 8192
+        packed, fscales = synth.nvfp4_tensor(R, Cc, 40)
+        G = 16
+        per = packed.nbytes + fscales.nbytes
+        w = gpu.DeviceBuffer(per * G)
+        for g in range(G):
+            w.upload(packed, g * per)
+            w.upload(fscales, g * per + packed.nbytes)
+        x = gpu.DeviceBuffer.from_host(synth.activations(Cc, 1, 41))
+        xq, y, st = gpu.DeviceBuffer(Cc * 4), gpu.DeviceBuffer(R * 4), gpu.DeviceBuffer(4, fill=0)
+
+        def fp4_step(s):
+            for g in range(G):
+                lib.salt_mi355_nvfp4_qdq_dev(x.ptr, Cc, 1, 64.0, None, None, xq.ptr, st.ptr, s)
+                lib.salt_mi355_nvfp4_matvec_dev(w.at(g * per), w.at(g * per + packed.nbytes), 2688.0, R, Cc, 1,
+                                                xq.ptr, y.ptr, 0, s)
+
+        ms_fp4 = timed(lib, stream, events, fp4_step, 2, 10) / G
+        extra["nvfp4_8192_matvec_us"] = round(ms_fp4 * 1e3, 2)
+        extra["nvfp4_8192_gbps"] = round(synth.nvfp4_bytes(R, Cc, 1) / (ms_fp4 * 1e-3) / 1e9, 1)
+        result["extra"] = extra
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(synth)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -84,31 +84,36 @@ int verify_converters() {
 
 }  // namespace
 
-// Grows the device copy of a host job table; returns the device pointer.
-void *stage_table(const void *host_table, size_t nbytes, hipStream_t stream) {
+State::TableSlot *table_acquire(const void *host_table, size_t nbytes, hipStream_t stream) {
     State &s = g_state;
-    if (nbytes > s.table_capacity) {
-        if (s.table_device) {
-            if (hip_ok(hipDeviceSynchronize(), "sync before table growth") != 0) return nullptr;
-            (void)hipFree(s.table_device);
-            (void)hipHostFree(s.table_pinned);
-            s.table_device = nullptr; s.table_pinned = nullptr; s.table_capacity = 0;
-        }
-        size_t capacity = 64 * 1024;
-        while (capacity < nbytes) capacity *= 2;
-        if (hip_ok(hipMalloc(&s.table_device, capacity), "hipMalloc job table") != 0 ||
-            hip_ok(hipHostMalloc(&s.table_pinned, capacity, hipHostMallocDefault), "hipHostMalloc job table") != 0)
-            return nullptr;
-        s.table_capacity = capacity;
+    State::TableSlot *slot = &s.tables[s.next_table];
+    s.next_table = (s.next_table + 1) % State::kTableSlots;
+    if (slot->busy) {
+        if (hip_ok(hipEventSynchronize(slot->done), "job table slot reuse") != 0) return nullptr;
+        slot->busy = 0;
     }
-    // The pinned staging copy is reused by the next call, so the previous
-    // upload must have been consumed: tables are tiny, wait for the stream.
-    if (hip_ok(hipStreamSynchronize(stream), "job table reuse") != 0) return nullptr;
-    memcpy(s.table_pinned, host_table, nbytes);
-    if (hip_ok(hipMemcpyAsync(s.table_device, s.table_pinned, nbytes, hipMemcpyHostToDevice, stream),
+    if (nbytes > slot->capacity) {
+        if (slot->device) { (void)hipFree(slot->device); (void)hipHostFree(slot->pinned); }
+        slot->device = slot->pinned = nullptr;
+        slot->capacity = 0;
+        size_t capacity = 16 * 1024;
+        while (capacity < nbytes) capacity *= 2;
+        if (hip_ok(hipMalloc(&slot->device, capacity), "hipMalloc job table") != 0 ||
+            hip_ok(hipHostMalloc(&slot->pinned, capacity, hipHostMallocDefault), "hipHostMalloc job table") != 0)
+            return nullptr;
+        slot->capacity = capacity;
+    }
+    if (!slot->done && hip_ok(hipEventCreateWithFlags(&slot->done, hipEventDisableTiming), "hipEventCreate") != 0)
+        return nullptr;
+    memcpy(slot->pinned, host_table, nbytes);
+    if (hip_ok(hipMemcpyAsync(slot->device, slot->pinned, nbytes, hipMemcpyHostToDevice, stream),
                "job table upload") != 0)
         return nullptr;
-    return s.table_device;
+    return slot;
+}
+
+void table_release(State::TableSlot *slot, hipStream_t stream) {
+    if (slot && hip_ok(hipEventRecord(slot->done, stream), "job table event") == 0) slot->busy = 1;
 }
 
 }  // namespace mi355
@@ -151,7 +156,10 @@ int salt_mi355_shutdown(void) {
     State &s = g_state;
     if (!s.ready) return 0;
     int failed = hip_ok(hipDeviceSynchronize(), "hipDeviceSynchronize at shutdown");
-    if (s.table_device) { (void)hipFree(s.table_device); (void)hipHostFree(s.table_pinned); }
+    for (State::TableSlot &slot : s.tables) {
+        if (slot.device) { (void)hipFree(slot.device); (void)hipHostFree(slot.pinned); }
+        if (slot.done) (void)hipEventDestroy(slot.done);
+    }
     if (s.stream) failed |= hip_ok(hipStreamDestroy(s.stream), "hipStreamDestroy");
     char keep[sizeof s.last_error];
     memcpy(keep, s.last_error, sizeof keep);
@@ -240,13 +248,16 @@ int salt_mi355_q4_jobs_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tok
         launch.cols = C;
         launch.tokens = group;
         launch.code_scale = s.code_scale;
+        State::TableSlot *slot = nullptr;
         if (njobs == 1) {
             launch.one = table[0];
         } else {
-            launch.table = (const Q4Job *)stage_table(table.data(), table.size() * sizeof(Q4Job), stream);
-            if (!launch.table) return -1;
+            slot = table_acquire(table.data(), table.size() * sizeof(Q4Job), stream);
+            if (!slot) return -1;
+            launch.table = (const Q4Job *)slot->device;
         }
         const int rc = tileable ? q4_launch(launch, chains, stream) : q4_launch_generic(launch, stream);
+        table_release(slot, stream);
         if (rc != 0) { set_error("q4: kernel launch failed: %s", hipGetErrorString(hipGetLastError())); return -1; }
     }
     return 0;

@@ -18,16 +18,27 @@ struct State {
     float fp8_table[256] = {0};
     float fp4_table[512] = {0};
     char last_error[256] = {0};
-    // device + pinned copies of the most recent multi-job table
-    void *table_device = nullptr;
-    void *table_pinned = nullptr;
-    size_t table_capacity = 0;
+    // Ring of device + pinned copies of multi-job tables.  A slot is reused
+    // only after the event recorded behind its last consumer has completed.
+    struct TableSlot {
+        void *device = nullptr;
+        void *pinned = nullptr;
+        size_t capacity = 0;
+        hipEvent_t done = nullptr;
+        int busy = 0;
+    };
+    static constexpr int kTableSlots = 8;
+    TableSlot tables[kTableSlots];
+    int next_table = 0;
 };
 
 extern State g_state;
 
 void set_error(const char *format, ...) __attribute__((format(printf, 1, 2)));
 int hip_ok(hipError_t status, const char *what);
-void *stage_table(const void *host_table, size_t nbytes, hipStream_t stream);
+// Copies a host job table to the device on `stream`; after the consuming
+// launch has been enqueued the caller hands the slot back with table_release.
+State::TableSlot *table_acquire(const void *host_table, size_t nbytes, hipStream_t stream);
+void table_release(State::TableSlot *slot, hipStream_t stream);
 
 }  // namespace mi355

@@ -471,10 +471,9 @@ int q4_launch(const Q4Launch &L, int chains_per_lane, hipStream_t stream) {
     if (L.total_tiles < 1 || L.tokens < 1 || L.tokens > 4 || L.cols < 64 || (L.cols & 63)) return -1;
     int S = chains_per_lane ? chains_per_lane : env_chains();
     if (S == 0) {
-        // enough waves to give every SIMD of the 256 CUs at least two
-        if (L.total_tiles * 4 >= 2048) S = 8;
-        else if (L.total_tiles * 8 >= 2048) S = 4;
-        else S = 2;
+        // Four chains per lane (eight waves per tile) measured fastest whenever
+        // there are enough tiles to spread; fewer tiles take sixteen waves each.
+        S = L.total_tiles >= 128 ? 4 : 2;
     }
     if (L.fused) {
         switch (S) {

@@ -18,6 +18,19 @@ class Q4Job(C.Structure):
 
 _lib = None
 
+INCLUDE_DIR = Path(__file__).resolve().parent.parent / "include"
+
+
+def declared_symbols() -> list[str]:
+    """Every function name the public headers declare."""
+    import re
+    names = []
+    for header in sorted(INCLUDE_DIR.glob("*.h")):
+        text = re.sub(r"/\*.*?\*/", " ", header.read_text(), flags=re.S)
+        names += re.findall(r"\b(salt_(?:gpu|mi355)_[a-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
 
 def _sig(fn, restype, *argtypes):
     fn.restype = restype
