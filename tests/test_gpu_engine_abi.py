@@ -1,0 +1,440 @@
+"""The engine-facing entry points (salt_gpu_*) driven the way the engine drives
+its physical backend: host pointers in and out, weights named inside described
+resources, expert seats filled through the residency operations.  Outputs are
+compared bit-for-bit with the CPU checker."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import engine_abi as abi
+from golden import cases
+from oracle_lib import ExpertGeometry, bits, host_threads, ptr
+
+pytestmark = pytest.mark.gpu
+synth = cases.synth
+TRUNK, EXPERT_LAYER = 1, 2
+
+
+@pytest.fixture(scope="module")
+def eng(pkg):
+    lib = abi.bind(pkg.lib.load())
+    assert lib.salt_gpu_init() == 0 and lib.salt_gpu_init() == 0      # idempotent
+    yield lib
+    assert lib.salt_gpu_sync() == 0
+
+
+def err(pkg):
+    return pkg.lib.load().salt_mi355_last_error().decode()
+
+
+def q4_want(oracle, vals, scales, biases, R, Cc, xs):
+    xs = xs.reshape(-1, Cc)
+    ys = np.zeros((xs.shape[0], R), np.float32)
+    for t in range(xs.shape[0]):
+        assert oracle.orc_q4_matvec_threads(ptr(vals), ptr(scales), ptr(biases), R, Cc, ptr(np.ascontiguousarray(xs[t])),
+                                            ptr(ys[t]), host_threads()) == 0
+    return ys
+
+
+class Trunk:
+    """Several Q4 tensors laid out back to back in one host byte range, the way
+    a model file maps them."""
+
+    def __init__(self, shapes, seed):
+        parts, self.views = [], []
+        at = 0
+        for k, (R, Cc) in enumerate(shapes):
+            vals, scales, biases = synth.q4_tensor(R, Cc, seed + k)
+            offs = []
+            for a in (vals, scales, biases):
+                offs.append(at); parts.append(a.view(np.uint8)); at += a.nbytes
+                pad = (-at) % 16
+                parts.append(np.zeros(pad, np.uint8)); at += pad
+            self.views.append((R, Cc, offs, vals, scales, biases))
+        self.blob = np.concatenate(parts)
+        self.base = self.blob.ctypes.data
+
+    def pointers(self, k):
+        R, Cc, offs, *_ = self.views[k]
+        return self.base + offs[0], self.base + offs[1], self.base + offs[2]
+
+
+def test_resource_lifecycle_matvec_batch_and_stats(eng, oracle, pkg):
+    trunk = Trunk([(704, 2816), (2816, 704), (130, 2816)], 11)
+    assert eng.salt_gpu_weight_resource_describe(TRUNK, 7, trunk.base, trunk.blob.nbytes) == 0
+    assert eng.salt_gpu_weight_resource_describe(TRUNK, 7, trunk.base, trunk.blob.nbytes) == 0       # same again is fine
+    assert eng.salt_gpu_weight_resource_describe(TRUNK, 7, trunk.base, trunk.blob.nbytes - 1) == -1  # conflicting
+    assert eng.salt_gpu_weight_resource_activate(TRUNK, 7, 3) == -1                                  # pageable refused
+    assert eng.salt_gpu_weight_resource_activate(TRUNK, 7, 2) == 0, err(pkg)
+    usage = abi.ResourceUsage()
+    assert eng.salt_gpu_weight_resource_usage(C.byref(usage), C.sizeof(usage)) == 0
+    assert usage.described_resources == 1 and usage.active_resources == 1
+    assert usage.device_copied_weight_bytes == trunk.blob.nbytes == usage.registered_bytes
+    keys = [0x1000 + k for k in range(3)]
+    for k in range(3):
+        R, Cc, *_ = trunk.views[k]
+        v, s, b = trunk.pointers(k)
+        assert eng.salt_gpu_weight_resource_slot(TRUNK, 7, keys[k], v, s, b, 4, R, Cc) == 0, err(pkg)
+        assert eng.salt_gpu_weight_resource_slot(TRUNK, 7, keys[k], v, s, b, 4, R, Cc) == 0          # identical re-registration
+    v0, s0, b0 = trunk.pointers(0)
+    assert eng.salt_gpu_weight_resource_slot(TRUNK, 7, keys[0], v0 + 16, s0, b0, 4, 704, 2816) == -1  # conflicting key
+    assert eng.salt_gpu_weight_resource_slot(TRUNK, 7, 0x2000, v0, s0, b0, 8, 704, 2816) == -1        # q8 is off-path
+    assert eng.salt_gpu_weight_resource_slot(TRUNK, 9, 0x2000, v0, s0, b0, 4, 704, 2816) == -1        # unknown resource
+    assert eng.salt_gpu_weight_resource_slot(TRUNK, 7, 0x2000, v0, s0, b0, 4, 70400, 2816) == -1      # outside the range
+
+    eng.salt_gpu_set_mapped_only(1)
+    before = abi.BatchStats(); eng.salt_gpu_batch_stats_get(C.byref(before))
+    # one matvec by pointers that lie inside the active resource
+    R, Cc, _, vals, scales, biases = trunk.views[0]
+    x = synth.activations(Cc, 1, 5)[0]; y = np.full(R, np.nan, np.float32)
+    assert eng.salt_gpu_q4_matvec(v0, s0, b0, R, Cc, ptr(x), ptr(y)) == 0, err(pkg)
+    assert np.array_equal(bits(y), bits(q4_want(oracle, vals, scales, biases, R, Cc, x)[0]))
+    # batch: two tensors sharing C = 2816, distinct inputs
+    xs = synth.activations(2816, 2, 6)
+    y0 = np.zeros(704, np.float32); y2 = np.zeros(130, np.float32)
+    v2, s2, b2 = trunk.pointers(2)
+    rc = eng.salt_gpu_q4_batch(abi.ptr_array([v0, v2]), abi.ptr_array([s0, s2]), abi.ptr_array([b0, b2]),
+                               abi.ptr_array([xs[0], xs[1]]), abi.ptr_array([y0, y2]), abi.ptr_array(keys[0:3:2]),
+                               (C.c_int * 2)(704, 130), 2816, 2)
+    assert rc == 0, err(pkg)
+    assert np.array_equal(bits(y0), bits(q4_want(oracle, *trunk.views[0][3:], 704, 2816, xs[0])[0]))
+    assert np.array_equal(bits(y2), bits(q4_want(oracle, *trunk.views[2][3:], 130, 2816, xs[1])[0]))
+    # a key that does not match the pointers it travels with is refused
+    assert eng.salt_gpu_q4_batch(abi.ptr_array([v0]), abi.ptr_array([s0]), abi.ptr_array([b0]), abi.ptr_array([xs[0]]),
+                                 abi.ptr_array([y0]), abi.ptr_array([keys[2]]), (C.c_int * 1)(704), 2816, 1) == -1
+    # projection adapter: B = 6 contiguous tokens through the down-shaped tensor
+    R, Cc, _, vals, scales, biases = trunk.views[1]
+    v1, s1, b1 = trunk.pointers(1)
+    xb = synth.activations(Cc, 6, 8); yb = np.zeros((6, R), np.float32)
+    rc = eng.salt_gpu_proj_batch(v1, s1, b1, R, Cc, 6, abi.ptr_array([xb[t] for t in range(6)]),
+                                 abi.ptr_array([yb[t] for t in range(6)]), keys[1])
+    assert rc == 0, err(pkg)
+    assert np.array_equal(bits(yb), bits(q4_want(oracle, vals, scales, biases, R, Cc, xb)))
+    scattered = [xb[t] for t in (0, 2, 1, 3, 4, 5)]
+    assert eng.salt_gpu_proj_batch(v1, s1, b1, R, Cc, 6, abi.ptr_array(scattered),
+                                   abi.ptr_array([yb[t] for t in range(6)]), keys[1]) == -1
+    after = abi.BatchStats(); eng.salt_gpu_batch_stats_get(C.byref(after))
+    assert after.trunk_batches == before.trunk_batches + 3 and after.arena_batches == before.arena_batches
+
+    # weights outside any resource: refused under mapped-only (and counted), copied per call otherwise
+    lv, ls, lb = synth.q4_tensor(64, 128, 3)
+    lx = synth.activations(128, 1, 4)[0]; ly = np.zeros(64, np.float32)
+    assert eng.salt_gpu_q4_matvec(ptr(lv), ptr(ls), ptr(lb), 64, 128, ptr(lx), ptr(ly)) == -1
+    miss = abi.BatchStats(); eng.salt_gpu_batch_stats_get(C.byref(miss))
+    assert miss.mapped_only_misses == after.mapped_only_misses + 1
+    eng.salt_gpu_set_mapped_only(0)
+    assert eng.salt_gpu_q4_matvec(ptr(lv), ptr(ls), ptr(lb), 64, 128, ptr(lx), ptr(ly)) == 0, err(pkg)
+    assert np.array_equal(bits(ly), bits(q4_want(oracle, lv, ls, lb, 64, 128, lx)[0]))
+    assert eng.salt_gpu_q4_matvec(ptr(lv), ptr(ls), None, 64, 128, ptr(lx), ptr(ly)) == 0          # NULL biases
+    assert np.array_equal(bits(ly), bits(q4_want(oracle, lv, ls, None, 64, 128, lx)[0]))
+    legacy = abi.BatchStats(); eng.salt_gpu_batch_stats_get(C.byref(legacy))
+    assert legacy.arena_batches == miss.arena_batches + 2
+
+    # deferred publication: outputs appear at salt_gpu_sync()
+    assert eng.salt_gpu_set_defer(1) == 0 and eng.salt_gpu_defer() == 1
+    R, Cc, _, vals, scales, biases = trunk.views[0]
+    y = np.full(R, 7.0, np.float32)
+    assert eng.salt_gpu_q4_matvec(v0, s0, b0, R, Cc, ptr(x), ptr(y)) == 0
+    assert (y == 7.0).all()
+    assert eng.salt_gpu_set_defer(0) == 0 and eng.salt_gpu_defer() == 0
+    assert np.array_equal(bits(y), bits(q4_want(oracle, vals, scales, biases, R, Cc, x)[0]))
+
+    assert eng.salt_gpu_weight_resource_deactivate(TRUNK, 7) == 0
+    eng.salt_gpu_set_mapped_only(1)
+    assert eng.salt_gpu_q4_matvec(v0, s0, b0, R, Cc, ptr(x), ptr(y)) == -1       # no longer resident
+    eng.salt_gpu_set_mapped_only(0)
+    assert eng.salt_gpu_weight_resource_unbind(TRUNK, 7) == 0
+    assert eng.salt_gpu_weight_resource_usage(C.byref(usage), C.sizeof(usage)) == 0
+    assert usage.described_resources == 0 and usage.device_copied_weight_bytes == 0
+
+
+def test_bounded_window_and_expert_layer_resource(eng, oracle, pkg):
+    trunk = Trunk([(128, 256), (64, 256)], 21)
+    assert eng.salt_gpu_weight_resource_describe(TRUNK, 3, trunk.base, trunk.blob.nbytes) == 0
+    assert eng.salt_gpu_weight_resource_activate(TRUNK, 3, 1) == 0
+    eng.salt_gpu_set_mapped_only(1)
+    R, Cc, offs, vals, scales, biases = trunk.views[1]
+    v, s, b = trunk.pointers(1)
+    x = synth.activations(Cc, 1, 2)[0]; y = np.zeros(R, np.float32)
+    assert eng.salt_gpu_q4_matvec(v, s, b, R, Cc, ptr(x), ptr(y)) == -1          # no window bound yet
+    assert eng.salt_gpu_weight_window_bind(TRUNK, 3, offs[0], trunk.blob.nbytes - offs[0]) == 0, err(pkg)
+    assert eng.salt_gpu_weight_window_bind(TRUNK, 3, 0, 64) == -1                # one window at a time
+    assert eng.salt_gpu_q4_matvec(v, s, b, R, Cc, ptr(x), ptr(y)) == 0, err(pkg)
+    assert np.array_equal(bits(y), bits(q4_want(oracle, vals, scales, biases, R, Cc, x)[0]))
+    usage = abi.ResourceUsage()
+    assert eng.salt_gpu_weight_resource_usage(C.byref(usage), C.sizeof(usage)) == 0
+    assert usage.active_windows == 1 and usage.active_window_bytes == trunk.blob.nbytes - offs[0]
+    assert eng.salt_gpu_weight_window_unbind(TRUNK, 3) == 0
+    assert eng.salt_gpu_q4_matvec(v, s, b, R, Cc, ptr(x), ptr(y)) == -1
+    assert eng.salt_gpu_weight_resource_unbind(TRUNK, 3) == 0
+    # command-scoped expert layer (reference src/gpu_layer.c:17-81): bind, slot, run, unbind
+    layer = Trunk([(64, 128)], 31)
+    assert eng.salt_gpu_expert_resource_bind(55, layer.base, layer.blob.nbytes) == 0
+    v, s, b = layer.pointers(0)
+    assert eng.salt_gpu_expert_resource_slot(55, 0xABC, v, s, b, 64, 128) == 0
+    assert eng.salt_gpu_resident_slot(0xABD, v, s, b, 64, 128) == 0
+    x = synth.activations(128, 1, 3)[0]; y = np.zeros(64, np.float32)
+    before = abi.BatchStats(); eng.salt_gpu_batch_stats_get(C.byref(before))
+    assert eng.salt_gpu_q4_matvec(v, s, b, 64, 128, ptr(x), ptr(y)) == 0
+    after = abi.BatchStats(); eng.salt_gpu_batch_stats_get(C.byref(after))
+    assert after.expert_layer_batches == before.expert_layer_batches + 1
+    assert np.array_equal(bits(y), bits(q4_want(oracle, *layer.views[0][3:], 64, 128, x)[0]))
+    assert eng.salt_gpu_expert_resource_unbind(55) == 0
+    assert eng.salt_gpu_q4_matvec(v, s, b, 64, 128, ptr(x), ptr(y)) == -1
+    eng.salt_gpu_set_mapped_only(0)
+
+
+def expert_record(pool, e, H, F, group, slot=-1, logical=0):
+    base = pool.ctypes.data + e * synth.expert_slot_bytes(H, F)
+    proj = synth.expert_proj_bytes(H, F)
+    n = H * F
+    rec = abi.MoeExpert()
+    for p, name in enumerate(("gate", "up", "down")):
+        at = base + p * proj
+        setattr(rec, name + "_vals", at)
+        setattr(rec, name + "_scales", at + n // 2)
+        setattr(rec, name + "_biases", at + n // 2 + (n // 64) * 2)
+        setattr(rec, name + "_id", at)
+    rec.group, rec.resource_slot, rec.logical_resource_id = group, slot, logical
+    return rec
+
+
+def chain_want(oracle, pool, H, F, experts, groups, inputs):
+    g = ExpertGeometry(H, F)
+    slot = synth.expert_slot_bytes(H, F)
+    out = np.zeros_like(inputs)
+    row = 0
+    for e, n in zip(experts, groups):
+        for _ in range(n):
+            gate = np.zeros(F, np.float32); up = np.zeros(F, np.float32)
+            assert oracle.orc_expert_ffn(C.byref(g), ptr(pool[e * slot:]), ptr(inputs[row]), ptr(gate), ptr(up),
+                                         ptr(out[row])) == 0
+            row += 1
+    return out
+
+
+def test_moe_chain_from_a_layer_resource(eng, oracle, pkg):
+    E, H, F = 6, 256, 128
+    pool = synth.expert_pool(E, H, F, 41)
+    assert eng.salt_gpu_expert_resource_bind(9, pool.ctypes.data, pool.nbytes) == 0, err(pkg)
+    experts, groups = [1, 3, 4], [2, 5, 1]              # prefill-shaped: several rows per expert
+    recs = (abi.MoeExpert * 3)(*[expert_record(pool, e, H, F, n) for e, n in zip(experts, groups)])
+    rows = sum(groups)
+    inputs = synth.activations(H, rows, 42); outputs = np.zeros((rows, H), np.float32)
+    scratch = np.zeros((2, rows * F), np.float32)
+    eng.salt_gpu_set_mapped_only(1)
+    rc = eng.salt_gpu_q4_moe_chain(recs, 3, H, F, ptr(inputs), ptr(outputs), ptr(scratch[0]), ptr(scratch[1]), rows * F)
+    assert rc == 0, err(pkg)
+    assert np.array_equal(bits(outputs), bits(chain_want(oracle, pool, H, F, experts, groups, inputs)))
+    # rejected: too little scratch, zero-row expert, not resident
+    assert eng.salt_gpu_q4_moe_chain(recs, 3, H, F, ptr(inputs), ptr(outputs), ptr(scratch[0]), ptr(scratch[1]), rows * F - 1) == -1
+    recs[1].group = 0
+    assert eng.salt_gpu_q4_moe_chain(recs, 3, H, F, ptr(inputs), ptr(outputs), ptr(scratch[0]), ptr(scratch[1]), rows * F) == -1
+    recs[1].group = 5
+    assert eng.salt_gpu_expert_resource_unbind(9) == 0
+    assert eng.salt_gpu_q4_moe_chain(recs, 3, H, F, ptr(inputs), ptr(outputs), ptr(scratch[0]), ptr(scratch[1]), rows * F) == -1
+    eng.salt_gpu_set_mapped_only(0)
+
+
+def shared_array(eng, nfloats):
+    buf = abi.SharedBuffer()
+    assert eng.salt_gpu_shared_buffer_alloc(C.byref(buf), nfloats * 4) == 0
+    assert buf.contents and buf.backend and buf.nbytes == nfloats * 4
+    arr = np.ctypeslib.as_array(C.cast(buf.contents, C.POINTER(C.c_float)), shape=(nfloats,))
+    return buf, arr
+
+
+def test_expert_seats_through_residency_and_selected_chain(eng, oracle, pkg):
+    E, H, F, K = 8, 256, 128, 3
+    pool = synth.expert_pool(E, H, F, 51)
+    slot_bytes = synth.expert_slot_bytes(H, F)
+    ops = eng.salt_gpu_residency_backend_ops().contents
+    seats, staging_count = 4, 2
+    plan = abi.ResidencyPlan(4096 + seats * slot_bytes, 0, 4096, slot_bytes, slot_bytes, seats, staging_count, 256, 0)
+    assert ops.create(None, C.byref(plan)) == 0, err(pkg)
+    assert ops.create(None, C.byref(plan)) == -1                      # one arena at a time
+    assert eng.salt_gpu_free() == -1                                  # refused while residency is live
+    layout = abi.PermanentLayout()
+    assert ops.permanent_layout(None, C.byref(layout), C.sizeof(layout)) == 0 and layout.span_count == 0
+    assert eng.salt_gpu_selected_resources_prepare(seats, 30 * 128) == 0
+    assert eng.salt_gpu_selected_resources_prepare(seats, 30 * 128) == 0
+    assert eng.salt_gpu_selected_resources_prepare(seats + 1, 30 * 128) == -1
+
+    chosen = [5, 0, 6]                       # experts placed in seats 0, 1, 2
+    layer = 2
+    addresses = []
+    for seat, e in enumerate(chosen):
+        staging, cap = C.c_void_p(), C.c_size_t()
+        st_slot = seat % staging_count
+        assert ops.staging(None, st_slot, C.byref(staging), C.byref(cap)) == 0 and cap.value >= slot_bytes
+        C.memmove(staging.value, pool.ctypes.data + e * slot_bytes, slot_bytes)   # the engine's read callback
+        offset = plan.slot_base_offset + seat * slot_bytes
+        ticket = 100 + seat
+        assert ops.populate(None, seat, offset + 1, st_slot, slot_bytes, ticket) == -1      # wrong offset
+        assert ops.populate(None, seat, offset, st_slot, slot_bytes, 0) == -1               # ticket 0
+        assert ops.populate(None, seat, offset, st_slot, slot_bytes, ticket) == 0, err(pkg)
+        assert ops.populate(None, seat, offset, st_slot, slot_bytes, ticket + 50) == -1     # seat busy
+        done = C.c_int(0)
+        assert ops.poll(None, seat, ticket + 1, C.byref(done)) == -1                        # stale ticket
+        for _ in range(100000):
+            assert ops.poll(None, seat, ticket, C.byref(done)) == 0
+            if done.value:
+                break
+        assert done.value == 1
+        assert ops.poll(None, seat, ticket, C.byref(done)) == -1                            # already published
+        addr = C.c_size_t()
+        assert ops.resolve(None, offset, slot_bytes, C.byref(addr)) == 0 and addr.value
+        assert ops.resolve(None, plan.device_budget_bytes, 1, C.byref(addr)) == -1
+        assert ops.resolve(None, offset, slot_bytes, C.byref(addr)) == 0
+        addresses.append(addr.value)
+        logical = layer * 128 + e
+        payload = pool.ctypes.data + e * slot_bytes
+        assert eng.salt_gpu_selected_resource_bind_resident(seat, logical, payload, slot_bytes, 12345, 1) == -1
+        assert eng.salt_gpu_selected_resource_bind_resident(seat, logical, payload, slot_bytes, addr.value, 1) == 0, err(pkg)
+        assert eng.salt_gpu_selected_resource_bind_resident(seat, logical, payload, slot_bytes, addr.value, 1) == 0
+        assert eng.salt_gpu_selected_resource_bind_resident(seat, logical + 1, payload, slot_bytes, addr.value, 1) == -1
+
+    # decode-shaped selected chain: one row per expert, ascending expert order, all four buffers shared
+    order = sorted(range(K), key=lambda i: chosen[i])
+    recs = (abi.MoeExpert * K)(*[expert_record(pool, chosen[i], H, F, 1, slot=i, logical=layer * 128 + chosen[i])
+                                 for i in order])
+    bin_, ain = shared_array(eng, K * H); bout, aout = shared_array(eng, K * H)
+    bg, _ = shared_array(eng, K * F); bu, _ = shared_array(eng, K * F)
+    x = synth.activations(H, 1, 52)[0]
+    ain[:] = np.tile(x, K)
+    eng.salt_gpu_set_mapped_only(1)
+    rc = eng.salt_gpu_q4_moe_chain_selected(recs, K, H, F, bin_.contents, bout.contents, bg.contents, bu.contents, K * F)
+    assert rc == 0, err(pkg)
+    want = chain_want(oracle, pool, H, F, [chosen[i] for i in order], [1] * K, np.tile(x, (K, 1)))
+    assert np.array_equal(bits(aout.reshape(K, H)), bits(want))
+    # plain host memory instead of shared buffers is refused
+    plain = np.zeros(K * H, np.float32)
+    assert eng.salt_gpu_q4_moe_chain_selected(recs, K, H, F, ptr(plain), bout.contents, bg.contents, bu.contents, K * F) == -1
+    # a seat that holds another expert is refused
+    recs[0].logical_resource_id += 1
+    assert eng.salt_gpu_q4_moe_chain_selected(recs, K, H, F, bin_.contents, bout.contents, bg.contents, bu.contents, K * F) == -1
+    recs[0].logical_resource_id -= 1
+
+    # heterogeneous projections inside one shared arena (reference gpu.h:311-316)
+    arena, aa = shared_array(eng, 4 * H + 4 * F)
+    aa[:H] = x; aa[H:2 * H] = x * 2
+    jobs = (abi.SelectedJob * 2)()
+    for j, i in enumerate(order[:2]):
+        r = recs[j]
+        jobs[j] = abi.SelectedJob(r.gate_vals, r.gate_scales, r.gate_biases, r.gate_id, arena.contents + j * H * 4,
+                                  arena.contents + (2 * H + j * F) * 4, F, H, 1, r.resource_slot, r.logical_resource_id)
+    assert eng.salt_gpu_q4_selected_shared(jobs, 2, C.byref(arena)) == 0, err(pkg)
+    for j, i in enumerate(order[:2]):
+        gv = synth.expert_views(pool, chosen[i], 0, H, F)
+        assert np.array_equal(bits(aa[2 * H + j * F:2 * H + (j + 1) * F]),
+                              bits(q4_want(oracle, gv[0], gv[1], gv[2], F, H, aa[j * H:(j + 1) * H].copy())[0]))
+    jobs[1].outputs = jobs[0].outputs                                  # overlapping outputs
+    assert eng.salt_gpu_q4_selected_shared(jobs, 2, C.byref(arena)) == -1
+
+    # asynchronous indexed projection straight into a shared buffer, published by sync
+    gv = synth.expert_views(pool, chosen[0], 0, H, F)
+    r0 = expert_record(pool, chosen[0], H, F, 1)
+    xb = synth.activations(H, 5, 53)
+    dest, adest = shared_array(eng, 16 + 5 * F)
+    adest[:] = -1.0
+    assert eng.salt_gpu_proj_batch_indexed(r0.gate_vals, r0.gate_scales, r0.gate_biases, F, H, 5, 1, 3, ptr(xb),
+                                           C.byref(dest), 16, r0.gate_id) == 0, err(pkg)
+    assert eng.salt_gpu_sync() == 0
+    want = q4_want(oracle, gv[0], gv[1], gv[2], F, H, xb)
+    got = adest[16:].reshape(5, F)
+    assert np.array_equal(bits(got[1:4]), bits(want[1:4])) and (got[0] == -1).all() and (got[4] == -1).all()
+    assert eng.salt_gpu_proj_batch_indexed(r0.gate_vals, r0.gate_scales, r0.gate_biases, F, H, 5, 4, 3, ptr(xb),
+                                           C.byref(dest), 16, r0.gate_id) == -1
+    stats = abi.BatchStats(); eng.salt_gpu_batch_stats_get(C.byref(stats))
+    assert stats.direct_output_batches >= 1 and stats.direct_output_jobs >= 3
+    eng.salt_gpu_set_mapped_only(0)
+
+    # eviction: fence, unbind, retire, then the seat can be populated again
+    assert eng.salt_gpu_selected_resources_fence() == 0
+    for seat, e in enumerate(chosen):
+        assert eng.salt_gpu_selected_resource_unbind(seat, layer * 128 + e + 1) == -1
+        assert eng.salt_gpu_selected_resource_unbind(seat, layer * 128 + e) == 0
+        assert eng.salt_gpu_selected_resource_unbind(seat, layer * 128 + e) == 0      # inactive seat: fine
+        assert ops.retire(None, seat, 1) == 0
+    # plain (non-resident) bind copies the payload itself
+    payload = pool.ctypes.data + 2 * slot_bytes
+    assert eng.salt_gpu_selected_resource_bind(3, 77, pool.ctypes.data, pool.nbytes, payload) == 0, err(pkg)
+    assert eng.salt_gpu_selected_resource_bind(3, 77, pool.ctypes.data, pool.nbytes, payload) == 0
+    assert eng.salt_gpu_selected_resource_bind(3, 78, pool.ctypes.data, pool.nbytes, payload) == -1
+    rec = (abi.MoeExpert * 1)(expert_record(pool, 2, H, F, 1, slot=3, logical=77))
+    ain[:H] = x
+    assert eng.salt_gpu_q4_moe_chain_selected(rec, 1, H, F, bin_.contents, bout.contents, bg.contents, bu.contents, F) == 0, err(pkg)
+    assert np.array_equal(bits(aout[:H]), bits(chain_want(oracle, pool, H, F, [2], [1], x[None, :])[0]))
+    assert eng.salt_gpu_selected_resource_unbind(3, 77) == 0
+    for b in (bin_, bout, bg, bu, arena, dest):
+        assert eng.salt_gpu_shared_buffer_free(C.byref(b)) == 0 and not b.contents
+    assert ops.destroy(None) == 0
+    assert ops.destroy(None) == -1
+
+
+def test_nvfp4_engine_entry_points(eng, oracle, pkg):
+    R, Cc = 96, 2816
+    packed, scales = synth.nvfp4_tensor(R, Cc, 61)
+    globals_ = np.array([2688.0, 64.0], np.float32)          # stored divisor, input global scale
+    blob = np.concatenate([packed, scales, globals_.view(np.uint8)])
+    base = blob.ctypes.data
+    assert eng.salt_gpu_weight_resource_bind(TRUNK, 12, base, blob.nbytes) == 0, err(pkg)
+    key = 0x7777
+    wg, ig = base + packed.nbytes + scales.nbytes, base + packed.nbytes + scales.nbytes + 4
+    assert eng.salt_gpu_nvfp4_resource_slot(TRUNK, 12, key, base, base + packed.nbytes, wg, ig, R, Cc) == 0, err(pkg)
+    assert eng.salt_gpu_nvfp4_resource_slot(TRUNK, 12, key, base, base + packed.nbytes, wg, ig, R, Cc + 32) == -1
+
+    def want(xs):
+        out = np.zeros((xs.shape[0], R), np.float32)
+        for t in range(xs.shape[0]):
+            s = (np.zeros(Cc // 2, np.uint8), np.zeros(Cc // 16, np.uint8), np.zeros(Cc, np.float32))
+            assert oracle.orc_nvfp4_matvec(ptr(packed), ptr(scales), 2688.0, 64.0, R, Cc, ptr(xs[t]), ptr(out[t]),
+                                           ptr(s[0]), ptr(s[1]), ptr(s[2])) == 0
+        return out
+
+    xs = synth.activations(Cc, 5, 62)
+    y = np.zeros(R, np.float32)
+    assert eng.salt_gpu_nvfp4_matvec(key, R, Cc, ptr(xs[0]), ptr(y)) == 0, err(pkg)
+    assert np.array_equal(bits(y), bits(want(xs[:1])[0]))
+    yb = np.zeros((5, R), np.float32)
+    assert eng.salt_gpu_nvfp4_matvec_batch(key, R, Cc, 5, ptr(xs), ptr(yb)) == 0, err(pkg)
+    assert np.array_equal(bits(yb), bits(want(xs)))
+    y1 = np.zeros((2, R), np.float32); y2 = np.zeros((1, R), np.float32)
+    rc = eng.salt_gpu_nvfp4_batch(abi.ptr_array([key, key]), abi.ptr_array([xs[0:2], xs[4:5]]),
+                                  abi.ptr_array([y1, y2]), (C.c_int * 2)(2, 1), R, Cc, 2)
+    assert rc == 0, err(pkg)
+    assert np.array_equal(bits(y1), bits(want(xs[0:2]))) and np.array_equal(bits(y2), bits(want(xs[4:5])))
+    assert eng.salt_gpu_nvfp4_matvec(0x9999, R, Cc, ptr(xs[0]), ptr(y)) == -1            # unknown key
+    assert eng.salt_gpu_nvfp4_matvec(key, R + 1, Cc, ptr(xs[0]), ptr(y)) == -1           # geometry mismatch
+    bad = xs[0].copy(); bad[17] = np.inf
+    y[:] = 3.0
+    assert eng.salt_gpu_nvfp4_matvec(key, R, Cc, ptr(bad), ptr(y)) == -1 and (y == 3.0).all()
+    stats = abi.BatchStatsV2()
+    assert eng.salt_gpu_batch_stats_get_v2(C.byref(stats), C.sizeof(stats)) == 0
+    assert stats.nvfp4_logical_packed_weight_bytes >= 3 * R * Cc // 2 and stats.nvfp4_completion_fences >= 3
+    # stand-alone activation Q/DQ
+    p = np.zeros(Cc // 2, np.uint8); s = np.zeros(Cc // 16, np.uint8); d = np.zeros(Cc, np.float32)
+    assert eng.salt_gpu_nvfp4_qdq(ptr(xs[1]), Cc, 64.0, ptr(p), ptr(s), ptr(d)) == 0, err(pkg)
+    op = np.zeros_like(p); os_ = np.zeros_like(s); od = np.zeros_like(d)
+    assert oracle.orc_nvfp4_qdq(ptr(xs[1]), Cc, 64.0, ptr(op), ptr(os_), ptr(od)) == 0
+    assert np.array_equal(p, op) and np.array_equal(s, os_) and np.array_equal(bits(d), bits(od))
+    assert eng.salt_gpu_nvfp4_qdq(ptr(bad), Cc, 64.0, ptr(p), ptr(s), ptr(d)) == -1
+    assert eng.salt_gpu_nvfp4_qdq(ptr(xs[1]), Cc, -1.0, ptr(p), ptr(s), ptr(d)) == -1
+    assert eng.salt_gpu_weight_resource_unbind(TRUNK, 12) == 0
+    assert eng.salt_gpu_nvfp4_matvec(key, R, Cc, ptr(xs[0]), ptr(y)) == -1
+
+
+def test_off_path_entry_points_answer_like_the_null_backend(eng):
+    z = np.zeros(64, np.float32)
+    assert eng.salt_gpu_q8_matvec(ptr(z), ptr(z), ptr(z), 1, 64, ptr(z), ptr(z)) == -1
+    assert eng.salt_gpu_bf16_matvec(1, 1, 64, ptr(z), ptr(z)) == -1
+    assert eng.salt_gpu_resident_trunk_map(ptr(z), 256) == -1 and eng.salt_gpu_resident_pool_map(ptr(z), 256) == -1
+    assert eng.salt_dispatch_get() is None and eng.salt_gpu_tensor_program_ops() is None
+
+
+def test_zz_free_and_reinit(eng, pkg):
+    assert eng.salt_gpu_free() == 0
+    z = np.zeros(64, np.float32)
+    assert eng.salt_gpu_q4_matvec(ptr(z), ptr(z), None, 1, 64, ptr(z), ptr(z)) == -1     # fails loudly when not initialised
+    assert eng.salt_gpu_init() == 0
