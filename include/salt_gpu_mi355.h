@@ -90,6 +90,13 @@ typedef struct SaltMi355Q4Job {
 } SaltMi355Q4Job;
 int salt_mi355_q4_jobs_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tokens,
                            int chains_per_lane, void *stream);
+/* Accumulation mode of the tiled Q4 kernel for later launches; returns the
+ * previous mode.  0 (default): acc = fl(acc + fl(w * x)), bit-identical to the
+ * reference.  1: acc = fma(w, x, acc) in the same chain order, one rounding
+ * fewer per element: not bit-identical, within a few ulp of the sum of
+ * magnitudes.  The environment variable SALT_MI355_Q4_FUSED=1 selects mode 1
+ * at initialisation. */
+int salt_mi355_set_q4_accumulate(int fused);
 
 /* ---- NVFP4, device-resident ---------------------------------------------
  * Layout as the reference's nvfp4.h:37-46: packed E2M1 codes, low nibble =

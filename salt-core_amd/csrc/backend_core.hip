@@ -145,6 +145,8 @@ int salt_mi355_init(void) {
         s.stream = nullptr;
         return -1;
     }
+    const char *fused = getenv("SALT_MI355_Q4_FUSED");
+    s.q4_fused = fused && *fused == '1';
     s.ready = 1;
     if (getenv("SALT_GPU_DIAG"))
         fprintf(stderr, "salt-mi355: ready on %s, %d CUs, fp8 code scale %g\n", prop.gcnArchName,
@@ -169,6 +171,12 @@ int salt_mi355_shutdown(void) {
 }
 
 const char *salt_mi355_last_error(void) { return g_state.last_error; }
+
+int salt_mi355_set_q4_accumulate(int fused) {
+    const int before = g_state.q4_fused;
+    g_state.q4_fused = fused ? 1 : 0;
+    return before;
+}
 
 int salt_mi355_converter_tables(float *fp8, float *fp4) {
     if (!g_state.ready || !fp8 || !fp4) return -1;
@@ -248,6 +256,7 @@ int salt_mi355_q4_jobs_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tok
         launch.cols = C;
         launch.tokens = group;
         launch.code_scale = s.code_scale;
+        launch.fused = s.q4_fused;
         State::TableSlot *slot = nullptr;
         if (njobs == 1) {
             launch.one = table[0];

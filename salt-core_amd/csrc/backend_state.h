@@ -14,6 +14,7 @@ struct State {
     int compute_units = 0;
     hipStream_t stream = nullptr;
     float code_scale = 0.0f;            // 1 / fp8_table[1]
+    int q4_fused = 0;                   // 1: fma accumulate (tolerance class) instead of mul + add
     int fp8_is_ocp = 0;                 // the converter decodes every byte as OCP E4M3FN
     float fp8_table[256] = {0};
     float fp4_table[512] = {0};

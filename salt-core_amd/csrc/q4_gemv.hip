@@ -138,7 +138,7 @@ __device__ __forceinline__ void consume_word(uint32_t w, int first_block, int xb
 
 // How many 64-column groups of activations are fetched into SGPRs at once.
 constexpr int x_batch_groups(int S, int NB) {
-    const int fit = (S == 8 ? 32 : 64) / (2 * S * NB);     // SGPR budget for activations
+    const int fit = ((S == 8 || NB > 1) ? 32 : 64) / (2 * S * NB);     // SGPR budget for activations
     return fit >= 8 ? 8 : fit >= 4 ? 4 : fit >= 2 ? 2 : 1;
 }
 

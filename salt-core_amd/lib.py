@@ -64,6 +64,7 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_event_elapsed_ms, i, vp, vp, C.POINTER(f))
     _sig(lib.salt_mi355_q4_matvec_dev, i, vp, vp, vp, i, i, i, vp, vp, i, vp)
     _sig(lib.salt_mi355_q4_jobs_dev, i, C.POINTER(Q4Job), i, i, i, i, vp)
+    _sig(lib.salt_mi355_set_q4_accumulate, i, i)
     _sig(lib.salt_mi355_nvfp4_qdq_dev, i, vp, i, i, f, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_nvfp4_matvec_dev, i, vp, vp, f, i, i, i, vp, vp, i, vp)
     _sig(lib.salt_mi355_router_topk_dev, i, vp, vp, i, i, i, vp, vp, vp, vp)
