@@ -98,6 +98,17 @@ int salt_mi355_q4_jobs_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tok
  * at initialisation. */
 int salt_mi355_set_q4_accumulate(int fused);
 
+/* Prefill-sized variant on the matrix cores: ys[t*R + r] for B tokens against
+ * one matrix, fp32-accurate but NOT bit-identical to the reference (different
+ * summation order): |error| <= 2^-18 * sum_c |w*x| + 1e-6 per output.  Needs
+ * C % 64 == 0 and device scratch of salt_mi355_q4_matmul_workspace_bytes().
+ * The reference has no counterpart: its CPU and GPU paths keep the 32-chain
+ * order at every batch size (kernels.c:1252-1261). */
+size_t salt_mi355_q4_matmul_workspace_bytes(int C, int B);
+int salt_mi355_q4_matmul_dev(const void *vals, const void *scales, const void *biases,
+                             int R, int C, int B, const float *xs, float *ys,
+                             void *workspace, void *stream);
+
 /* ---- NVFP4, device-resident ---------------------------------------------
  * Layout as the reference's nvfp4.h:37-46: packed E2M1 codes, low nibble =
  * even element; E4M3FN scales [R][C/16]; one fp32 stored divisor per tensor

@@ -8,6 +8,39 @@ using namespace mi355;
 
 extern "C" {
 
+size_t salt_mi355_q4_matmul_workspace_bytes(int C, int B) {
+    if (C < 64 || (C & 63) || B < 1) return 0;
+    return 3 * (size_t)B * C * 2 + (((size_t)B * (C / 64) * 4 + 255) & ~(size_t)255) + 256;
+}
+
+int salt_mi355_q4_matmul_dev(const void *vals, const void *scales, const void *biases, int R, int C, int B,
+                             const float *xs, float *ys, void *workspace, void *stream) {
+    if (!g_state.ready) { set_error("q4 matmul: library not initialised"); return -1; }
+    if (!vals || !scales || !xs || !ys || !workspace || R < 1 || C < 64 || (C & 63) || B < 1 || B > 65535 ||
+        ((uintptr_t)vals & 15) || ((uintptr_t)scales & 1) || ((uintptr_t)biases & 1) || ((uintptr_t)xs & 15) ||
+        ((uintptr_t)workspace & 255)) {
+        set_error("q4 matmul: bad arguments (C multiple of 64, vals / xs 16-byte and workspace 256-byte aligned)");
+        return -1;
+    }
+    uint16_t *planes = (uint16_t *)workspace;
+    const size_t plane_stride = (size_t)B * C;
+    float *xsum = (float *)((uint8_t *)workspace + ((3 * plane_stride * 2 + 255) & ~(size_t)255));
+    if (x_split_launch(xs, nullptr, 1, C, B, C, planes, plane_stride, xsum, (hipStream_t)stream) != 0) {
+        set_error("q4 matmul: activation split launch failed");
+        return -1;
+    }
+    MfmaLaunch launch;
+    memset(&launch, 0, sizeof launch);
+    launch.one.vals = (const uint8_t *)vals; launch.one.scales = (const uint8_t *)scales;
+    launch.one.biases = (const uint8_t *)biases;
+    launch.one.planes = planes; launch.one.xsum = xsum; launch.one.y = ys;
+    launch.one.tokens = B; launch.one.rows = R;
+    launch.njobs = 1; launch.cols = C; launch.plane_stride = plane_stride;
+    launch.total_tiles = mfma_tiles(B, R);
+    if (q4_mfma_launch(launch, (hipStream_t)stream) != 0) { set_error("q4 matmul: launch failed"); return -1; }
+    return 0;
+}
+
 int salt_mi355_nvfp4_qdq_dev(const float *input, int C, int B, float input_global_scale, uint8_t *packed,
                              uint8_t *scales, float *dequant, int *status_dev, void *stream) {
     if (!g_state.ready) { set_error("nvfp4 qdq: library not initialised"); return -1; }

@@ -45,6 +45,36 @@ bool q4_job_is_tileable(const Q4Job &job, int cols);
 // fills table[i].tile0 and returns the launch's tile count
 int q4_assign_tiles(Q4Job *table, int njobs);
 
+// ---------------------------------------------------------------- affine Q4 on MFMA (tolerance class)
+
+// One weight matrix against `tokens` activation rows that have been split
+// into three bf16 planes (x = hi + mid + lo) with per-64-column sums.
+struct MfmaJob {
+    const uint8_t *vals, *scales, *biases;   // biases may be null
+    const uint16_t *planes;   // plane 0 of this job's first token; plane p lies p * plane_stride elements further
+    const float *xsum;        // [tokens][C/64]
+    float *y;                 // [tokens][rows]
+    int tokens;
+    int rows;
+    int tile0;
+    int reserved;
+};
+
+struct MfmaLaunch {
+    MfmaJob one;
+    const MfmaJob *table;
+    int njobs;
+    int cols;
+    int total_tiles;
+    size_t plane_stride;      // elements between planes
+};
+
+int q4_mfma_launch(const MfmaLaunch &launch, hipStream_t stream);
+int mfma_tiles(int tokens, int rows);
+// rows of fp32 -> bf16 planes + group sums; output row r reads input row row_map[r] / map_divisor when a map is given
+int x_split_launch(const float *x, const int *row_map, int map_divisor, int x_stride, int rows, int cols,
+                   uint16_t *planes, size_t plane_stride, float *xsum, hipStream_t stream);
+
 // ---------------------------------------------------------------- NVFP4
 
 struct Fp4Job {

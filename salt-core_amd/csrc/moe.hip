@@ -83,7 +83,15 @@ __global__ __launch_bounds__(ROUTER_MAX_EXPERTS) void router_topk_kernel(
     __syncthreads();
     if (e == 0 && !bad) {
         float all = 0.0f;
-        for (int j = 0; j < n_experts; ++j) all = all + s_exp[j];
+        int j0 = 0;
+        for (; j0 + 16 <= n_experts; j0 += 16) {       // batches of LDS reads, then the ordered adds
+            float v[16];
+#pragma unroll
+            for (int k = 0; k < 16; ++k) v[k] = s_exp[j0 + k];
+#pragma unroll
+            for (int k = 0; k < 16; ++k) all = all + v[k];
+        }
+        for (int j = j0; j < n_experts; ++j) all = all + s_exp[j];
         if (!(all > 0.0f) || !(all < __builtin_inff())) bad = 1;
         float chosen = 0.0f;
         if (!bad) {

@@ -65,6 +65,8 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_q4_matvec_dev, i, vp, vp, vp, i, i, i, vp, vp, i, vp)
     _sig(lib.salt_mi355_q4_jobs_dev, i, C.POINTER(Q4Job), i, i, i, i, vp)
     _sig(lib.salt_mi355_set_q4_accumulate, i, i)
+    _sig(lib.salt_mi355_q4_matmul_workspace_bytes, sz, i, i)
+    _sig(lib.salt_mi355_q4_matmul_dev, i, vp, vp, vp, i, i, i, vp, vp, vp, vp)
     _sig(lib.salt_mi355_nvfp4_qdq_dev, i, vp, i, i, f, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_nvfp4_matvec_dev, i, vp, vp, f, i, i, i, vp, vp, i, vp)
     _sig(lib.salt_mi355_router_topk_dev, i, vp, vp, i, i, i, vp, vp, vp, vp)
@@ -233,3 +235,19 @@ class MoeLayer:
         status = int(self.ws.to_host(np.int32, 1)[0])
         return (status, self.sel.to_host(np.int32), self.w.to_host(np.float32),
                 self.eo.to_host(np.float32).reshape(self.K, self.H), self.out.to_host(np.float32))
+
+
+def q4_matmul(vals, scales, biases, R: int, C_: int, xs: np.ndarray) -> np.ndarray:
+    """Host-array convenience around salt_mi355_q4_matmul_dev (MFMA, tolerance class)."""
+    lib = init()
+    xs = np.ascontiguousarray(xs, np.float32).reshape(-1, C_)
+    B = xs.shape[0]
+    dv, ds = DeviceBuffer.from_host(vals), DeviceBuffer.from_host(scales)
+    db = DeviceBuffer.from_host(biases) if biases is not None else None
+    dx, dy = DeviceBuffer.from_host(xs), DeviceBuffer(B * R * 4, fill=0xFF)
+    ws = DeviceBuffer(lib.salt_mi355_q4_matmul_workspace_bytes(C_, B))
+    stream = lib.salt_mi355_stream()
+    check(lib.salt_mi355_q4_matmul_dev(dv.ptr, ds.ptr, db.ptr if db else None, R, C_, B, dx.ptr, dy.ptr, ws.ptr, stream),
+          "q4_matmul_dev")
+    check(lib.salt_mi355_stream_sync(stream), "sync")
+    return dy.to_host(np.float32).reshape(B, R)
