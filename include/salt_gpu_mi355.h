@@ -156,6 +156,26 @@ int salt_mi355_moe_decode_step_dev(const void *pool, size_t expert_stride,
                                    const float *x, int *selected, float *weights,
                                    float *expert_out, float *out,
                                    void *workspace, void *stream);
+/* Many tokens through the experts of one MoE layer, grouped per expert
+ * (reference src/moe_group.c:24-97 validation, :138-184 grouping in ascending
+ * expert / token / rank order, :211-224 weighted sum over ranks in rank order
+ * from +0; per-expert arithmetic gemma4_text.c:8749-9137).  The bucketing is
+ * exact; the projections run on the matrix-core kernel of
+ * salt_mi355_q4_matmul_dev and carry its tolerance.  selected / weights:
+ * [tokens][topk] (any order inside a token; experts distinct, weights
+ * finite); inputs / outputs: [tokens][hidden].  Optional results: group_rows
+ * [n_experts] rows per expert, row_pairs [tokens*topk] the pair index
+ * token*topk+rank of each grouped row.  status_dev (optional device int):
+ * receives 0 or -1 and the call stays asynchronous; without it the call waits
+ * for the stream and returns -1 for an invalid selection.  Outputs are not
+ * written for an invalid selection. */
+size_t salt_mi355_moe_prefill_workspace_bytes(int hidden, int routed, int n_experts, int topk, int tokens);
+int salt_mi355_moe_prefill_dev(const void *pool, size_t expert_stride,
+                               int hidden, int routed, int n_experts, int topk, int tokens,
+                               const int *selected, const float *weights,
+                               const float *inputs, float *outputs,
+                               int *group_rows, int *row_pairs, int *status_dev,
+                               void *workspace, void *stream);
 /* The pieces of the step on their own: act = gelu_tanh(gate) * up over n
  * floats (gemma4.c:80-83, gemma4_text.c:7635), and out[d] = sum_i
  * expert_out[i][d] * weights[i] from +0 in ascending i (gemma4_text.c:8301-8304). */

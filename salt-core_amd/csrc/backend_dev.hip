@@ -25,7 +25,7 @@ int salt_mi355_q4_matmul_dev(const void *vals, const void *scales, const void *b
     uint16_t *planes = (uint16_t *)workspace;
     const size_t plane_stride = (size_t)B * C;
     float *xsum = (float *)((uint8_t *)workspace + ((3 * plane_stride * 2 + 255) & ~(size_t)255));
-    if (x_split_launch(xs, nullptr, 1, C, B, C, planes, plane_stride, xsum, (hipStream_t)stream) != 0) {
+    if (x_split_launch(xs, nullptr, nullptr, 1, C, B, C, planes, plane_stride, xsum, (hipStream_t)stream) != 0) {
         set_error("q4 matmul: activation split launch failed");
         return -1;
     }
@@ -97,6 +97,45 @@ int salt_mi355_router_topk_dev(const float *logits, const float *per_expert_scal
         set_error("router: unsupported geometry (experts %d, topk %d) or launch failure", n_experts, topk);
         return -1;
     }
+    return 0;
+}
+
+size_t salt_mi355_moe_prefill_workspace_bytes(int hidden, int routed, int n_experts, int topk, int tokens) {
+    if (hidden < 64 || routed < 64 || n_experts < 1 || topk < 1 || tokens < 1) return 0;
+    const MoeGeometry g = {hidden, routed, n_experts, topk};
+    return moe_prefill_workspace_bytes(g, tokens);
+}
+
+int salt_mi355_moe_prefill_dev(const void *pool, size_t expert_stride, int hidden, int routed, int n_experts, int topk,
+                               int tokens, const int *selected, const float *weights, const float *inputs,
+                               float *outputs, int *group_rows, int *row_pairs, int *status_dev, void *workspace,
+                               void *stream) {
+    if (!g_state.ready) { set_error("moe prefill: library not initialised"); return -1; }
+    if (!pool || !selected || !weights || !inputs || !outputs || !workspace || ((uintptr_t)pool & 15) ||
+        (expert_stride & 15) || ((uintptr_t)workspace & 255) || ((uintptr_t)inputs & 15)) {
+        set_error("moe prefill: bad arguments (pool, stride and inputs 16-byte aligned, workspace 256-byte aligned)");
+        return -1;
+    }
+    const MoeGeometry g = {hidden, routed, n_experts, topk};
+    const size_t n = (size_t)hidden * (size_t)routed;
+    if (hidden < 64 || (hidden & 63) || routed < 64 || (routed & 63) || expert_stride < 3 * (n / 2 + 4 * (n / 64))) {
+        set_error("moe prefill: hidden and routed must be multiples of 64 and the stride must cover a slot");
+        return -1;
+    }
+    if (moe_prefill_launch(g, (const uint8_t *)pool, expert_stride, tokens, selected, weights, inputs, outputs,
+                           group_rows, row_pairs, status_dev, workspace, (hipStream_t)stream) != 0) {
+        set_error("moe prefill: unsupported geometry (experts %d, topk %d, tokens %d) or launch failure", n_experts,
+                  topk, tokens);
+        return -1;
+    }
+    if (status_dev) return 0;
+    // no status word from the caller: wait, and report an invalid selection as a failed call
+    int status = -1;
+    if (hip_ok(hipMemcpyAsync(&status, workspace, sizeof status, hipMemcpyDeviceToHost, (hipStream_t)stream),
+               "moe prefill status") != 0 ||
+        hip_ok(hipStreamSynchronize((hipStream_t)stream), "moe prefill sync") != 0)
+        return -1;
+    if (status != 0) { set_error("moe prefill: invalid selection (expert id, duplicate or weight)"); return -1; }
     return 0;
 }
 

@@ -65,15 +65,18 @@ struct MfmaLaunch {
     const MfmaJob *table;
     int njobs;
     int cols;
-    int total_tiles;
+    int total_tiles;          // grid size; an upper bound when the counts below live on the device
     size_t plane_stride;      // elements between planes
+    const int *njobs_dev;     // optional: job and tile counts produced by an earlier kernel;
+    const int *total_tiles_dev;   // workgroups past *total_tiles_dev exit at once
 };
 
 int q4_mfma_launch(const MfmaLaunch &launch, hipStream_t stream);
 int mfma_tiles(int tokens, int rows);
-// rows of fp32 -> bf16 planes + group sums; output row r reads input row row_map[r] / map_divisor when a map is given
-int x_split_launch(const float *x, const int *row_map, int map_divisor, int x_stride, int rows, int cols,
-                   uint16_t *planes, size_t plane_stride, float *xsum, hipStream_t stream);
+// rows of fp32 -> bf16 planes + group sums; output row r reads input row row_map[r] / map_divisor when a map is
+// given; with a gate the value split is gelu_tanh(gate) * x (gate has the layout of x)
+int x_split_launch(const float *x, const float *gate, const int *row_map, int map_divisor, int x_stride, int rows,
+                   int cols, uint16_t *planes, size_t plane_stride, float *xsum, hipStream_t stream);
 
 // ---------------------------------------------------------------- NVFP4
 
@@ -139,6 +142,15 @@ int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t exp
 int moe_activate_launch(const float *gate, const float *up, float *act, size_t n, hipStream_t stream);
 int moe_reduce_launch(const float *expert_out, const float *weights, int topk, int hidden, float *out,
                       hipStream_t stream);
+
+// Grouped prefill MoE (reference src/moe_group.c): rows bucketed per expert in
+// ascending expert / token / rank order, gate-up and down on the MFMA kernel,
+// ordered weighted reduction.  Device workspace sized by moe_prefill_workspace_bytes.
+size_t moe_prefill_workspace_bytes(const MoeGeometry &g, int tokens);
+// status_dev receives 0, or -1 for an invalid selection (then outputs are not written).
+int moe_prefill_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_stride, int tokens,
+                       const int *selected, const float *weights, const float *inputs, float *outputs,
+                       int *group_rows, int *row_pairs, int *status_dev, void *workspace, hipStream_t stream);
 
 // ---------------------------------------------------------------- probes
 

@@ -22,6 +22,7 @@
 // (scale, bias) pair per group).  Per group the planes, the packed codes, the
 // (scale, bias - 16*scale) pairs and the group sums of x are staged in LDS with
 // the next group's loads in flight.
+#include "device_math.h"
 #include "mi355_internal.h"
 
 #include <stddef.h>
@@ -46,7 +47,8 @@ static_assert(sizeof(MfmaJob) == 64, "find_job reads a job record as eight 64-bi
 __device__ __forceinline__ MfmaJob find_job(const MfmaLaunch &L, int tile) {
     if (L.table == nullptr) return L.one;
     const uniform_u64_ptr words = (uniform_u64_ptr)(uintptr_t)L.table;
-    int lo = 0, hi = L.njobs - 1;
+    const int njobs = L.njobs_dev ? *(const int __attribute__((address_space(4))) *)(uintptr_t)L.njobs_dev : L.njobs;
+    int lo = 0, hi = njobs - 1;
     while (lo < hi) {
         const int mid = (lo + hi + 1) >> 1;
         if ((int)(uint32_t)words[8 * mid + 7] <= tile) lo = mid; else hi = mid - 1;
@@ -92,6 +94,9 @@ __global__ __launch_bounds__(256) void q4_mfma_kernel(const MfmaLaunch L) {
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, half = lane >> 5;
 
+    if (L.total_tiles_dev &&
+        (int)blockIdx.x >= *(const int __attribute__((address_space(4))) *)(uintptr_t)L.total_tiles_dev)
+        return;                                     // uniform: the whole workgroup leaves
     const MfmaJob job = find_job(L, blockIdx.x);
     const int C = L.cols, ngrp = C >> 6;
     const int ntiles = (job.rows + TN - 1) / TN;
@@ -204,12 +209,16 @@ __device__ __forceinline__ uint32_t f32_to_bf16_rne(float v) {
     return (bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16;
 }
 
-__global__ __launch_bounds__(256) void x_split_kernel(const float *__restrict__ x, const int *__restrict__ row_map,
-                                                      int map_divisor, int x_stride, int rows, int cols,
-                                                      uint16_t *__restrict__ planes, size_t plane_stride,
-                                                      float *__restrict__ xsum) {
-    const int row = blockIdx.y;
-    const int c0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+// With GATED the value split is gelu_tanh(gate) * x (the expert activation,
+// reference gemma4_text.c:8749-9137 "down input"), so the activations never
+// make a round trip through memory in fp32.
+template <bool GATED>
+__global__ __launch_bounds__(256) void x_split_kernel(const float *__restrict__ x, const float *__restrict__ gate,
+                                                      const int *__restrict__ row_map, int map_divisor, int x_stride,
+                                                      int rows, int cols, uint16_t *__restrict__ planes,
+                                                      size_t plane_stride, float *__restrict__ xsum) {
+    const int row = blockIdx.x;
+    const int c0 = (blockIdx.y * 256 + threadIdx.x) * 8;
     const bool live = c0 < cols;
     float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     if (live) {
@@ -217,6 +226,13 @@ __global__ __launch_bounds__(256) void x_split_kernel(const float *__restrict__ 
         const float4 *src = reinterpret_cast<const float4 *>(x + (size_t)src_row * x_stride + c0);
         const float4 a = src[0], b = src[1];
         v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+        if (GATED) {
+            const float4 *gsrc = reinterpret_cast<const float4 *>(gate + (size_t)src_row * x_stride + c0);
+            const float4 ga = gsrc[0], gb = gsrc[1];
+            const float gv[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = det_gelu_tanh(gv[j]) * v[j];
+        }
     }
     uint32_t hi[4], mid[4], lo[4];
     float sum = 0.0f;
@@ -252,12 +268,16 @@ int q4_mfma_launch(const MfmaLaunch &L, hipStream_t stream) {
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
-int x_split_launch(const float *x, const int *row_map, int map_divisor, int x_stride, int rows, int cols,
-                   uint16_t *planes, size_t plane_stride, float *xsum, hipStream_t stream) {
+int x_split_launch(const float *x, const float *gate, const int *row_map, int map_divisor, int x_stride, int rows,
+                   int cols, uint16_t *planes, size_t plane_stride, float *xsum, hipStream_t stream) {
     if (rows < 1 || cols < 64 || (cols & 63)) return -1;
-    const dim3 grid((cols / 8 + 255) / 256, rows);
-    hipLaunchKernelGGL(x_split_kernel, grid, dim3(256), 0, stream, x, row_map, map_divisor, x_stride, rows, cols,
-                       planes, plane_stride, xsum);
+    const dim3 grid(rows, (cols / 8 + 255) / 256);
+    if (gate)
+        hipLaunchKernelGGL(x_split_kernel<true>, grid, dim3(256), 0, stream, x, gate, row_map, map_divisor, x_stride,
+                           rows, cols, planes, plane_stride, xsum);
+    else
+        hipLaunchKernelGGL(x_split_kernel<false>, grid, dim3(256), 0, stream, x, gate, row_map, map_divisor, x_stride,
+                           rows, cols, planes, plane_stride, xsum);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

@@ -72,6 +72,8 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_router_topk_dev, i, vp, vp, i, i, i, vp, vp, vp, vp)
     _sig(lib.salt_mi355_moe_workspace_bytes, sz, i, i, i, i)
     _sig(lib.salt_mi355_moe_decode_step_dev, i, vp, sz, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, vp, vp)
+    _sig(lib.salt_mi355_moe_prefill_workspace_bytes, sz, i, i, i, i, i)
+    _sig(lib.salt_mi355_moe_prefill_dev, i, vp, sz, i, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_moe_activate_dev, i, vp, vp, vp, sz, vp)
     _sig(lib.salt_mi355_moe_reduce_dev, i, vp, vp, i, i, vp, vp)
     _lib = lib
@@ -251,3 +253,40 @@ def q4_matmul(vals, scales, biases, R: int, C_: int, xs: np.ndarray) -> np.ndarr
           "q4_matmul_dev")
     check(lib.salt_mi355_stream_sync(stream), "sync")
     return dy.to_host(np.float32).reshape(B, R)
+
+
+class MoePrefill:
+    """One MoE layer's experts in HBM plus the workspace of the grouped prefill
+    path (salt_mi355_moe_prefill_dev) for up to `tokens` tokens."""
+
+    def __init__(self, pool: np.ndarray, n_experts: int, hidden: int, routed: int, topk: int, tokens: int):
+        self.lib = init()
+        self.E, self.H, self.F, self.K, self.T = n_experts, hidden, routed, topk, tokens
+        self.stride = pool.nbytes // n_experts
+        self.pool = DeviceBuffer.from_host(pool)
+        self.ws = DeviceBuffer(self.lib.salt_mi355_moe_prefill_workspace_bytes(hidden, routed, n_experts, topk, tokens))
+        self.sel, self.w = DeviceBuffer(tokens * topk * 4), DeviceBuffer(tokens * topk * 4)
+        self.x, self.out = DeviceBuffer(tokens * hidden * 4), DeviceBuffer(tokens * hidden * 4)
+        self.group_rows, self.row_pairs = DeviceBuffer(n_experts * 4), DeviceBuffer(tokens * topk * 4)
+        self.status = DeviceBuffer(4)
+
+    def enqueue(self, stream, tokens: int | None = None):
+        T = self.T if tokens is None else tokens
+        return self.lib.salt_mi355_moe_prefill_dev(self.pool.ptr, self.stride, self.H, self.F, self.E, self.K, T,
+                                                   self.sel.ptr, self.w.ptr, self.x.ptr, self.out.ptr,
+                                                   self.group_rows.ptr, self.row_pairs.ptr, self.status.ptr,
+                                                   self.ws.ptr, stream)
+
+    def run(self, selected: np.ndarray, weights: np.ndarray, xs: np.ndarray):
+        """-> (status, outputs [T][hidden], rows per expert, pair index of each grouped row)"""
+        T = selected.shape[0]
+        assert T <= self.T
+        self.sel.upload(np.ascontiguousarray(selected, np.int32))
+        self.w.upload(np.ascontiguousarray(weights, np.float32))
+        self.x.upload(np.ascontiguousarray(xs, np.float32))
+        self.lib.salt_mi355_dev_fill(self.out.ptr, 0xFF, T * self.H * 4)
+        stream = self.lib.salt_mi355_stream()
+        check(self.enqueue(stream, T), "moe_prefill_dev")
+        check(self.lib.salt_mi355_stream_sync(stream), "sync")
+        return (int(self.status.to_host(np.int32)[0]), self.out.to_host(np.float32, T * self.H).reshape(T, self.H),
+                self.group_rows.to_host(np.int32), self.row_pairs.to_host(np.int32, T * self.K))
