@@ -49,6 +49,8 @@ int q4_assign_tiles(Q4Job *table, int njobs);
 
 // One weight matrix against `tokens` activation rows that have been split
 // into three bf16 planes (x = hi + mid + lo) with per-64-column sums.
+constexpr int MFMA_TM = 64, MFMA_TN = 128;   // tokens x weight rows per workgroup of the matrix-core kernel
+
 struct MfmaJob {
     const uint8_t *vals, *scales, *biases;   // biases may be null
     const uint16_t *planes;   // plane 0 of this job's first token; plane p lies p * plane_stride elements further

@@ -64,7 +64,7 @@ __global__ __launch_bounds__(MAX_EXPERTS) void group_scan_kernel(const ScanArgs 
     const int e = threadIdx.x;
     const int n = e < a.n_experts ? a.counts[e] : 0;
     s_rows[e] = n;
-    s_mtiles[e] = (n + 63) / 64;
+    s_mtiles[e] = (n + MFMA_TM - 1) / MFMA_TM;
     s_used[e] = n > 0;
     __syncthreads();
     int row0 = 0, mt0 = 0, job = 0;
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(MAX_EXPERTS) void group_scan_kernel(const ScanArgs 
         a.offsets[e] = row0;
         if (a.group_rows) a.group_rows[e] = n;
     }
-    const int nt_up = (a.routed + 63) / 64, nt_down = (a.hidden + 63) / 64;
+    const int nt_up = (a.routed + MFMA_TN - 1) / MFMA_TN, nt_down = (a.hidden + MFMA_TN - 1) / MFMA_TN;
     const bool valid = a.plan->status == 0;          // written by the previous kernel on this stream
     if (e == a.n_experts - 1) {
         a.offsets[a.n_experts] = row0 + n;
@@ -206,7 +206,7 @@ int moe_prefill_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_
         return -1;
     const PrefillWorkspace w = carve(g, tokens, workspace);
     const int rows = tokens * g.topk;
-    const int nt_up = g.routed / 64, nt_down = g.hidden / 64;
+    const int nt_up = (g.routed + MFMA_TN - 1) / MFMA_TN, nt_down = (g.hidden + MFMA_TN - 1) / MFMA_TN;
     if (hipMemsetAsync(w.plan, 0, sizeof(PrefillPlan), stream) != hipSuccess ||
         hipMemsetAsync(w.counts, 0, (size_t)g.n_experts * 4, stream) != hipSuccess)
         return -1;
@@ -229,9 +229,9 @@ int moe_prefill_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_
                        w.xsum_in, stream) != 0)
         return -1;
     // The number of 64-token tiles is known only on the device; the grid covers
-    // its upper bound (sum over experts of ceil(n_e / 64) <= rows / 64 + experts)
+    // its upper bound (sum over experts of ceil(n_e / TM) <= rows / TM + experts)
     // and surplus workgroups leave at once.
-    const int m_upper = rows / 64 + (g.n_experts < rows ? g.n_experts : rows);
+    const int m_upper = rows / MFMA_TM + (g.n_experts < rows ? g.n_experts : rows);
     MfmaLaunch gu;
     memset(&gu, 0, sizeof gu);
     gu.table = w.gate_up_jobs; gu.cols = g.hidden; gu.total_tiles = 2 * m_upper * nt_up;

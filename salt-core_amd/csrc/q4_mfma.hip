@@ -8,24 +8,32 @@
 //
 // How the affine weights reach the matrix cores without losing bits:
 //  * per 64-column scale group,  sum_c (q s + b) x = s * sum_c q x + b * sum_c x.
-//    The integer codes are exact in bf16, so only sum_c q x goes through MFMA;
-//    scale and bias are applied per group in fp32 on the VALU.
-//  * a nibble becomes the bf16 value 16 + q with three bit operations
-//    (0x4180 | q << 3); the surplus 16 * sum_c x is removed with the bias term.
-//  * the fp32 activation is split once into three bf16 planes
-//    (x = hi + mid + lo to 2^-24), each of which is an exact MFMA operand;
-//    accumulation is fp32.
+//    The integer codes are exact in bf16, so only sum_c q x goes through MFMA
+//    per group; the scale is applied per group in fp32 on the VALU.
+//  * a nibble becomes the bf16 value 16 + q with two bit operations per pair
+//    ((w >> n) & 0x00780078 | 0x41804180); the surplus 16 * s * sum_c x joins
+//    the bias term.
+//  * the bias term sum_g (b_g - 16 s_g) * X_g (X_g = the group sums of x) is
+//    itself a small contraction over the groups; b and s are bf16, so it runs
+//    on the matrix cores once per tile before the main loop.
+//  * every fp32 operand (x, X_g) is split into three bf16 planes
+//    (v = hi + mid + lo to 2^-24), each an exact MFMA operand; accumulation is
+//    fp32.
 //
-// Tiling: a workgroup of four waves computes 64 tokens x 64 weight rows, each
-// wave a 32 x 32 block with v_mfma_f32_32x32x16_bf16 (tokens are the M rows,
-// weight rows the N columns, so a lane owns one weight row and needs one
-// (scale, bias) pair per group).  Per group the planes, the packed codes, the
-// (scale, bias - 16*scale) pairs and the group sums of x are staged in LDS with
-// the next group's loads in flight.
+// Tiling: a workgroup of four waves computes 64 tokens x 128 weight rows, each
+// wave 32 tokens x 64 rows as two 32 x 32 blocks of v_mfma_f32_32x32x16_bf16
+// that share the token operand (tokens are the M rows, weight rows the N
+// columns, so a lane owns one weight row per block and needs one scale per
+// group).  Per group the planes, the packed codes and the scales are staged in
+// one of two LDS stages, the next group's loads in flight during the matrix
+// work, one barrier per group.  Inside every aligned run of eight columns the
+// planes are stored in the order 0,4,1,5,2,6,3,7, which is the order the pair
+// extraction above yields the codes in.
 #include "device_math.h"
 #include "mi355_internal.h"
 
 #include <stddef.h>
+#include <type_traits>
 
 namespace mi355 {
 namespace {
@@ -38,9 +46,16 @@ typedef const u32x4 __attribute__((address_space(1))) *global_u128_ptr;
 typedef const uint16_t __attribute__((address_space(1))) *global_u16_ptr;
 typedef const float __attribute__((address_space(1))) *global_f32_ptr;
 
-constexpr int TM = 64, TN = 64;            // tokens x weight rows per workgroup
+constexpr int TM = MFMA_TM, TN = MFMA_TN;   // tokens x weight rows per workgroup
 constexpr int X_PITCH = 144;               // bytes per staged token row of one plane: 64 bf16 + 16 pad
 constexpr int W_PITCH = 36;                // bytes per staged weight row of one group: 32 + 4 pad
+constexpr int XS_BYTES = 3 * TM * X_PITCH, WS_BYTES = TN * W_PITCH;
+constexpr int SC_OFF = XS_BYTES + WS_BYTES;                 // float scale[TN]
+constexpr int STAGE_BYTES = (SC_OFF + TN * 4 + 15) & ~15;
+// bias pass (before the main loop, in the same LDS): 16 groups per step
+constexpr int G_PITCH = 48;                // bytes per staged row of 16 bf16: 32 + 16 pad
+constexpr int XG_BYTES = 3 * TM * G_PITCH, BS_BYTES = 2 * TN * G_PITCH;
+static_assert(XG_BYTES + BS_BYTES <= 2 * STAGE_BYTES, "the bias pass reuses the staging memory");
 
 static_assert(sizeof(MfmaJob) == 64, "find_job reads a job record as eight 64-bit words");
 
@@ -70,28 +85,82 @@ __device__ __forceinline__ MfmaJob find_job(const MfmaLaunch &L, int tile) {
 
 __device__ __forceinline__ float bf16_to_f32(uint32_t half) { return __uint_as_float(half << 16); }
 
-// Eight nibbles -> eight bf16 values 16 + q, in column order.
-__device__ __forceinline__ bf16x8 codes_to_bf16(uint32_t w) {
-    const uint32_t even = (w << 3) & 0x78787878u;        // q0, q2, q4, q6 (each << 3) in bytes 0..3
-    const uint32_t odd = (w >> 1) & 0x78787878u;         // q1, q3, q5, q7
+// Eight nibbles -> eight bf16 values 16 + q, in the column order 0,4,1,5,2,6,3,7.
+// (a & mask) | bits in one instruction; the three-operand form takes no
+// literals, so the mask travels in a scalar register and the bits in a vector one.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t bits) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(bits));
+    return r;
+}
+
+__device__ __forceinline__ bf16x8 codes_to_bf16(uint32_t w, uint32_t mask, uint32_t sixteen) {
     u32x4 r;
-    r.x = __builtin_amdgcn_perm(odd, even, 0x0C040C00u) | 0x41804180u;
-    r.y = __builtin_amdgcn_perm(odd, even, 0x0C050C01u) | 0x41804180u;
-    r.z = __builtin_amdgcn_perm(odd, even, 0x0C060C02u) | 0x41804180u;
-    r.w = __builtin_amdgcn_perm(odd, even, 0x0C070C03u) | 0x41804180u;
+    r.x = and_or((w << 3), mask, sixteen);               // columns 0 and 4
+    r.y = and_or((w >> 1), mask, sixteen);               // 1 and 5
+    r.z = and_or((w >> 5), mask, sixteen);               // 2 and 6
+    r.w = and_or((w >> 9), mask, sixteen);               // 3 and 7
     return __builtin_bit_cast(bf16x8, r);
 }
 
-__global__ __launch_bounds__(256) void q4_mfma_kernel(const MfmaLaunch L) {
-    __shared__ __attribute__((aligned(16))) uint8_t xs[3 * TM * X_PITCH];
-    __shared__ __attribute__((aligned(16))) uint8_t ws[TN * W_PITCH];
-    __shared__ float2 ms[TN];
-    __shared__ float xg[TM];
+__device__ __forceinline__ uint32_t f32_to_bf16_rne(float v) {
+    const uint32_t bits = __float_as_uint(v);
+    return (bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16;
+}
+
+// v = hi + mid + lo, each a bf16 (bit patterns in the low halves)
+__device__ __forceinline__ void split3(float v, uint32_t &h, uint32_t &m, uint32_t &l) {
+    h = f32_to_bf16_rne(v);
+    const float r1 = v - bf16_to_f32(h);
+    m = f32_to_bf16_rne(r1);
+    const float r2 = r1 - bf16_to_f32(m);
+    l = f32_to_bf16_rne(r2);
+}
+
+// One scale group of one wave: NB blocks of 32 rows against the wave's 32 tokens.
+template <int NB>
+__device__ __forceinline__ void group_product(const uint8_t *cur, int wm, int wn, int l32, int half, f32x16 (&acc)[2]) {
+    const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    f32x16 part[NB];
+    uint32_t sixteen;                                   // two bf16 values 16.0, kept in a vector register
+    asm("v_mov_b32 %0, 0x41804180" : "=v"(sixteen));
+    const uint8_t *wrow = cur + XS_BYTES + (wn * 64 + l32) * W_PITCH + half * 4;
+    const uint8_t *xrow = cur + (wm * 32 + l32) * X_PITCH + half * 16;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        bf16x8 a[3], b[NB];
+#pragma unroll
+        for (int plane = 0; plane < 3; ++plane)
+            a[plane] = __builtin_bit_cast(bf16x8,
+                                          *reinterpret_cast<const u32x4 *>(xrow + plane * (TM * X_PITCH) + ks * 32));
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+            b[nb] = codes_to_bf16(*reinterpret_cast<const uint32_t *>(wrow + nb * 32 * W_PITCH + ks * 8), 0x00780078u,
+                                  sixteen);
+#pragma unroll
+        for (int plane = 0; plane < 3; ++plane)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+                part[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[plane], b[nb], (ks | plane) ? part[nb] : zero, 0, 0, 0);
+    }
+    const float *sc = reinterpret_cast<const float *>(cur + SC_OFF) + wn * 64 + l32;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const float s = sc[nb * 32];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[nb][i] = __builtin_fmaf(s, part[nb][i], acc[nb][i]);
+    }
+}
+
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+void q4_mfma_kernel(const MfmaLaunch L) {
+    // two stages of { planes [3][64 tokens], codes [128 rows], scales [128] }
+    __shared__ __attribute__((aligned(16))) uint8_t stage[2 * STAGE_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave >> 1, wn = wave & 1;       // wave tile: tokens wm*32.., rows wn*64.. (two 32-row blocks)
     const int l32 = lane & 31, half = lane >> 5;
 
     if (L.total_tiles_dev &&
@@ -118,97 +187,135 @@ __global__ __launch_bounds__(256) void q4_mfma_kernel(const MfmaLaunch L) {
         x_dst[i] = plane * (TM * X_PITCH) + tok * X_PITCH + seg * 16;
     }
     const size_t plane_stride = L.plane_stride;
-    // codes: 64 rows * 2 pieces of 16 bytes, threads 0..127
-    const int w_row = (tid >> 1) & 63, w_half = tid & 1;
+    // codes: 128 rows * 2 pieces of 16 bytes, one per thread
+    const int w_row = tid >> 1, w_half = tid & 1;
     const int w_rc = w_row < rows_here ? w_row : rows_here - 1;
     const global_u128_ptr w_src = (global_u128_ptr)((uintptr_t)job.vals + (size_t)(row0 + w_rc) * (C >> 1) + w_half * 16);
-    // (scale, bias): threads 128..191; group sums of x: threads 192..255
-    const int m_row = tid & 63;
+    // scales: threads 0..127
+    const int m_row = tid & 127;
     const int m_rc = m_row < rows_here ? m_row : rows_here - 1;
-    const int g_tc = m_row < toks_here ? m_row : toks_here - 1;
     const global_u16_ptr scales = (global_u16_ptr)(uintptr_t)job.scales + (size_t)(row0 + m_rc) * ngrp;
-    const global_u16_ptr biases = job.biases ? (global_u16_ptr)(uintptr_t)job.biases + (size_t)(row0 + m_rc) * ngrp
-                                             : (global_u16_ptr)0;
-    const global_f32_ptr xsum = (global_f32_ptr)(uintptr_t)job.xsum + (size_t)(tok0 + g_tc) * ngrp;
 
     u32x4 xreg[6], wreg;
-    uint32_t sreg = 0, breg = 0;
-    float greg = 0.0f;
+    uint32_t sreg = 0;
     auto issue = [&](int g) {
 #pragma unroll
         for (int i = 0; i < 6; ++i) {
             const int plane = (tid + i * 256) >> 9;
             xreg[i] = *(global_u128_ptr)(planes + (size_t)plane * plane_stride + x_src[i] + (uint32_t)g * 64u);
         }
-        if (tid < 128) wreg = w_src[g * 2];
-        else if (tid < 192) { sreg = scales[g]; breg = biases ? (uint32_t)biases[g] : 0u; }
-        else greg = xsum[g];
+        wreg = w_src[g * 2];
+        if (tid < 128) sreg = scales[g];
     };
-    auto commit = [&]() {
+    auto commit = [&](uint8_t *base) {
 #pragma unroll
-        for (int i = 0; i < 6; ++i) *reinterpret_cast<u32x4 *>(xs + x_dst[i]) = xreg[i];
-        if (tid < 128) {
-            uint32_t *dst = reinterpret_cast<uint32_t *>(ws + w_row * W_PITCH + w_half * 16);
-            dst[0] = wreg.x; dst[1] = wreg.y; dst[2] = wreg.z; dst[3] = wreg.w;
-        } else if (tid < 192) {
-            const float s = bf16_to_f32(sreg), b = bf16_to_f32(breg);
-            ms[m_row] = make_float2(s, b - 16.0f * s);
-        } else {
-            xg[m_row] = greg;
-        }
+        for (int i = 0; i < 6; ++i) *reinterpret_cast<u32x4 *>(base + x_dst[i]) = xreg[i];
+        uint32_t *dst = reinterpret_cast<uint32_t *>(base + XS_BYTES + w_row * W_PITCH + w_half * 16);
+        dst[0] = wreg.x; dst[1] = wreg.y; dst[2] = wreg.z; dst[3] = wreg.w;
+        if (tid < 128) reinterpret_cast<float *>(base + SC_OFF)[m_row] = bf16_to_f32(sreg);
     };
 
-    f32x16 acc;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    // a wave whose second (or both) 32-row blocks lie past the matrix skips their matrix work
+    const int nblocks = rows_here - wn * 64 <= 0 ? 0 : (rows_here - wn * 64 <= 32 ? 1 : 2);
 
-    issue(0);
-    for (int g = 0; g < ngrp; ++g) {
-        commit();
-        __syncthreads();
-        if (g + 1 < ngrp) issue(g + 1);
+    const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    f32x16 acc[2] = {zero, zero};
 
-        f32x16 part;
+    // ---- bias pass: acc[tok][row] = sum_g (b[row][g] - 16 s[row][g]) * X[tok][g]
+    {
+        const global_f32_ptr xsum = (global_f32_ptr)(uintptr_t)job.xsum;
+        const int xg_tok = tid >> 2, xg_g = (tid & 3) * 4;
+        const int xg_tc = xg_tok < toks_here ? xg_tok : toks_here - 1;
+        const int bs_arr = tid >> 7;                            // 0: biases, 1: scales
+        const global_u16_ptr bs_src = bs_arr ? scales : (job.biases ? (global_u16_ptr)(uintptr_t)job.biases +
+                                                                          (size_t)(row0 + m_rc) * ngrp
+                                                                    : (global_u16_ptr)0);
+        f32x16 tb[2] = {zero, zero}, ts[2] = {zero, zero};
+        for (int g0 = 0; g0 < ngrp; g0 += 16) {
+            uint32_t h[4], m[4], l[4];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) part[i] = 0.0f;
-        const uint8_t *wrow = ws + (wn * 32 + l32) * W_PITCH + half * 4;
-        const uint8_t *xrow = xs + (wm * 32 + l32) * X_PITCH + half * 16;
+            for (int j = 0; j < 4; ++j) {
+                const int g = g0 + xg_g + j;
+                const float v = g < ngrp ? xsum[(size_t)(tok0 + xg_tc) * ngrp + g] : 0.0f;
+                split3(v, h[j], m[j], l[j]);
+            }
+            uint32_t bs[8];
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            const bf16x8 b = codes_to_bf16(*reinterpret_cast<const uint32_t *>(wrow + ks * 8));
+            for (int j = 0; j < 16; ++j) {
+                const int g = g0 + j;
+                const uint32_t v = (g < ngrp && bs_src) ? (uint32_t)bs_src[g] : 0u;
+                if (j & 1) bs[j >> 1] |= v << 16; else bs[j >> 1] = v;
+            }
+            __syncthreads();                                    // the previous step's operands have been read
+            uint8_t *xgp = stage + xg_tok * G_PITCH + xg_g * 2;
+            *reinterpret_cast<uint2 *>(xgp) = make_uint2(h[0] | h[1] << 16, h[2] | h[3] << 16);
+            *reinterpret_cast<uint2 *>(xgp + TM * G_PITCH) = make_uint2(m[0] | m[1] << 16, m[2] | m[3] << 16);
+            *reinterpret_cast<uint2 *>(xgp + 2 * TM * G_PITCH) = make_uint2(l[0] | l[1] << 16, l[2] | l[3] << 16);
+            uint32_t *bsp = reinterpret_cast<uint32_t *>(stage + XG_BYTES + (bs_arr * TN + m_row) * G_PITCH);
 #pragma unroll
-            for (int plane = 0; plane < 3; ++plane) {
-                const u32x4 raw = *reinterpret_cast<const u32x4 *>(xrow + plane * (TM * X_PITCH) + ks * 32);
-                part = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, raw), b, part, 0, 0, 0);
+            for (int j = 0; j < 8; ++j) bsp[j] = bs[j];
+            __syncthreads();
+            if (nblocks > 0) {
+                const uint8_t *arow = stage + (wm * 32 + l32) * G_PITCH + half * 16;
+                const uint8_t *brow = stage + XG_BYTES + (wn * 64 + l32) * G_PITCH + half * 16;
+#pragma unroll
+                for (int plane = 0; plane < 3; ++plane) {
+                    const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(arow + plane * TM * G_PITCH));
+#pragma unroll
+                    for (int nb = 0; nb < 2; ++nb) {
+                        const bf16x8 bb = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(brow + nb * 32 * G_PITCH));
+                        const bf16x8 sb = __builtin_bit_cast(
+                            bf16x8, *reinterpret_cast<const u32x4 *>(brow + (TN + nb * 32) * G_PITCH));
+                        tb[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bb, tb[nb], 0, 0, 0);
+                        ts[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, sb, ts[nb], 0, 0, 0);
+                    }
+                }
             }
         }
-        const float2 sc = ms[wn * 32 + l32];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int tok = (i >> 2) * 8 + half * 4 + (i & 3);
-            acc[i] = __builtin_fmaf(sc.x, part[i], acc[i]);
-            acc[i] = __builtin_fmaf(sc.y, xg[wm * 32 + tok], acc[i]);
-        }
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[nb][i] = __builtin_fmaf(-16.0f, ts[nb][i], tb[nb][i]);
         __syncthreads();
     }
 
-    const int row = wn * 32 + l32;
-    if (row < rows_here) {
+    // ---- main loop: acc += s[row][g] * sum_{c in g} (16 + q[row][c]) * x[tok][c]
+    // The loop exists once per block count so that the accumulators stay in place.
+    auto main_loop = [&](auto block_count) {
+        constexpr int NB = decltype(block_count)::value;
+        issue(0);
+        commit(stage);
+        __syncthreads();
+        for (int g = 0; g < ngrp; ++g) {
+            const uint8_t *cur = stage + (g & 1) * STAGE_BYTES;
+            if (g + 1 < ngrp) issue(g + 1);
+            if (NB > 0) group_product<(NB > 0 ? NB : 1)>(cur, wm, wn, l32, half, acc);
+            if (g + 1 < ngrp) commit(stage + ((g + 1) & 1) * STAGE_BYTES);
+            __syncthreads();
+        }
+    };
+    if (nblocks == 2) main_loop(std::integral_constant<int, 2>{});
+    else if (nblocks == 1) main_loop(std::integral_constant<int, 1>{});
+    else main_loop(std::integral_constant<int, 0>{});
+
+    float __attribute__((address_space(1))) *y = (float __attribute__((address_space(1))) *)(uintptr_t)job.y;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int tok = wm * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
-            if (tok < toks_here) job.y[(size_t)(tok0 + tok) * job.rows + row0 + row] = acc[i];
+    for (int nb = 0; nb < 2; ++nb) {
+        const int row = wn * 64 + nb * 32 + l32;
+        if (row < rows_here) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int tok = wm * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
+                if (tok < toks_here) y[(size_t)(tok0 + tok) * job.rows + row0 + row] = acc[nb][i];
+            }
         }
     }
 }
 
-// fp32 rows -> three bf16 planes and per-64-column sums.  Row r of the output
-// is row row_map[r] of the input when a map is given (the grouped MoE gather).
-__device__ __forceinline__ uint32_t f32_to_bf16_rne(float v) {
-    const uint32_t bits = __float_as_uint(v);
-    return (bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16;
-}
-
+// fp32 rows -> three bf16 planes (columns permuted inside every run of eight,
+// see the top of the file) and per-64-column sums.  Row r of the output is row
+// row_map[r] / map_divisor of the input when a map is given (the grouped MoE
+// gather).
 // With GATED the value split is gelu_tanh(gate) * x (the expert activation,
 // reference gemma4_text.c:8749-9137 "down input"), so the activations never
 // make a round trip through memory in fp32.
@@ -238,13 +345,11 @@ __global__ __launch_bounds__(256) void x_split_kernel(const float *__restrict__ 
     float sum = 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        const uint32_t h = f32_to_bf16_rne(v[j]);
-        const float r1 = v[j] - bf16_to_f32(h);
-        const uint32_t m = f32_to_bf16_rne(r1);
-        const float r2 = r1 - bf16_to_f32(m);
-        const uint32_t l = f32_to_bf16_rne(r2);
-        if (j & 1) { hi[j >> 1] |= h << 16; mid[j >> 1] |= m << 16; lo[j >> 1] |= l << 16; }
-        else { hi[j >> 1] = h; mid[j >> 1] = m; lo[j >> 1] = l; }
+        uint32_t h, m, l;
+        split3(v[j], h, m, l);
+        const int k = j & 3;                           // dword k holds columns k (low half) and k + 4 (high half)
+        if (j & 4) { hi[k] |= h << 16; mid[k] |= m << 16; lo[k] |= l << 16; }
+        else { hi[k] = h; mid[k] = m; lo[k] = l; }
         sum += v[j];
     }
     // eight lanes cover one 64-column group
