@@ -130,6 +130,21 @@ int salt_mi355_nvfp4_matvec_dev(const void *packed, const void *scales, float st
                                 int R, int C, int B, const float *xs, float *ys,
                                 int chains_per_lane, void *stream);
 
+/* Prefill-sized NVFP4 matmul on the matrix cores (tolerance class): every
+ * token is quantised and dequantised as salt_nvfp4_quantize_input_reference
+ * does (nvfp4.c:82-130) and ys[token][row] approximates the reference matvec
+ * (nvfp4.c:228-256) of that token: code * block scale is exact in bf16 for both
+ * operands, products are exact, fp32 accumulation runs in the matrix cores'
+ * order and the two per-tensor factors are applied once at the end.
+ * xs: [B][C] fp32, ys: [B][R]; C a multiple of 64.  status_dev (optional device
+ * int) receives 0 or -1 (a non-finite activation: nothing is published) and
+ * the call stays asynchronous; without it the call waits and returns -1. */
+size_t salt_mi355_nvfp4_matmul_workspace_bytes(int R, int C, int B);
+int salt_mi355_nvfp4_matmul_dev(const void *packed, const void *scales,
+                                float stored_divisor, float input_global_scale,
+                                int R, int C, int B, const float *xs, float *ys,
+                                int *status_dev, void *workspace, void *stream);
+
 /* ---- MoE decode layer-step, device-resident ----------------------------- */
 
 /* reference salt_gemma4_router_topk (gemma4.c:132-186).  sorted_by_id = 0

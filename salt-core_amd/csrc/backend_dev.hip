@@ -51,7 +51,8 @@ int salt_mi355_nvfp4_qdq_dev(const float *input, int C, int B, float input_globa
         set_error("nvfp4 qdq: bad arguments");
         return -1;
     }
-    if (fp4_qdq_launch(input, C, B, input_global_scale, packed, scales, dequant, status_dev, (hipStream_t)stream) != 0) {
+    if (fp4_qdq_launch(input, C, B, input_global_scale, packed, scales, dequant, nullptr, status_dev,
+                       (hipStream_t)stream) != 0) {
         set_error("nvfp4 qdq: launch failed");
         return -1;
     }
@@ -85,6 +86,65 @@ int salt_mi355_nvfp4_matvec_dev(const void *packed, const void *scales, float st
         launch.total_tiles = (R + 63) / 64;
         if (fp4_launch(launch, chains, (hipStream_t)stream) != 0) { set_error("nvfp4 matvec: launch failed"); return -1; }
     }
+    return 0;
+}
+
+namespace {
+struct Fp4MatmulWorkspace { int *status; uint16_t *plane; float *partials; size_t bytes; };
+Fp4MatmulWorkspace fp4_matmul_carve(void *base, int R, int C, int B) {
+    Fp4MatmulWorkspace w;
+    uint8_t *p = (uint8_t *)base;
+    auto take = [&](size_t n) { uint8_t *q = p; p += (n + 255) & ~(size_t)255; return q; };
+    w.status = (int *)take(4);
+    w.plane = (uint16_t *)take((size_t)B * C * 2);
+    const int splits = fp4_mfma_splits(R, C, B);
+    w.partials = splits > 1 ? (float *)take((size_t)splits * B * R * 4) : nullptr;
+    w.bytes = (size_t)(p - (uint8_t *)base);
+    return w;
+}
+}  // namespace
+
+size_t salt_mi355_nvfp4_matmul_workspace_bytes(int R, int C, int B) {
+    if (R < 1 || C < 64 || (C & 63) || B < 1) return 0;
+    return fp4_matmul_carve(nullptr, R, C, B).bytes;
+}
+
+int salt_mi355_nvfp4_matmul_dev(const void *packed, const void *scales, float stored_divisor, float input_global_scale,
+                                int R, int C, int B, const float *xs, float *ys, int *status_dev, void *workspace,
+                                void *stream) {
+    if (!g_state.ready) { set_error("nvfp4 matmul: library not initialised"); return -1; }
+    if (!g_state.fp8_is_ocp) { set_error("nvfp4: this device's fp8 converter is not OCP E4M3FN"); return -1; }
+    if (!packed || !scales || !xs || !ys || !workspace || R < 1 || C < 64 || (C & 63) || B < 1 ||
+        !isfinite(stored_divisor) || stored_divisor == 0.0f || !isfinite(input_global_scale) ||
+        input_global_scale <= 0.0f || ((uintptr_t)packed & 15) || ((uintptr_t)scales & 1) || ((uintptr_t)xs & 15) ||
+        ((uintptr_t)ys & 15) || ((uintptr_t)workspace & 255)) {
+        set_error("nvfp4 matmul: bad arguments (C a multiple of 64; packed, xs, ys 16-byte and workspace 256-byte aligned)");
+        return -1;
+    }
+    const Fp4MatmulWorkspace w = fp4_matmul_carve(workspace, R, C, B);
+    hipStream_t s = (hipStream_t)stream;
+    if (hip_ok(hipMemsetAsync(w.status, 0, 4, s), "nvfp4 matmul status") != 0) return -1;
+    if (fp4_qdq_launch(xs, C, B, input_global_scale, nullptr, nullptr, nullptr, w.plane, w.status, s) != 0) {
+        set_error("nvfp4 matmul: activation pass failed to launch");
+        return -1;
+    }
+    Fp4MfmaLaunch launch;
+    memset(&launch, 0, sizeof launch);
+    launch.packed = (const uint8_t *)packed; launch.scales = (const uint8_t *)scales;
+    launch.plane = w.plane; launch.ys = ys; launch.partials = w.partials; launch.status = w.status;
+    launch.rows = R; launch.cols = C; launch.tokens = B; launch.ksplit = fp4_mfma_splits(R, C, B);
+    launch.out_scale = (1.0f / stored_divisor) / input_global_scale;
+    if (fp4_mfma_launch(launch, s) != 0) { set_error("nvfp4 matmul: launch failed"); return -1; }
+    if (status_dev) {
+        if (hip_ok(hipMemcpyAsync(status_dev, w.status, 4, hipMemcpyDeviceToDevice, s), "nvfp4 matmul status copy") != 0)
+            return -1;
+        return 0;
+    }
+    int status = -1;
+    if (hip_ok(hipMemcpyAsync(&status, w.status, 4, hipMemcpyDeviceToHost, s), "nvfp4 matmul status") != 0 ||
+        hip_ok(hipStreamSynchronize(s), "nvfp4 matmul sync") != 0)
+        return -1;
+    if (status != 0) { set_error("nvfp4 matmul: non-finite activation"); return -1; }
     return 0;
 }
 

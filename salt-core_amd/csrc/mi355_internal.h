@@ -103,10 +103,25 @@ struct Fp4Launch {
 };
 
 int fp4_launch(const Fp4Launch &launch, int chains_per_lane, hipStream_t stream);
-// activation quantise/dequantise per 16-block; any of packed/scales may be null
+// activation quantise/dequantise per 16-block; any of packed/scales/dequant/plane may be null.  plane receives
+// code value * block scale as bf16 (exact), the activation operand of the matrix-core matmul.
 int fp4_qdq_launch(const float *input, int cols, int tokens, float input_global_scale,
-                   uint8_t *packed, uint8_t *scales, float *dequant, int *status,
+                   uint8_t *packed, uint8_t *scales, float *dequant, uint16_t *plane, int *status,
                    hipStream_t stream);
+
+// Prefill-sized NVFP4 matmul on the matrix cores (tolerance class): ys[token][row] =
+// out_scale * sum_c (code * block scale)[row][c] * plane[token][c].
+struct Fp4MfmaLaunch {
+    const uint8_t *packed, *scales;
+    const uint16_t *plane;    // [tokens][cols] bf16
+    float *ys;                // [tokens][rows]
+    float *partials;          // [ksplit][tokens][rows], used when ksplit > 1
+    const int *status;        // nothing is published unless *status == 0
+    int rows, cols, tokens, ksplit;
+    float out_scale;
+};
+int fp4_mfma_splits(int rows, int cols, int tokens);
+int fp4_mfma_launch(const Fp4MfmaLaunch &launch, hipStream_t stream);
 
 // ---------------------------------------------------------------- MoE
 

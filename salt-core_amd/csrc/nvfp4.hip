@@ -289,7 +289,7 @@ __device__ __forceinline__ float e2m1_decode(uint32_t code) {
 __global__ __launch_bounds__(256) void fp4_qdq_kernel(const float *__restrict__ input, int cols, int tokens,
                                                       float g, uint8_t *__restrict__ packed,
                                                       uint8_t *__restrict__ scales, float *__restrict__ dequant,
-                                                      int *__restrict__ status) {
+                                                      uint16_t *__restrict__ plane, int *__restrict__ status) {
     const int blocks_per_token = cols >> 4;
     const long long item = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (item >= (long long)blocks_per_token * tokens) return;
@@ -321,6 +321,7 @@ __global__ __launch_bounds__(256) void fp4_qdq_kernel(const float *__restrict__ 
     const float from_code = scale / g;
     uint32_t bytes[2] = {0u, 0u};
     float out[16];
+    uint32_t halves[8];                  // code value * block scale: at most six significant bits, exact in bf16
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         float s = v[i] * to_code;
@@ -328,13 +329,23 @@ __global__ __launch_bounds__(256) void fp4_qdq_kernel(const float *__restrict__ 
         if (s < -6.0f) s = -6.0f;
         const uint32_t code = e2m1_encode(s);
         bytes[i >> 3] |= code << (4 * (i & 7));
-        out[i] = e2m1_decode(code) * from_code;
+        const float value = e2m1_decode(code);
+        out[i] = value * from_code;
+        const uint32_t h = __float_as_uint(value * scale) >> 16;
+        if (i & 1) halves[i >> 1] |= h << 16; else halves[i >> 1] = h;
     }
     if (scales) scales[item] = (uint8_t)scale_code;
     if (packed) reinterpret_cast<uint2 *>(packed)[item] = make_uint2(bytes[0], bytes[1]);
-    float4 *dst = reinterpret_cast<float4 *>(dequant + item * 16);
+    if (dequant) {
+        float4 *dst = reinterpret_cast<float4 *>(dequant + item * 16);
 #pragma unroll
-    for (int q = 0; q < 4; ++q) dst[q] = make_float4(out[4 * q], out[4 * q + 1], out[4 * q + 2], out[4 * q + 3]);
+        for (int q = 0; q < 4; ++q) dst[q] = make_float4(out[4 * q], out[4 * q + 1], out[4 * q + 2], out[4 * q + 3]);
+    }
+    if (plane) {
+        uint4 *dst = reinterpret_cast<uint4 *>(plane + item * 16);
+        dst[0] = make_uint4(halves[0], halves[1], halves[2], halves[3]);
+        dst[1] = make_uint4(halves[4], halves[5], halves[6], halves[7]);
+    }
 }
 
 }  // namespace
@@ -352,12 +363,12 @@ int fp4_launch(const Fp4Launch &L, int chains_per_lane, hipStream_t stream) {
 }
 
 int fp4_qdq_launch(const float *input, int cols, int tokens, float input_global_scale, uint8_t *packed,
-                   uint8_t *scales, float *dequant, int *status, hipStream_t stream) {
+                   uint8_t *scales, float *dequant, uint16_t *plane, int *status, hipStream_t stream) {
     const long long items = (long long)(cols >> 4) * tokens;
     if (items < 1 || (cols & 15)) return -1;
     const unsigned grid = (unsigned)((items + 255) / 256);
     hipLaunchKernelGGL(fp4_qdq_kernel, dim3(grid), dim3(256), 0, stream, input, cols, tokens, input_global_scale,
-                       packed, scales, dequant, status);
+                       packed, scales, dequant, plane, status);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

@@ -69,6 +69,8 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_q4_matmul_dev, i, vp, vp, vp, i, i, i, vp, vp, vp, vp)
     _sig(lib.salt_mi355_nvfp4_qdq_dev, i, vp, i, i, f, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_nvfp4_matvec_dev, i, vp, vp, f, i, i, i, vp, vp, i, vp)
+    _sig(lib.salt_mi355_nvfp4_matmul_workspace_bytes, sz, i, i, i)
+    _sig(lib.salt_mi355_nvfp4_matmul_dev, i, vp, vp, f, f, i, i, i, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_router_topk_dev, i, vp, vp, i, i, i, vp, vp, vp, vp)
     _sig(lib.salt_mi355_moe_workspace_bytes, sz, i, i, i, i)
     _sig(lib.salt_mi355_moe_decode_step_dev, i, vp, sz, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, vp, vp)
@@ -290,3 +292,20 @@ class MoePrefill:
         check(self.lib.salt_mi355_stream_sync(stream), "sync")
         return (int(self.status.to_host(np.int32)[0]), self.out.to_host(np.float32, T * self.H).reshape(T, self.H),
                 self.group_rows.to_host(np.int32), self.row_pairs.to_host(np.int32, T * self.K))
+
+
+def nvfp4_matmul(packed: np.ndarray, scales: np.ndarray, divisor: float, input_global_scale: float, R: int, C_: int,
+                 xs: np.ndarray):
+    """Host-array convenience around salt_mi355_nvfp4_matmul_dev (MFMA, tolerance class) -> (status, ys [B][R])."""
+    lib = init()
+    xs = np.ascontiguousarray(xs, np.float32).reshape(-1, C_)
+    B = xs.shape[0]
+    dp, ds = DeviceBuffer.from_host(packed), DeviceBuffer.from_host(scales)
+    dx, dy = DeviceBuffer.from_host(xs), DeviceBuffer(B * R * 4, fill=0xFF)
+    ws = DeviceBuffer(lib.salt_mi355_nvfp4_matmul_workspace_bytes(R, C_, B))
+    status = DeviceBuffer(4, fill=0x7F)
+    stream = lib.salt_mi355_stream()
+    check(lib.salt_mi355_nvfp4_matmul_dev(dp.ptr, ds.ptr, divisor, input_global_scale, R, C_, B, dx.ptr, dy.ptr,
+                                          status.ptr, ws.ptr, stream), "nvfp4_matmul_dev")
+    check(lib.salt_mi355_stream_sync(stream), "sync")
+    return int(status.to_host(np.int32)[0]), dy.to_host(np.float32).reshape(B, R)
