@@ -44,12 +44,6 @@ __device__ __forceinline__ uniform_f32_ptr as_uniform(const float *p) {
 }
 
 constexpr int TILE_ROWS = 64;
-constexpr int CHUNK_BLOCKS = 16;                       // 32-column blocks per staged step
-constexpr int CHUNK_GROUPS = CHUNK_BLOCKS / 2;         // 64-column scale groups per step
-constexpr int W_PITCH = 16 * CHUNK_BLOCKS + 4;         // bytes per staged row: odd dword pitch
-constexpr int M_PITCH = 2 * CHUNK_GROUPS + 2;          // floats per staged row of (scale, bias)
-constexpr int W_STAGE = TILE_ROWS * W_PITCH;
-constexpr int M_STAGE = TILE_ROWS * M_PITCH;
 constexpr int FOLD_PITCH = 33;
 constexpr float BIG_SCALE = 0x1p118f;
 
@@ -142,8 +136,18 @@ constexpr int x_batch_groups(int S, int NB) {
     return fit >= 8 ? 8 : fit >= 4 ? 4 : fit >= 2 ? 2 : 1;
 }
 
-template <int S, int NB, bool FUSED>
+// CB = 32-column blocks staged per step.  16 keeps the tile's LDS small enough
+// for three workgroups per compute unit; 32 is for launches with too few tiles
+// to share a compute unit, where the amount of data in flight per workgroup is
+// what hides the memory latency.
+template <int S, int NB, bool FUSED, int CB>
 __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L) {
+    constexpr int CHUNK_BLOCKS = CB;
+    constexpr int CHUNK_GROUPS = CB / 2;                   // 64-column scale groups per step
+    constexpr int W_PITCH = 16 * CB + 4;                   // bytes per staged row: odd dword pitch
+    constexpr int M_PITCH = 2 * CHUNK_GROUPS + 2;          // floats per staged row of (scale, bias)
+    constexpr int W_STAGE = TILE_ROWS * W_PITCH;
+    constexpr int M_STAGE = TILE_ROWS * M_PITCH;
     constexpr int WAVES = 32 / S;
     constexpr int THREADS = WAVES * 64;
     constexpr int PIECES = (TILE_ROWS * CHUNK_BLOCKS) / THREADS;              // 16-byte pieces per thread
@@ -181,27 +185,27 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
     // Per-thread staging geometry, fixed for the whole tile.  Piece i of a
     // thread lies (THREADS / 16) rows below piece 0 in the same 16-byte column,
     // so only the clamped source row offsets need registers.
-    constexpr int W_ROW_STEP = THREADS / 16, M_ROW_STEP = THREADS / 8;
-    const uint32_t w_seg = tid & 15;
-    const uint32_t w_dst0 = (tid >> 4) * W_PITCH + w_seg * 16;
+    constexpr int W_ROW_STEP = THREADS / CHUNK_BLOCKS, M_ROW_STEP = THREADS / CHUNK_GROUPS;
+    const uint32_t w_seg = tid % CHUNK_BLOCKS;
+    const uint32_t w_dst0 = (tid / CHUNK_BLOCKS) * W_PITCH + w_seg * 16;
     uint32_t w_src[PIECES];
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
-        const int row = (tid >> 4) + i * W_ROW_STEP;
+        const int row = (tid / CHUNK_BLOCKS) + i * W_ROW_STEP;
         w_src[i] = (uint32_t)(row < rows_here ? row : rows_here - 1) * row_bytes;
     }
     const bool has_meta = tid < TILE_ROWS * CHUNK_GROUPS;    // only narrower than the block when THREADS == 1024
-    const uint32_t m_grp = tid & 7;
-    const uint32_t m_dst0 = ((tid >> 3) & (TILE_ROWS - 1)) * M_PITCH + 2 * m_grp;
+    const uint32_t m_grp = tid % CHUNK_GROUPS;
+    const uint32_t m_dst0 = ((tid / CHUNK_GROUPS) & (TILE_ROWS - 1)) * M_PITCH + 2 * m_grp;
     uint32_t m_src[META_ITEMS];
 #pragma unroll
     for (int i = 0; i < META_ITEMS; ++i) {
-        const int row = ((tid >> 3) + i * M_ROW_STEP) & (TILE_ROWS - 1);
+        const int row = ((tid / CHUNK_GROUPS) + i * M_ROW_STEP) & (TILE_ROWS - 1);
         m_src[i] = (uint32_t)(row < rows_here ? row : rows_here - 1) * ngrp;
     }
 
     u32x4 wreg[PIECES];
-    uint32_t mreg[META_ITEMS];
+    uint32_t sreg[META_ITEMS], breg[META_ITEMS];     // raw bf16 bits; nothing may consume them before commit
 
     // Loads of step ck into registers.  Block and group indices past the end
     // of the row (last step only) are clamped: the data is staged but never
@@ -218,9 +222,8 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
             int g = ck * CHUNK_GROUPS + (int)m_grp;
             g = g < ngrp ? g : ngrp - 1;
             const uint32_t at = m_src[i] + (uint32_t)g;
-            const uint32_t sbits = scales16[at];
-            const uint32_t bbits = biases16 ? (uint32_t)biases16[at] : 0u;
-            mreg[i] = sbits | (bbits << 16);
+            sreg[i] = scales16[at];
+            breg[i] = biases16 ? (uint32_t)biases16[at] : 0u;
         }
     };
 
@@ -233,8 +236,8 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
         if (has_meta) {
 #pragma unroll
             for (int i = 0; i < META_ITEMS; ++i) {
-                const float sc = bf16_to_f32(mreg[i] & 0xFFFFu);
-                const float bi = __uint_as_float(mreg[i] & 0xFFFF0000u);
+                const float sc = bf16_to_f32(sreg[i]);
+                const float bi = bf16_to_f32(breg[i]);
                 if (!(__builtin_fabsf(sc) < BIG_SCALE)) slow_flag = 1;
                 float *dst = m_lds + stage * M_STAGE + m_dst0 + i * M_ROW_STEP * M_PITCH;
                 dst[0] = sc * L.code_scale;
@@ -323,8 +326,28 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
                 }
             }
         } else {
-            // Partial last step, or a tile that met an out-of-range scale.
-            for (int g = 0; g < gcount; ++g) {
+            // Partial last step, or a tile that met an out-of-range scale:
+            // whole activation batches first, then single groups.
+            int g = 0;
+            if (!slow) {
+                for (; g + XG <= gcount; g += XG) {
+                    load_x(ck * CHUNK_GROUPS + g, xq, XG);
+#pragma unroll
+                    for (int gl = 0; gl < XG; ++gl) {
+                        uint32_t w0, w1;
+                        float scale, bias;
+                        fetch(g + gl, w0, w1, scale, bias);
+                        if (S == 8) {
+                            consume_word<S, NB, XN, 8, false, FUSED>(w0, 0, gl * 2 * S, scale, bias, xq, L.code_scale, acc);
+                            consume_word<S, NB, XN, 8, false, FUSED>(w1, 1, gl * 2 * S, scale, bias, xq, L.code_scale, acc);
+                        } else {
+                            consume_word<S, NB, XN, (S == 4 ? 8 : 4), false, FUSED>(w0, 0, gl * 2 * S, scale, bias, xq,
+                                                                                     L.code_scale, acc);
+                        }
+                    }
+                }
+            }
+            for (; g < gcount; ++g) {
                 uint32_t w0, w1;
                 float scale, bias;
                 fetch(g, w0, w1, scale, bias);
@@ -428,14 +451,30 @@ __global__ __launch_bounds__(256) void q4_generic_kernel(const Q4Launch L) {
     }
 }
 
+// Launches of at most this many tiles use the wide-step variant (tuning: SALT_MI355_Q4_WIDE_TILES).
+int env_wide_limit() {
+    static int cached = -1;
+    if (cached < 0) {
+        const char *e = getenv("SALT_MI355_Q4_WIDE_TILES");
+        cached = e ? atoi(e) : 256;
+        if (cached < 0) cached = 0;
+    }
+    return cached;
+}
+
 template <int S, bool FUSED>
 int launch_tiles(const Q4Launch &L, hipStream_t stream) {
     const dim3 grid(L.total_tiles), block((32 / S) * 64);
+    // One token with few tiles: a workgroup has its compute unit to itself and stages twice as much per step.
+    if (L.tokens == 1 && !FUSED && S <= 4 && L.total_tiles <= env_wide_limit()) {
+        hipLaunchKernelGGL((q4_tile_kernel<S, 1, false, 32>), grid, block, 0, stream, L);
+        return hipGetLastError() == hipSuccess ? 0 : -1;
+    }
     switch (L.tokens) {
-        case 1: hipLaunchKernelGGL((q4_tile_kernel<S, 1, FUSED>), grid, block, 0, stream, L); break;
-        case 2: hipLaunchKernelGGL((q4_tile_kernel<S, 2, FUSED>), grid, block, 0, stream, L); break;
-        case 3: hipLaunchKernelGGL((q4_tile_kernel<S, 3, FUSED>), grid, block, 0, stream, L); break;
-        case 4: hipLaunchKernelGGL((q4_tile_kernel<S, 4, FUSED>), grid, block, 0, stream, L); break;
+        case 1: hipLaunchKernelGGL((q4_tile_kernel<S, 1, FUSED, 16>), grid, block, 0, stream, L); break;
+        case 2: hipLaunchKernelGGL((q4_tile_kernel<S, 2, FUSED, 16>), grid, block, 0, stream, L); break;
+        case 3: hipLaunchKernelGGL((q4_tile_kernel<S, 3, FUSED, 16>), grid, block, 0, stream, L); break;
+        case 4: hipLaunchKernelGGL((q4_tile_kernel<S, 4, FUSED, 16>), grid, block, 0, stream, L); break;
         default: return -1;
     }
     return hipGetLastError() == hipSuccess ? 0 : -1;
