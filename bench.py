@@ -32,6 +32,7 @@ import numpy as np
 ROOT = Path(__file__).resolve().parent
 sys.path[:0] = [str(ROOT), str(ROOT / "tests")]
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
 SWEEP = [(2816, 2816), (16384, 2816), (2816, 8192)]        # (R, C) = (N, K)
 INSTANCE_BYTES = 640e6                                      # distinct weight bytes per launch
@@ -235,6 +236,39 @@ def main():
         ms_fp4 = timed(lib, stream, events, fp4_step, 2, 10) / G
         extra["nvfp4_8192_matvec_us"] = round(ms_fp4 * 1e3, 2)
         extra["nvfp4_8192_gbps"] = round(synth.nvfp4_bytes(R, Cc, 1) / (ms_fp4 * 1e-3) / 1e9, 1)
+        # NVFP4 8192 x 8192, batch 256, on the matrix cores (tolerance class); activation pass included
+        B = 256
+        xb = gpu.DeviceBuffer.from_host(synth.activations(Cc, B, 42))
+        yb = gpu.DeviceBuffer(B * R * 4)
+        wsb = gpu.DeviceBuffer(lib.salt_mi355_nvfp4_matmul_workspace_bytes(R, Cc, B))
+
+        def fp4_matmul_step(s):
+            if lib.salt_mi355_nvfp4_matmul_dev(w.at(0), w.at(packed.nbytes), 2688.0, 64.0, R, Cc, B, xb.ptr, yb.ptr,
+                                               st.ptr, wsb.ptr, s) != 0:
+                raise RuntimeError(lib.salt_mi355_last_error().decode())
+
+        ms_mm = timed(lib, stream, events, fp4_matmul_step, 2, 20)
+        extra["nvfp4_8192_b256_matmul_us"] = round(ms_mm * 1e3, 2)
+        extra["nvfp4_8192_b256_tflops"] = round(2.0 * R * Cc * B / (ms_mm * 1e-3) / 1e12, 1)
+        extra["nvfp4_8192_b256_mfma_frac"] = round(2.0 * R * Cc * B / (ms_mm * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
+        del w, xb, yb, wsb
+        # MoE prefill, 2048 tokens through one layer (E = 128, top-8, Zipf 1.1), grouped per expert, matrix cores
+        T = 2048
+        sel, wts = synth.zipf_selection(T, E, K, 1.1, 60)
+        prefill = gpu.MoePrefill(pool, E, H, F, K, T)
+        prefill.sel.upload(sel); prefill.w.upload(wts); prefill.x.upload(synth.activations(H, T, 61))
+
+        def prefill_step(s):
+            if prefill.enqueue(s) != 0:
+                raise RuntimeError(lib.salt_mi355_last_error().decode())
+
+        ms_pf = timed(lib, stream, events, prefill_step, 2, 10)
+        flops = 2.0 * T * K * 3 * H * F                       # useful: one pass over the weights per routed row
+        extra["moe_prefill_2048_us"] = round(ms_pf * 1e3, 1)
+        extra["moe_prefill_tokens_per_s"] = round(T / (ms_pf * 1e-3), 0)
+        extra["moe_prefill_useful_tflops"] = round(flops / (ms_pf * 1e-3) / 1e12, 1)
+        # the activation travels as three exact bf16 planes, so the matrix cores execute three times the useful flops
+        extra["moe_prefill_mfma_frac"] = round(3 * flops / (ms_pf * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
         result["extra"] = extra
 
     if not args.no_cpu:

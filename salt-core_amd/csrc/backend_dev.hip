@@ -36,7 +36,7 @@ int salt_mi355_q4_matmul_dev(const void *vals, const void *scales, const void *b
     launch.one.planes = planes; launch.one.xsum = xsum; launch.one.y = ys;
     launch.one.tokens = B; launch.one.rows = R;
     launch.njobs = 1; launch.cols = C; launch.plane_stride = plane_stride;
-    launch.total_tiles = mfma_tiles(B, R);
+    launch.blocks_per_wave = 0;                  // the launcher picks the tile width and counts the tiles
     if (q4_mfma_launch(launch, (hipStream_t)stream) != 0) { set_error("q4 matmul: launch failed"); return -1; }
     return 0;
 }

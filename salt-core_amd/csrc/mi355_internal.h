@@ -49,7 +49,7 @@ int q4_assign_tiles(Q4Job *table, int njobs);
 
 // One weight matrix against `tokens` activation rows that have been split
 // into three bf16 planes (x = hi + mid + lo) with per-64-column sums.
-constexpr int MFMA_TM = 64, MFMA_TN = 128;   // tokens x weight rows per workgroup of the matrix-core kernel
+constexpr int MFMA_TM = 64;   // tokens per workgroup of the matrix-core kernel; its weight rows: mfma_tile_rows()
 
 struct MfmaJob {
     const uint8_t *vals, *scales, *biases;   // biases may be null
@@ -59,7 +59,7 @@ struct MfmaJob {
     int tokens;
     int rows;
     int tile0;
-    int reserved;
+    int row_base;             // with a row map: index of this job's first token in the map
 };
 
 struct MfmaLaunch {
@@ -71,10 +71,15 @@ struct MfmaLaunch {
     size_t plane_stride;      // elements between planes
     const int *njobs_dev;     // optional: job and tile counts produced by an earlier kernel;
     const int *total_tiles_dev;   // workgroups past *total_tiles_dev exit at once
+    const int *row_map;       // optional gather: token t of a job reads plane row row_map[row_base + t] / map_divisor
+    int map_divisor;
+    int blocks_per_wave;      // the tile is 64 tokens x 64 * blocks_per_wave rows (mfma_blocks_per_wave()); 0 = choose (single job only)
 };
 
 int q4_mfma_launch(const MfmaLaunch &launch, hipStream_t stream);
-int mfma_tiles(int tokens, int rows);
+int mfma_tile_rows(int blocks_per_wave);
+int mfma_tiles(int tokens, int rows, int blocks_per_wave);
+int mfma_blocks_per_wave(long long wide_tiles);
 // rows of fp32 -> bf16 planes + group sums; output row r reads input row row_map[r] / map_divisor when a map is
 // given; with a gate the value split is gelu_tanh(gate) * x (gate has the layout of x)
 int x_split_launch(const float *x, const float *gate, const int *row_map, int map_divisor, int x_stride, int rows,

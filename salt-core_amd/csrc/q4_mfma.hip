@@ -46,16 +46,20 @@ typedef const u32x4 __attribute__((address_space(1))) *global_u128_ptr;
 typedef const uint16_t __attribute__((address_space(1))) *global_u16_ptr;
 typedef const float __attribute__((address_space(1))) *global_f32_ptr;
 
-constexpr int TM = MFMA_TM, TN = MFMA_TN;   // tokens x weight rows per workgroup
+constexpr int TM = MFMA_TM;                 // tokens per workgroup; weight rows per workgroup: 64 * NBW
 constexpr int X_PITCH = 144;               // bytes per staged token row of one plane: 64 bf16 + 16 pad
 constexpr int W_PITCH = 36;                // bytes per staged weight row of one group: 32 + 4 pad
-constexpr int XS_BYTES = 3 * TM * X_PITCH, WS_BYTES = TN * W_PITCH;
-constexpr int SC_OFF = XS_BYTES + WS_BYTES;                 // float scale[TN]
-constexpr int STAGE_BYTES = (SC_OFF + TN * 4 + 15) & ~15;
-// bias pass (before the main loop, in the same LDS): 16 groups per step
-constexpr int G_PITCH = 48;                // bytes per staged row of 16 bf16: 32 + 16 pad
-constexpr int XG_BYTES = 3 * TM * G_PITCH, BS_BYTES = 2 * TN * G_PITCH;
-static_assert(XG_BYTES + BS_BYTES <= 2 * STAGE_BYTES, "the bias pass reuses the staging memory");
+constexpr int XS_BYTES = 3 * TM * X_PITCH;
+constexpr int G_PITCH = 48;                // bias pass: bytes per staged row of 16 bf16: 32 + 16 pad
+constexpr int XG_BYTES = 3 * TM * G_PITCH;
+
+// LDS layout of one stage for a tile of TN weight rows
+template <int TN> struct Stage {
+    static constexpr int WS_OFF = XS_BYTES;                        // codes [TN][W_PITCH]
+    static constexpr int SC_OFF = WS_OFF + TN * W_PITCH;           // float scale[TN]
+    static constexpr int BYTES = (SC_OFF + TN * 4 + 15) & ~15;
+    static_assert(XG_BYTES + 2 * TN * G_PITCH <= 2 * BYTES, "the bias pass reuses the staging memory");
+};
 
 static_assert(sizeof(MfmaJob) == 64, "find_job reads a job record as eight 64-bit words");
 
@@ -79,7 +83,7 @@ __device__ __forceinline__ MfmaJob find_job(const MfmaLaunch &L, int tile) {
     job.tokens = (int)(uint32_t)rec[6];
     job.rows = (int)(rec[6] >> 32);
     job.tile0 = (int)(uint32_t)rec[7];
-    job.reserved = 0;
+    job.row_base = (int)(rec[7] >> 32);
     return job;
 }
 
@@ -118,49 +122,70 @@ __device__ __forceinline__ void split3(float v, uint32_t &h, uint32_t &m, uint32
 }
 
 // One scale group of one wave: NB blocks of 32 rows against the wave's 32 tokens.
-template <int NB>
-__device__ __forceinline__ void group_product(const uint8_t *cur, int wm, int wn, int l32, int half, f32x16 (&acc)[2]) {
+template <int NB, int NBW>
+__device__ __forceinline__ void group_product(const uint8_t *cur, int wm, int wn, int l32, int half,
+                                              f32x16 (&acc)[NBW]) {
+    using S = Stage<64 * NBW>;
     const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    f32x16 part[NB];
     uint32_t sixteen;                                   // two bf16 values 16.0, kept in a vector register
     asm("v_mov_b32 %0, 0x41804180" : "=v"(sixteen));
-    const uint8_t *wrow = cur + XS_BYTES + (wn * 64 + l32) * W_PITCH + half * 4;
+    const uint8_t *wrow = cur + S::WS_OFF + (wn * 32 * NBW + l32) * W_PITCH + half * 4;
     const uint8_t *xrow = cur + (wm * 32 + l32) * X_PITCH + half * 16;
+    const float *sc = reinterpret_cast<const float *>(cur + S::SC_OFF) + wn * 32 * NBW + l32;
+    // The token operand of the whole group stays in registers; the row blocks
+    // then run two at a time so that only two partial products are live.
+    bf16x8 a[4][3];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-        bf16x8 a[3], b[NB];
-#pragma unroll
-        for (int plane = 0; plane < 3; ++plane)
-            a[plane] = __builtin_bit_cast(bf16x8,
-                                          *reinterpret_cast<const u32x4 *>(xrow + plane * (TM * X_PITCH) + ks * 32));
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-            b[nb] = codes_to_bf16(*reinterpret_cast<const uint32_t *>(wrow + nb * 32 * W_PITCH + ks * 8), 0x00780078u,
-                                  sixteen);
+    for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
         for (int plane = 0; plane < 3; ++plane)
+            a[ks][plane] = __builtin_bit_cast(
+                bf16x8, *reinterpret_cast<const u32x4 *>(xrow + plane * (TM * X_PITCH) + ks * 32));
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
-                part[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[plane], b[nb], (ks | plane) ? part[nb] : zero, 0, 0, 0);
-    }
-    const float *sc = reinterpret_cast<const float *>(cur + SC_OFF) + wn * 64 + l32;
+    for (int nb0 = 0; nb0 < NB; nb0 += 2) {
+        constexpr int PAIR_MAX = 2;
+        const int pair = NB - nb0 < PAIR_MAX ? NB - nb0 : PAIR_MAX;
+        f32x16 part[PAIR_MAX];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-        const float s = sc[nb * 32];
+        for (int ks = 0; ks < 4; ++ks) {
+            bf16x8 b[PAIR_MAX];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[nb][i] = __builtin_fmaf(s, part[nb][i], acc[nb][i]);
+            for (int k = 0; k < PAIR_MAX; ++k)
+                if (k < pair)
+                    b[k] = codes_to_bf16(*reinterpret_cast<const uint32_t *>(wrow + (nb0 + k) * 32 * W_PITCH + ks * 8),
+                                         0x00780078u, sixteen);
+#pragma unroll
+            for (int plane = 0; plane < 3; ++plane)
+#pragma unroll
+                for (int k = 0; k < PAIR_MAX; ++k)
+                    if (k < pair)
+                        part[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks][plane], b[k],
+                                                                          (ks | plane) ? part[k] : zero, 0, 0, 0);
+        }
+#pragma unroll
+        for (int k = 0; k < PAIR_MAX; ++k)
+            if (k < pair) {
+                const float s = sc[(nb0 + k) * 32];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[nb0 + k][i] = __builtin_fmaf(s, part[k][i], acc[nb0 + k][i]);
+            }
     }
 }
 
+// NBW = 32-row blocks per wave: the workgroup's tile is 64 tokens x 64 * NBW rows.
+template <int NBW>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 void q4_mfma_kernel(const MfmaLaunch L) {
-    // two stages of { planes [3][64 tokens], codes [128 rows], scales [128] }
+    constexpr int TN = 64 * NBW;
+    using S = Stage<TN>;
+    constexpr int STAGE_BYTES = S::BYTES;
+    // two stages of { planes [3][64 tokens], codes [TN rows], scales [TN] }
     __shared__ __attribute__((aligned(16))) uint8_t stage[2 * STAGE_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;       // wave tile: tokens wm*32.., rows wn*64.. (two 32-row blocks)
+    const int wm = wave >> 1, wn = wave & 1;       // wave tile: tokens wm*32.., rows wn*32*NBW.. (NBW 32-row blocks)
     const int l32 = lane & 31, half = lane >> 5;
 
     if (L.total_tiles_dev &&
@@ -174,134 +199,165 @@ void q4_mfma_kernel(const MfmaLaunch L) {
     const int toks_here = job.tokens - tok0 < TM ? job.tokens - tok0 : TM;
     const int rows_here = job.rows - row0 < TN ? job.rows - row0 : TN;
 
+    // Token t of the job is row (tok0 + t) of the planes, or, with a map, row
+    // row_map[row_base + tok0 + t] / map_divisor (the grouped MoE gather).
+    const int *row_map = L.row_map;
+    auto source_row = [&](int tok) -> uint32_t {
+        const int tc = tok < toks_here ? tok : toks_here - 1;
+        return row_map ? (uint32_t)(row_map[job.row_base + tok0 + tc] / L.map_divisor) : (uint32_t)(tok0 + tc);
+    };
+
     // staging geometry of this thread
     // planes: 3 * 64 tokens * 8 segments of 16 bytes = 1536 pieces, 6 per thread
     const global_u16_ptr planes = (global_u16_ptr)(uintptr_t)job.planes;
-    uint32_t x_src[6], x_dst[6];
+    uint32_t x_src[6], x_dst[6];                    // element offsets: the planes of one launch stay below 2^32 elements
 #pragma unroll
     for (int i = 0; i < 6; ++i) {
         const int p = tid + i * 256;
         const int plane = p >> 9, tok = (p >> 3) & 63, seg = p & 7;
-        const int tc = tok < toks_here ? tok : toks_here - 1;
-        x_src[i] = (uint32_t)(tok0 + tc) * (uint32_t)C + seg * 8;          // element offset inside the plane
+        x_src[i] = (uint32_t)plane * (uint32_t)L.plane_stride + source_row(tok) * (uint32_t)C + seg * 8;
         x_dst[i] = plane * (TM * X_PITCH) + tok * X_PITCH + seg * 16;
     }
-    const size_t plane_stride = L.plane_stride;
-    // codes: 128 rows * 2 pieces of 16 bytes, one per thread
-    const int w_row = tid >> 1, w_half = tid & 1;
-    const int w_rc = w_row < rows_here ? w_row : rows_here - 1;
-    const global_u128_ptr w_src = (global_u128_ptr)((uintptr_t)job.vals + (size_t)(row0 + w_rc) * (C >> 1) + w_half * 16);
-    // scales: threads 0..127
-    const int m_row = tid & 127;
+    // codes: TN rows * 2 pieces of 16 bytes, NBW / 2 per thread
+    constexpr int WP = NBW / 2;
+    const int w_half = tid & 1;
+    global_u128_ptr w_src[WP];
+    uint32_t w_dst[WP];
+#pragma unroll
+    for (int i = 0; i < WP; ++i) {
+        const int row = (tid >> 1) + i * 128;
+        const int rc = row < rows_here ? row : rows_here - 1;
+        w_src[i] = (global_u128_ptr)((uintptr_t)job.vals + (size_t)(row0 + rc) * (C >> 1) + w_half * 16);
+        w_dst[i] = S::WS_OFF + row * W_PITCH + w_half * 16;
+    }
+    // scales: threads 0..TN-1
+    const int m_row = tid & (TN - 1);
     const int m_rc = m_row < rows_here ? m_row : rows_here - 1;
     const global_u16_ptr scales = (global_u16_ptr)(uintptr_t)job.scales + (size_t)(row0 + m_rc) * ngrp;
 
-    u32x4 xreg[6], wreg;
-    uint32_t sreg = 0;
-    auto issue = [&](int g) {
+    // Loads travel through registers; two sets are in flight so that a load has
+    // two groups of matrix work (of both workgroups on the compute unit) to land.
+    struct Loads { u32x4 x[6], w[WP]; uint32_t s; };
+    auto issue = [&](int g, Loads &r) {
 #pragma unroll
-        for (int i = 0; i < 6; ++i) {
-            const int plane = (tid + i * 256) >> 9;
-            xreg[i] = *(global_u128_ptr)(planes + (size_t)plane * plane_stride + x_src[i] + (uint32_t)g * 64u);
+        for (int i = 0; i < 6; ++i) r.x[i] = *(global_u128_ptr)(planes + x_src[i] + (uint32_t)g * 64u);
+#pragma unroll
+        for (int i = 0; i < WP; ++i) r.w[i] = w_src[i][g * 2];
+        if (tid < TN) r.s = scales[g];
+    };
+    auto commit = [&](uint8_t *base, const Loads &r) {
+#pragma unroll
+        for (int i = 0; i < 6; ++i) *reinterpret_cast<u32x4 *>(base + x_dst[i]) = r.x[i];
+#pragma unroll
+        for (int i = 0; i < WP; ++i) {
+            uint32_t *dst = reinterpret_cast<uint32_t *>(base + w_dst[i]);
+            dst[0] = r.w[i].x; dst[1] = r.w[i].y; dst[2] = r.w[i].z; dst[3] = r.w[i].w;
         }
-        wreg = w_src[g * 2];
-        if (tid < 128) sreg = scales[g];
+        if (tid < TN) reinterpret_cast<float *>(base + S::SC_OFF)[m_row] = bf16_to_f32(r.s);
     };
-    auto commit = [&](uint8_t *base) {
-#pragma unroll
-        for (int i = 0; i < 6; ++i) *reinterpret_cast<u32x4 *>(base + x_dst[i]) = xreg[i];
-        uint32_t *dst = reinterpret_cast<uint32_t *>(base + XS_BYTES + w_row * W_PITCH + w_half * 16);
-        dst[0] = wreg.x; dst[1] = wreg.y; dst[2] = wreg.z; dst[3] = wreg.w;
-        if (tid < 128) reinterpret_cast<float *>(base + SC_OFF)[m_row] = bf16_to_f32(sreg);
-    };
-
-    // a wave whose second (or both) 32-row blocks lie past the matrix skips their matrix work
-    const int nblocks = rows_here - wn * 64 <= 0 ? 0 : (rows_here - wn * 64 <= 32 ? 1 : 2);
 
     const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    f32x16 acc[2] = {zero, zero};
+    f32x16 acc[NBW];
+#pragma unroll
+    for (int nb = 0; nb < NBW; ++nb) acc[nb] = zero;
 
     // ---- bias pass: acc[tok][row] = sum_g (b[row][g] - 16 s[row][g]) * X[tok][g]
     {
         const global_f32_ptr xsum = (global_f32_ptr)(uintptr_t)job.xsum;
         const int xg_tok = tid >> 2, xg_g = (tid & 3) * 4;
-        const int xg_tc = xg_tok < toks_here ? xg_tok : toks_here - 1;
-        const int bs_arr = tid >> 7;                            // 0: biases, 1: scales
-        const global_u16_ptr bs_src = bs_arr ? scales : (job.biases ? (global_u16_ptr)(uintptr_t)job.biases +
-                                                                          (size_t)(row0 + m_rc) * ngrp
-                                                                    : (global_u16_ptr)0);
-        f32x16 tb[2] = {zero, zero}, ts[2] = {zero, zero};
-        for (int g0 = 0; g0 < ngrp; g0 += 16) {
-            uint32_t h[4], m[4], l[4];
+        const size_t xg_row = (size_t)source_row(xg_tok) * ngrp;
+        const global_u16_ptr all_scales = (global_u16_ptr)(uintptr_t)job.scales;
+        const global_u16_ptr all_biases = (global_u16_ptr)(uintptr_t)job.biases;
+        // Two 32-row blocks per pass keep the four partial products in registers.
+#pragma unroll 1
+        for (int pass = 0; pass < NBW / 2; ++pass) {
+            f32x16 tb[2] = {zero, zero}, ts[2] = {zero, zero};
+            for (int g0 = 0; g0 < ngrp; g0 += 16) {
+                uint32_t h[4], m[4], l[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int g = g0 + xg_g + j;
-                const float v = g < ngrp ? xsum[(size_t)(tok0 + xg_tc) * ngrp + g] : 0.0f;
-                split3(v, h[j], m[j], l[j]);
-            }
-            uint32_t bs[8];
+                for (int j = 0; j < 4; ++j) {
+                    const int g = g0 + xg_g + j;
+                    const float v = g < ngrp ? xsum[xg_row + g] : 0.0f;
+                    split3(v, h[j], m[j], l[j]);
+                }
+                __syncthreads();                                // the previous step's operands have been read
+                uint8_t *xgp = stage + xg_tok * G_PITCH + xg_g * 2;
+                *reinterpret_cast<uint2 *>(xgp) = make_uint2(h[0] | h[1] << 16, h[2] | h[3] << 16);
+                *reinterpret_cast<uint2 *>(xgp + TM * G_PITCH) = make_uint2(m[0] | m[1] << 16, m[2] | m[3] << 16);
+                *reinterpret_cast<uint2 *>(xgp + 2 * TM * G_PITCH) = make_uint2(l[0] | l[1] << 16, l[2] | l[3] << 16);
+                // (bias, scale) bits of 16 groups for every row of the tile: item = array * TN + row
+                for (int item = tid; item < 2 * TN; item += 256) {
+                    const int arr = item / TN, row = item % TN;
+                    const int rc = row < rows_here ? row : rows_here - 1;
+                    const global_u16_ptr src = (arr ? all_scales : all_biases) + (size_t)(row0 + rc) * ngrp;
+                    const bool present = arr || job.biases;
+                    uint32_t *bsp = reinterpret_cast<uint32_t *>(stage + XG_BYTES + item * G_PITCH);
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const int g = g0 + j;
-                const uint32_t v = (g < ngrp && bs_src) ? (uint32_t)bs_src[g] : 0u;
-                if (j & 1) bs[j >> 1] |= v << 16; else bs[j >> 1] = v;
-            }
-            __syncthreads();                                    // the previous step's operands have been read
-            uint8_t *xgp = stage + xg_tok * G_PITCH + xg_g * 2;
-            *reinterpret_cast<uint2 *>(xgp) = make_uint2(h[0] | h[1] << 16, h[2] | h[3] << 16);
-            *reinterpret_cast<uint2 *>(xgp + TM * G_PITCH) = make_uint2(m[0] | m[1] << 16, m[2] | m[3] << 16);
-            *reinterpret_cast<uint2 *>(xgp + 2 * TM * G_PITCH) = make_uint2(l[0] | l[1] << 16, l[2] | l[3] << 16);
-            uint32_t *bsp = reinterpret_cast<uint32_t *>(stage + XG_BYTES + (bs_arr * TN + m_row) * G_PITCH);
+                    for (int j = 0; j < 8; ++j) {
+                        const int g = g0 + 2 * j;
+                        const uint32_t lo = (present && g < ngrp) ? (uint32_t)src[g] : 0u;
+                        const uint32_t hi = (present && g + 1 < ngrp) ? (uint32_t)src[g + 1] : 0u;
+                        bsp[j] = lo | hi << 16;
+                    }
+                }
+                __syncthreads();
+                {
+                    const uint8_t *arow = stage + (wm * 32 + l32) * G_PITCH + half * 16;
+                    const uint8_t *brow = stage + XG_BYTES + (wn * 32 * NBW + pass * 64 + l32) * G_PITCH + half * 16;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) bsp[j] = bs[j];
-            __syncthreads();
-            if (nblocks > 0) {
-                const uint8_t *arow = stage + (wm * 32 + l32) * G_PITCH + half * 16;
-                const uint8_t *brow = stage + XG_BYTES + (wn * 64 + l32) * G_PITCH + half * 16;
+                    for (int plane = 0; plane < 3; ++plane) {
+                        const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(arow + plane * TM * G_PITCH));
 #pragma unroll
-                for (int plane = 0; plane < 3; ++plane) {
-                    const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(arow + plane * TM * G_PITCH));
-#pragma unroll
-                    for (int nb = 0; nb < 2; ++nb) {
-                        const bf16x8 bb = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(brow + nb * 32 * G_PITCH));
-                        const bf16x8 sb = __builtin_bit_cast(
-                            bf16x8, *reinterpret_cast<const u32x4 *>(brow + (TN + nb * 32) * G_PITCH));
-                        tb[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bb, tb[nb], 0, 0, 0);
-                        ts[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, sb, ts[nb], 0, 0, 0);
+                        for (int nb = 0; nb < 2; ++nb) {
+                            const bf16x8 bb = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(brow + nb * 32 * G_PITCH));
+                            const bf16x8 sb = __builtin_bit_cast(
+                                bf16x8, *reinterpret_cast<const u32x4 *>(brow + (TN + nb * 32) * G_PITCH));
+                            tb[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bb, tb[nb], 0, 0, 0);
+                            ts[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, sb, ts[nb], 0, 0, 0);
+                        }
                     }
                 }
             }
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float v = __builtin_fmaf(-16.0f, ts[nb][i], tb[nb][i]);
+                    if (NBW == 2 || pass == 0) acc[nb][i] = v; else acc[(NBW > 2 ? 2 : 0) + nb][i] = v;
+                }
         }
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) acc[nb][i] = __builtin_fmaf(-16.0f, ts[nb][i], tb[nb][i]);
         __syncthreads();
     }
 
     // ---- main loop: acc += s[row][g] * sum_{c in g} (16 + q[row][c]) * x[tok][c]
-    // The loop exists once per block count so that the accumulators stay in place.
-    auto main_loop = [&](auto block_count) {
-        constexpr int NB = decltype(block_count)::value;
-        issue(0);
-        commit(stage);
+    // Row blocks past the end of the matrix are computed on clamped rows and
+    // dropped at the store: one instantiation of the loop keeps the
+    // accumulators in place and the register count inside the budget.
+    {
+        Loads even, odd;
+        even.s = 0; odd.s = 0;
+        uint8_t *stage0 = stage, *stage1 = stage + STAGE_BYTES;
+        issue(0, even);
+        if (ngrp > 1) issue(1, odd);
+        commit(stage0, even);
         __syncthreads();
-        for (int g = 0; g < ngrp; ++g) {
-            const uint8_t *cur = stage + (g & 1) * STAGE_BYTES;
-            if (g + 1 < ngrp) issue(g + 1);
-            if (NB > 0) group_product<(NB > 0 ? NB : 1)>(cur, wm, wn, l32, half, acc);
-            if (g + 1 < ngrp) commit(stage + ((g + 1) & 1) * STAGE_BYTES);
+        for (int g = 0; g < ngrp; g += 2) {
+            if (g + 2 < ngrp) issue(g + 2, even);
+            group_product<NBW, NBW>(stage0, wm, wn, l32, half, acc);
+            if (g + 1 < ngrp) commit(stage1, odd);
+            __syncthreads();
+            if (g + 1 >= ngrp) break;
+            if (g + 3 < ngrp) issue(g + 3, odd);
+            group_product<NBW, NBW>(stage1, wm, wn, l32, half, acc);
+            if (g + 2 < ngrp) commit(stage0, even);
             __syncthreads();
         }
-    };
-    if (nblocks == 2) main_loop(std::integral_constant<int, 2>{});
-    else if (nblocks == 1) main_loop(std::integral_constant<int, 1>{});
-    else main_loop(std::integral_constant<int, 0>{});
+    }
 
     float __attribute__((address_space(1))) *y = (float __attribute__((address_space(1))) *)(uintptr_t)job.y;
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
-        const int row = wn * 64 + nb * 32 + l32;
+    for (int nb = 0; nb < NBW; ++nb) {
+        const int row = wn * 32 * NBW + nb * 32 + l32;
         if (row < rows_here) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
@@ -367,9 +423,34 @@ __global__ __launch_bounds__(256) void x_split_kernel(const float *__restrict__ 
 
 }  // namespace
 
-int q4_mfma_launch(const MfmaLaunch &L, hipStream_t stream) {
-    if (L.total_tiles < 1 || L.cols < 64 || (L.cols & 63)) return -1;
-    hipLaunchKernelGGL(q4_mfma_kernel, dim3(L.total_tiles), dim3(256), 0, stream, L);
+int mfma_tile_rows(int blocks_per_wave) { return 64 * blocks_per_wave; }
+
+int mfma_tiles(int tokens, int rows, int blocks_per_wave) {
+    const int tn = mfma_tile_rows(blocks_per_wave);
+    return ((tokens + TM - 1) / TM) * ((rows + tn - 1) / tn);
+}
+
+// Blocks of 32 rows per wave.  Four (a 64 x 256 tile) halves the LDS and cache
+// traffic per matrix instruction but measured no faster than two: on this
+// device the matrix instructions and the other vector instructions of a SIMD
+// do not overlap, so the kernel is bound by their sum, not by data movement.
+int mfma_blocks_per_wave(long long wide_tiles) {
+    (void)wide_tiles;
+    return 2;
+}
+
+int q4_mfma_launch(const MfmaLaunch &launch, hipStream_t stream) {
+    MfmaLaunch L = launch;
+    if (L.cols < 64 || (L.cols & 63)) return -1;
+    if (L.table == nullptr) {                   // one job: the tiling is chosen here
+        if (L.blocks_per_wave == 0) L.blocks_per_wave = mfma_blocks_per_wave(mfma_tiles(L.one.tokens, L.one.rows, 4));
+        L.one.tile0 = 0;
+        L.total_tiles = mfma_tiles(L.one.tokens, L.one.rows, L.blocks_per_wave);
+    }
+    if (3 * (unsigned long long)L.plane_stride >= (1ull << 32)) return -1;      // 32-bit element offsets in the kernel
+    if (L.total_tiles < 1 || L.blocks_per_wave != 2 || (L.row_map && L.map_divisor < 1))
+        return -1;
+    hipLaunchKernelGGL(q4_mfma_kernel<2>, dim3(L.total_tiles), dim3(256), 0, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -386,6 +467,5 @@ int x_split_launch(const float *x, const float *gate, const int *row_map, int ma
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
-int mfma_tiles(int tokens, int rows) { return ((tokens + TM - 1) / TM) * ((rows + TN - 1) / TN); }
 
 }  // namespace mi355
