@@ -242,7 +242,7 @@ int salt_mi355_moe_reduce_dev(const float *expert_out, const float *weights, int
         set_error("moe reduce: bad arguments");
         return -1;
     }
-    return moe_reduce_launch(expert_out, weights, topk, hidden, out, (hipStream_t)stream);
+    return moe_reduce_launch(expert_out, weights, topk, hidden, out, nullptr, (hipStream_t)stream);
 }
 
 }  // extern "C"

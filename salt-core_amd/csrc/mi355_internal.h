@@ -24,6 +24,24 @@ struct Q4Job {
     int y_stride;
 };
 
+// The MoE decode step folded into two launches of the tile kernel: the gate/up launch runs the router in its
+// prologue (every workgroup finds its own expert; one extra workgroup publishes selection, weights and status), the
+// down launch computes gelu_tanh(gate) * up of its expert into LDS and reads its activations from there.
+struct MoeFuse {
+    const float *logits, *per_expert_scale;
+    const uint8_t *pool;
+    size_t expert_stride;
+    const float *x;               // [hidden]
+    float *gate, *up;             // [topk][routed]
+    float *expert_out;            // [topk][hidden]
+    int *selected;                // [topk], ascending expert id
+    float *weights;               // [topk]
+    int *status;                  // 0, or -1 when the router rejected its input (then nothing else is written)
+    int n_experts, topk, hidden, routed;
+};
+constexpr int MOE_FUSE_MAX_ROUTED = 4096;      // activations of one expert held in LDS by the down launch
+constexpr int MOE_FUSE_MAX_EXPERTS = 512;      // one thread per expert in the gate/up prologue
+
 struct Q4Launch {
     Q4Job one;                // used when table == nullptr
     const Q4Job *table;       // device array of njobs jobs sorted by tile0
@@ -33,7 +51,10 @@ struct Q4Launch {
     int total_tiles;
     float code_scale;         // 1 / (value the fp8 converter gives byte 1)
     int fused;                // 0: separately rounded multiply and add (bit-exact); 1: fma accumulate
+    MoeFuse moe;              // only read by q4_moe_gate_up_launch / q4_moe_down_launch
 };
+int q4_moe_gate_up_launch(const Q4Launch &launch, hipStream_t stream);   // fills tiles and jobs from launch.moe
+int q4_moe_down_launch(const Q4Launch &launch, hipStream_t stream);
 
 // chains_per_lane: 8, 4 or 2; 0 lets the launcher choose from the tile count.
 int q4_launch(const Q4Launch &launch, int chains_per_lane, hipStream_t stream);
@@ -163,7 +184,7 @@ int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t exp
 
 int moe_activate_launch(const float *gate, const float *up, float *act, size_t n, hipStream_t stream);
 int moe_reduce_launch(const float *expert_out, const float *weights, int topk, int hidden, float *out,
-                      hipStream_t stream);
+                      const int *status, hipStream_t stream);
 
 // Grouped prefill MoE (reference src/moe_group.c): rows bucketed per expert in
 // ascending expert / token / rank order, gate-up and down on the MFMA kernel,

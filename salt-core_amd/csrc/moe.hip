@@ -15,14 +15,12 @@
 // over the selected experts in list order) are done by one lane, in order.
 #include "device_math.h"
 #include "mi355_internal.h"
+#include "router_device.h"
 
 #include <string.h>
 
 namespace mi355 {
 namespace {
-
-constexpr int ROUTER_MAX_EXPERTS = 1024;
-constexpr int ROUTER_MAX_TOPK = 64;
 
 struct JobEmit {                 // where the router kernel writes the step's Q4 job tables (may be all-null)
     Q4Job *gate_up_jobs;
@@ -38,95 +36,17 @@ __global__ __launch_bounds__(ROUTER_MAX_EXPERTS) void router_topk_kernel(
         const float *__restrict__ logits, const float *__restrict__ per_expert_scale, int n_experts, int topk,
         int sorted_by_id, int *__restrict__ selected, float *__restrict__ weights, int *__restrict__ status,
         JobEmit emit) {
-    __shared__ float s_logit[ROUTER_MAX_EXPERTS];
-    __shared__ float s_exp[ROUTER_MAX_EXPERTS];
-    __shared__ float s_wave_max[ROUTER_MAX_EXPERTS / 64];
-    __shared__ int s_sel[ROUTER_MAX_TOPK];
-    __shared__ float s_w[ROUTER_MAX_TOPK];
-    __shared__ int s_bad;
-    __shared__ float s_peak;
-
+    __shared__ RouterShared sh;
+    router_topk_block(logits, per_expert_scale, n_experts, topk, sorted_by_id != 0, true, sh);
     const int e = threadIdx.x;
-    const bool live = e < n_experts;
-    if (e == 0) s_bad = 0;
-    __syncthreads();
-    float mine = -__builtin_inff();
-    if (live) {
-        mine = logits[e];
-        const float sc = per_expert_scale[e];
-        if (!(__builtin_fabsf(mine) < __builtin_inff()) || !(__builtin_fabsf(sc) < __builtin_inff())) s_bad = 1;
-        s_logit[e] = mine;
-    }
-    // max over finite values is exact in any order
-    float m = mine;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
-    if ((e & 63) == 0) s_wave_max[e >> 6] = m;
-    __syncthreads();
-    int bad = s_bad;
-    if (e == 0) {
-        float peak = s_wave_max[0];
-        for (int w = 1; w < (int)((blockDim.x + 63) >> 6); ++w) peak = fmaxf(peak, s_wave_max[w]);
-        s_peak = peak;
-    }
-    __syncthreads();
-    const float peak = s_peak;
-    if (!bad && live) {
-        int rank = 0;
-        for (int j = 0; j < n_experts; ++j) {
-            const float other = s_logit[j];
-            rank += (other > mine) || (other == mine && j < e);
-        }
-        s_exp[e] = det_expf(mine - peak);
-        if (rank < topk) s_sel[rank] = e;
-    }
-    __syncthreads();
-    if (e == 0 && !bad) {
-        float all = 0.0f;
-        int j0 = 0;
-        for (; j0 + 16 <= n_experts; j0 += 16) {       // batches of LDS reads, then the ordered adds
-            float v[16];
-#pragma unroll
-            for (int k = 0; k < 16; ++k) v[k] = s_exp[j0 + k];
-#pragma unroll
-            for (int k = 0; k < 16; ++k) all = all + v[k];
-        }
-        for (int j = j0; j < n_experts; ++j) all = all + s_exp[j];
-        if (!(all > 0.0f) || !(all < __builtin_inff())) bad = 1;
-        float chosen = 0.0f;
-        if (!bad) {
-            for (int j = 0; j < topk; ++j) {
-                s_w[j] = s_exp[s_sel[j]] / all;
-                chosen = chosen + s_w[j];
-            }
-            if (!(chosen > 0.0f) || !(chosen < __builtin_inff())) bad = 1;
-        }
-        if (!bad)
-            for (int j = 0; j < topk; ++j) {
-                const float share = s_w[j] / chosen;
-                s_w[j] = share * per_expert_scale[s_sel[j]];
-            }
-        s_bad = bad;
-    }
-    __syncthreads();
-    bad = s_bad;
+    const int bad = sh.bad;
     if (e == 0) *status = bad ? -1 : 0;
     if (e < topk) {
-        int expert, place = e;
-        float weight = 0.0f;
-        if (bad) {
-            expert = e;                          // a valid placeholder so that later launches stay in bounds
-        } else {
-            expert = s_sel[e];
-            weight = s_w[e];
-            if (sorted_by_id) {
-                place = 0;
-                for (int j = 0; j < topk; ++j) place += s_sel[j] < expert;
-            }
-        }
+        const int place = e;
+        const int expert = sh.out_sel[place];
         if (!bad) {                              // a rejected call leaves the caller's outputs untouched
             selected[place] = expert;
-            weights[place] = weight;
+            weights[place] = sh.out_w[place];
         }
         if (emit.gate_up_jobs) {
             const size_t n = (size_t)emit.hidden * (size_t)emit.routed;
@@ -171,7 +91,8 @@ __global__ __launch_bounds__(256) void moe_activate_kernel(const float *__restri
 
 __global__ __launch_bounds__(256) void moe_reduce_kernel(const float *__restrict__ expert_out,
                                                          const float *__restrict__ weights, int topk, int hidden,
-                                                         float *__restrict__ out) {
+                                                         const int *__restrict__ status, float *__restrict__ out) {
+    if (status && *status != 0) return;          // the router rejected its input: nothing was computed
     const int d = blockIdx.x * blockDim.x + threadIdx.x;
     if (d >= hidden) return;
     float sum = 0.0f;
@@ -221,9 +142,9 @@ int moe_activate_launch(const float *gate, const float *up, float *act, size_t n
 }
 
 int moe_reduce_launch(const float *expert_out, const float *weights, int topk, int hidden, float *out,
-                      hipStream_t stream) {
+                      const int *status, hipStream_t stream) {
     hipLaunchKernelGGL(moe_reduce_kernel, dim3((hidden + 255) / 256), dim3(256), 0, stream, expert_out, weights, topk,
-                       hidden, out);
+                       hidden, status, out);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -235,6 +156,19 @@ int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t exp
         g.topk > ROUTER_MAX_TOPK || g.hidden < 64 || (g.hidden & 63) || g.routed < 64 || (g.routed & 63))
         return -1;
     float *eo = expert_out ? expert_out : ws.expert_out;
+    if (g.n_experts <= MOE_FUSE_MAX_EXPERTS && g.routed <= MOE_FUSE_MAX_ROUTED) {
+        // Three launches: router + gate/up, activation + down, ordered reduction.
+        Q4Launch fused;
+        memset(&fused, 0, sizeof fused);
+        fused.code_scale = code_scale;
+        MoeFuse &m = fused.moe;
+        m.logits = logits; m.per_expert_scale = per_expert_scale; m.pool = pool; m.expert_stride = expert_stride;
+        m.x = x; m.gate = ws.gate; m.up = ws.up; m.expert_out = eo; m.selected = selected; m.weights = weights;
+        m.status = ws.status; m.n_experts = g.n_experts; m.topk = g.topk; m.hidden = g.hidden; m.routed = g.routed;
+        if (q4_moe_gate_up_launch(fused, stream) != 0) return -1;
+        if (q4_moe_down_launch(fused, stream) != 0) return -1;
+        return moe_reduce_launch(eo, weights, g.topk, g.hidden, out, ws.status, stream);
+    }
     JobEmit emit;
     emit.gate_up_jobs = ws.gate_up_jobs;
     emit.down_jobs = ws.down_jobs;
@@ -270,7 +204,7 @@ int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t exp
     down.code_scale = code_scale;
     if (q4_launch(down, 0, stream) != 0) return -1;
 
-    return moe_reduce_launch(eo, weights, g.topk, g.hidden, out, stream);
+    return moe_reduce_launch(eo, weights, g.topk, g.hidden, out, nullptr, stream);
 }
 
 }  // namespace mi355

@@ -24,7 +24,9 @@
 //    per wave.  A scale so large that scale * 2^9 would overflow flips the
 //    tile to a path that multiplies and adds separately with the raw scale.
 //  * The per-row fold runs in the documented order from LDS.
+#include "device_math.h"
 #include "mi355_internal.h"
+#include "router_device.h"
 
 #include <stddef.h>
 #include <stdio.h>
@@ -140,7 +142,13 @@ constexpr int x_batch_groups(int S, int NB) {
 // for three workgroups per compute unit; 32 is for launches with too few tiles
 // to share a compute unit, where the amount of data in flight per workgroup is
 // what hides the memory latency.
-template <int S, int NB, bool FUSED, int CB>
+//
+// PRO selects a prologue of the MoE decode step (0: none, jobs come from the
+// launch): 1 = router top-k, the workgroup derives its gate or up job from the
+// selection; 2 = the down projection of one selected expert, whose activations
+// gelu_tanh(gate) * up are computed into LDS and reach the VALU through
+// v_readfirstlane instead of scalar loads.
+template <int S, int NB, bool FUSED, int CB, int PRO = 0>
 __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L) {
     constexpr int CHUNK_BLOCKS = CB;
     constexpr int CHUNK_GROUPS = CB / 2;                   // 64-column scale groups per step
@@ -160,13 +168,64 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
 
     __shared__ __attribute__((aligned(16))) uint8_t w_lds[W_BYTES];
     __shared__ __attribute__((aligned(16))) float m_lds[2 * M_STAGE];
+    __shared__ __attribute__((aligned(16))) float x_lds[PRO == 2 ? MOE_FUSE_MAX_ROUTED : 4];
     __shared__ int slow_flag;
+    static_assert(PRO == 0 || (NB == 1 && !FUSED), "the MoE prologues serve the single-token bit-exact kernel");
+    static_assert(PRO != 1 || (sizeof(RouterShared) <= W_BYTES && THREADS >= MOE_FUSE_MAX_EXPERTS),
+                  "the router prologue borrows the weight staging memory and one thread per expert");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    const Q4Job job = find_job(L, blockIdx.x);
+    Q4Job job;
+    if (PRO == 0) {
+        job = find_job(L, blockIdx.x);
+    } else {
+        const MoeFuse &m = L.moe;
+        const size_t n = (size_t)m.hidden * (size_t)m.routed;
+        const size_t vals_bytes = n / 2, meta_bytes = (n / 64) * 2, proj_bytes = vals_bytes + 2 * meta_bytes;
+        if (PRO == 1) {
+            RouterShared &sh = *reinterpret_cast<RouterShared *>(w_lds);
+            const bool publisher = (int)blockIdx.x == L.total_tiles;       // one workgroup past the tiles
+            router_topk_block(m.logits, m.per_expert_scale, m.n_experts, m.topk, true, publisher, sh);
+            const int bad = sh.bad;
+            if (publisher) {
+                if (tid == 0) *m.status = bad ? -1 : 0;
+                if (tid < m.topk && !bad) { m.selected[tid] = sh.out_sel[tid]; m.weights[tid] = sh.out_w[tid]; }
+                return;
+            }
+            if (bad) return;                                               // uniform
+            const int up_tiles = (m.routed + TILE_ROWS - 1) / TILE_ROWS;
+            const int slot_index = (int)blockIdx.x / up_tiles;             // 2 * place + (0 gate | 1 up)
+            const int place = slot_index >> 1, proj = slot_index & 1;
+            const int expert = __builtin_amdgcn_readfirstlane(sh.out_sel[place]);
+            __syncthreads();                                               // the staging memory is free again
+            job.vals = m.pool + (size_t)expert * m.expert_stride + (size_t)proj * proj_bytes;
+            job.x = m.x;
+            job.y = (proj ? m.up : m.gate) + (size_t)place * m.routed;
+            job.rows = m.routed;
+            job.tile0 = slot_index * up_tiles;
+            job.x_stride = m.hidden;
+            job.y_stride = m.routed;
+        } else {
+            if (*(const int __attribute__((address_space(4))) *)(uintptr_t)m.status != 0) return;
+            const int down_tiles = (m.hidden + TILE_ROWS - 1) / TILE_ROWS;
+            const int place = (int)blockIdx.x / down_tiles;
+            const int expert = ((const int __attribute__((address_space(4))) *)(uintptr_t)m.selected)[place];
+            const float *gate = m.gate + (size_t)place * m.routed, *up = m.up + (size_t)place * m.routed;
+            for (int i = tid; i < m.routed; i += THREADS) x_lds[i] = det_gelu_tanh(gate[i]) * up[i];
+            job.vals = m.pool + (size_t)expert * m.expert_stride + 2 * proj_bytes;
+            job.x = nullptr;
+            job.y = m.expert_out + (size_t)place * m.hidden;
+            job.rows = m.hidden;
+            job.tile0 = place * down_tiles;
+            job.x_stride = m.routed;
+            job.y_stride = m.hidden;
+        }
+        job.scales = job.vals + vals_bytes;
+        job.biases = job.scales + meta_bytes;
+    }
     const int row0 = (blockIdx.x - job.tile0) * TILE_ROWS;
     const int R = job.rows;
     const int rows_here = R - row0 < TILE_ROWS ? R - row0 : TILE_ROWS;
@@ -260,6 +319,14 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
 
     // x of `groups` consecutive scale groups starting at group g0 of the row
     auto load_x = [&](int g0, float (&xq)[NB][XN], int groups) {
+        if (PRO == 2) {                   // wave-uniform LDS reads, broadcast into scalar registers
+            const float *xl = x_lds + g0 * 64 + S * wave;
+#pragma unroll
+            for (int k = 0; k < XN; ++k)
+                if (k < groups * 2 * S)
+                    xq[0][k] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(xl[(k / S) * 32 + (k % S)])));
+            return;
+        }
         const uniform_f32_ptr xg = xbase + (size_t)g0 * 64;
 #pragma unroll
         for (int t = 0; t < NB; ++t)
@@ -504,6 +571,38 @@ int q4_assign_tiles(Q4Job *table, int njobs) {
         tiles += (table[i].rows + TILE_ROWS - 1) / TILE_ROWS;
     }
     return tiles;
+}
+
+int q4_moe_gate_up_launch(const Q4Launch &launch, hipStream_t stream) {
+    Q4Launch L = launch;
+    const MoeFuse &m = L.moe;
+    if (m.n_experts < 1 || m.n_experts > MOE_FUSE_MAX_EXPERTS || m.topk < 1 || m.topk > m.n_experts ||
+        m.topk > ROUTER_MAX_TOPK || m.hidden < 64 || (m.hidden & 63) || m.routed < 64 || (m.routed & 63))
+        return -1;
+    L.table = nullptr; L.njobs = 1; L.cols = m.hidden; L.tokens = 1; L.fused = 0;
+    L.total_tiles = 2 * m.topk * ((m.routed + TILE_ROWS - 1) / TILE_ROWS);
+    const dim3 grid(L.total_tiles + 1), block(512);            // the extra workgroup publishes the router's outputs
+    if (L.total_tiles <= env_wide_limit())
+        hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 32, 1>), grid, block, 0, stream, L);
+    else
+        hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 16, 1>), grid, block, 0, stream, L);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int q4_moe_down_launch(const Q4Launch &launch, hipStream_t stream) {
+    Q4Launch L = launch;
+    const MoeFuse &m = L.moe;
+    if (m.topk < 1 || m.hidden < 64 || (m.hidden & 63) || m.routed < 64 || (m.routed & 63) ||
+        m.routed > MOE_FUSE_MAX_ROUTED)
+        return -1;
+    L.table = nullptr; L.njobs = 1; L.cols = m.routed; L.tokens = 1; L.fused = 0;
+    L.total_tiles = m.topk * ((m.hidden + TILE_ROWS - 1) / TILE_ROWS);
+    const dim3 grid(L.total_tiles), block(512);
+    if (L.total_tiles <= env_wide_limit())
+        hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 32, 2>), grid, block, 0, stream, L);
+    else
+        hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 16, 2>), grid, block, 0, stream, L);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
 int q4_launch(const Q4Launch &L, int chains_per_lane, hipStream_t stream) {

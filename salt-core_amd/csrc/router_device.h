@@ -1,0 +1,127 @@
+// Router top-k of one workgroup (reference models/gemma4-26b-a4b/src/gemma4.c:132-186,
+// ascending sort gemma4_text.c:7923-7930), shared by the stand-alone router
+// kernel and by the prologue of the fused gate/up launch.
+//
+// The reference's insertion list is the stable descending order of the logits
+// (a later expert must be strictly greater to pass an earlier one), so an
+// expert's position is its rank: the number of larger logits plus the number
+// of equal logits with a smaller index.  Ranks are computed in parallel; the
+// two fp32 sums whose order the reference fixes (over all experts ascending,
+// over the selected experts in list order) are done by one lane, in order.
+#pragma once
+
+#include "device_math.h"
+
+#include <hip/hip_runtime.h>
+
+namespace mi355 {
+
+constexpr int ROUTER_MAX_EXPERTS = 1024;
+constexpr int ROUTER_MAX_TOPK = 64;
+
+struct RouterShared {
+    float logit[ROUTER_MAX_EXPERTS];
+    float expv[ROUTER_MAX_EXPERTS];
+    float wave_max[ROUTER_MAX_EXPERTS / 64];
+    int sel[ROUTER_MAX_TOPK];          // list order (descending logit)
+    float w[ROUTER_MAX_TOPK];
+    int out_sel[ROUTER_MAX_TOPK];      // output order: list order, or ascending expert id
+    float out_w[ROUTER_MAX_TOPK];
+    int bad;
+    float peak;
+};
+
+// Every thread of the workgroup calls this; blockDim.x is a multiple of 64 and
+// at least max(n_experts, topk).  On return (after its last barrier) sh.bad
+// tells whether an input was non-finite, sh.out_sel[0..topk) holds the chosen
+// experts and, when want_weights, sh.out_w their weights.  With finite inputs
+// the two sums cannot fail (the largest term of the first is exp(0) = 1 and its
+// expert is always chosen), so a caller that only needs the selection may skip
+// the weights and still learn every rejection.
+__device__ __forceinline__ void router_topk_block(const float *__restrict__ logits,
+                                                  const float *__restrict__ per_expert_scale, int n_experts, int topk,
+                                                  bool sorted_by_id, bool want_weights, RouterShared &sh) {
+    const int e = threadIdx.x;
+    const bool live = e < n_experts;
+    if (e == 0) sh.bad = 0;
+    __syncthreads();
+    float mine = -__builtin_inff();
+    if (live) {
+        mine = logits[e];
+        const float sc = per_expert_scale[e];
+        if (!(__builtin_fabsf(mine) < __builtin_inff()) || !(__builtin_fabsf(sc) < __builtin_inff())) sh.bad = 1;
+        sh.logit[e] = mine;
+    }
+    // max over finite values is exact in any order
+    float m = mine;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    if ((e & 63) == 0 && e < ROUTER_MAX_EXPERTS) sh.wave_max[e >> 6] = m;
+    __syncthreads();
+    int bad = sh.bad;
+    if (e == 0) {
+        float peak = sh.wave_max[0];
+        const int waves = (n_experts + 63) >> 6;
+        for (int w = 1; w < waves; ++w) peak = fmaxf(peak, sh.wave_max[w]);
+        sh.peak = peak;
+    }
+    __syncthreads();
+    const float peak = sh.peak;
+    if (!bad && live) {
+        int rank = 0;
+        for (int j = 0; j < n_experts; ++j) {
+            const float other = sh.logit[j];
+            rank += (other > mine) || (other == mine && j < e);
+        }
+        if (want_weights) sh.expv[e] = det_expf(mine - peak);
+        if (rank < topk) sh.sel[rank] = e;
+    }
+    __syncthreads();
+    if (want_weights && e == 0 && !bad) {
+        float all = 0.0f;
+        int j0 = 0;
+        for (; j0 + 16 <= n_experts; j0 += 16) {       // batches of LDS reads, then the ordered adds
+            float v[16];
+#pragma unroll
+            for (int k = 0; k < 16; ++k) v[k] = sh.expv[j0 + k];
+#pragma unroll
+            for (int k = 0; k < 16; ++k) all = all + v[k];
+        }
+        for (int j = j0; j < n_experts; ++j) all = all + sh.expv[j];
+        if (!(all > 0.0f) || !(all < __builtin_inff())) bad = 1;
+        float chosen = 0.0f;
+        if (!bad) {
+            for (int j = 0; j < topk; ++j) {
+                sh.w[j] = sh.expv[sh.sel[j]] / all;
+                chosen = chosen + sh.w[j];
+            }
+            if (!(chosen > 0.0f) || !(chosen < __builtin_inff())) bad = 1;
+        }
+        if (!bad)
+            for (int j = 0; j < topk; ++j) {
+                const float share = sh.w[j] / chosen;
+                sh.w[j] = share * per_expert_scale[sh.sel[j]];
+            }
+        sh.bad = bad;
+    }
+    __syncthreads();
+    bad = sh.bad;
+    if (e < topk) {
+        int place = e;
+        if (bad) {
+            sh.out_sel[e] = e;                   // a valid placeholder so that dependent work stays in bounds
+            sh.out_w[e] = 0.0f;
+        } else {
+            const int expert = sh.sel[e];
+            if (sorted_by_id) {
+                place = 0;
+                for (int j = 0; j < topk; ++j) place += sh.sel[j] < expert;
+            }
+            sh.out_sel[place] = expert;
+            sh.out_w[place] = want_weights ? sh.w[e] : 0.0f;
+        }
+    }
+    __syncthreads();
+}
+
+}  // namespace mi355
