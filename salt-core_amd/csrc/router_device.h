@@ -23,6 +23,7 @@ struct RouterShared {
     float logit[ROUTER_MAX_EXPERTS];
     float expv[ROUTER_MAX_EXPERTS];
     float wave_max[ROUTER_MAX_EXPERTS / 64];
+    int rank[ROUTER_MAX_EXPERTS];
     int sel[ROUTER_MAX_TOPK];          // list order (descending logit)
     float w[ROUTER_MAX_TOPK];
     int out_sel[ROUTER_MAX_TOPK];      // output order: list order, or ascending expert id
@@ -67,14 +68,30 @@ __device__ __forceinline__ void router_topk_block(const float *__restrict__ logi
     }
     __syncthreads();
     const float peak = sh.peak;
-    if (!bad && live) {
-        int rank = 0;
-        for (int j = 0; j < n_experts; ++j) {
-            const float other = sh.logit[j];
-            rank += (other > mine) || (other == mine && j < e);
+    // Ranks: the comparisons of one expert are spread over as many threads as
+    // the workgroup has to spare (integer counts, so the split changes nothing).
+    const int padded = (n_experts + 63) & ~63;
+    const int parts = (int)blockDim.x / padded > 0 ? (int)blockDim.x / padded : 1;
+    if (live) sh.rank[e] = 0;
+    __syncthreads();
+    if (!bad && e < padded * parts) {
+        const int who = e % padded, part = e / padded;
+        if (who < n_experts) {
+            const float self = sh.logit[who];
+            const int span = (n_experts + parts - 1) / parts;
+            const int first = part * span, last = first + span < n_experts ? first + span : n_experts;
+            int count = 0;
+            for (int j = first; j < last; ++j) {
+                const float other = sh.logit[j];
+                count += (other > self) || (other == self && j < who);
+            }
+            if (parts > 1) atomicAdd(&sh.rank[who], count); else sh.rank[who] = count;
         }
+    }
+    __syncthreads();
+    if (!bad && live) {
         if (want_weights) sh.expv[e] = det_expf(mine - peak);
-        if (rank < topk) sh.sel[rank] = e;
+        if (sh.rank[e] < topk) sh.sel[sh.rank[e]] = e;
     }
     __syncthreads();
     if (want_weights && e == 0 && !bad) {
