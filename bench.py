@@ -38,7 +38,7 @@ SWEEP = [(2816, 2816), (16384, 2816), (2816, 8192)]        # (R, C) = (N, K)
 INSTANCE_BYTES = 640e6                                      # distinct weight bytes per launch
 # HBM bytes one launch of the default workload moves, from FETCH_SIZE / WRITE_SIZE counter runs scaled by a copy of
 # known size (profiles/q4_tile_kernel_decode_sweep_b1.md); valid for the default instance counts only.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 660_204_000
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 663_509_000
 
 
 class Events:
@@ -180,7 +180,7 @@ def main():
             "bound": "hbm", "achieved": round(bytes_per_launch / (launch_us * 1e-6) / 1e9, 1),
             "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(bytes_per_launch / (launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH, "kernel": "q4_tile_kernel<4,1,false>",
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH, "kernel": "q4_tile_kernel<4,1,false,16,0>",
             "bytes_per_launch": int(bytes_per_launch), "launch_us": round(launch_us, 2),
         },
     }
