@@ -353,7 +353,7 @@ __global__ __launch_bounds__(256) void fp4_qdq_kernel(const float *__restrict__ 
 int fp4_launch(const Fp4Launch &L, int chains_per_lane, hipStream_t stream) {
     if (L.total_tiles < 1 || L.tokens < 1 || L.tokens > 4 || L.cols < 32 || (L.cols & 31)) return -1;
     int S = chains_per_lane;
-    if (S == 0) S = L.total_tiles >= 128 ? 4 : 2;
+    if (S == 0) S = L.total_tiles > 512 ? 4 : 2;      // as for the affine-Q4 kernel: sixteen waves per tile up to two tiles per unit
     switch (S) {
         case 8: return launch_tiles<8>(L, stream);
         case 4: return launch_tiles<4>(L, stream);

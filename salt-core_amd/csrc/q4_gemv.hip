@@ -581,11 +581,13 @@ int q4_moe_gate_up_launch(const Q4Launch &launch, hipStream_t stream) {
         return -1;
     L.table = nullptr; L.njobs = 1; L.cols = m.hidden; L.tokens = 1; L.fused = 0;
     L.total_tiles = 2 * m.topk * ((m.routed + TILE_ROWS - 1) / TILE_ROWS);
-    const dim3 grid(L.total_tiles + 1), block(512);            // the extra workgroup publishes the router's outputs
+    const dim3 grid(L.total_tiles + 1);                         // the extra workgroup publishes the router's outputs
     if (L.total_tiles <= env_wide_limit())
-        hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 32, 1>), grid, block, 0, stream, L);
+        hipLaunchKernelGGL((q4_tile_kernel<2, 1, false, 32, 1>), grid, dim3(1024), 0, stream, L);
+    else if (L.total_tiles <= 512)
+        hipLaunchKernelGGL((q4_tile_kernel<2, 1, false, 16, 1>), grid, dim3(1024), 0, stream, L);
     else
-        hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 16, 1>), grid, block, 0, stream, L);
+        hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 16, 1>), grid, dim3(512), 0, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -597,11 +599,13 @@ int q4_moe_down_launch(const Q4Launch &launch, hipStream_t stream) {
         return -1;
     L.table = nullptr; L.njobs = 1; L.cols = m.routed; L.tokens = 1; L.fused = 0;
     L.total_tiles = m.topk * ((m.hidden + TILE_ROWS - 1) / TILE_ROWS);
-    const dim3 grid(L.total_tiles), block(512);
+    const dim3 grid(L.total_tiles);
     if (L.total_tiles <= env_wide_limit())
-        hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 32, 2>), grid, block, 0, stream, L);
+        hipLaunchKernelGGL((q4_tile_kernel<2, 1, false, 32, 2>), grid, dim3(1024), 0, stream, L);
+    else if (L.total_tiles <= 512)
+        hipLaunchKernelGGL((q4_tile_kernel<2, 1, false, 16, 2>), grid, dim3(1024), 0, stream, L);
     else
-        hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 16, 2>), grid, block, 0, stream, L);
+        hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 16, 2>), grid, dim3(512), 0, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -609,9 +613,10 @@ int q4_launch(const Q4Launch &L, int chains_per_lane, hipStream_t stream) {
     if (L.total_tiles < 1 || L.tokens < 1 || L.tokens > 4 || L.cols < 64 || (L.cols & 63)) return -1;
     int S = chains_per_lane ? chains_per_lane : env_chains();
     if (S == 0) {
-        // Four chains per lane (eight waves per tile) measured fastest whenever
-        // there are enough tiles to spread; fewer tiles take sixteen waves each.
-        S = L.total_tiles >= 128 ? 4 : 2;
+        // Four chains per lane (eight waves per tile) measured fastest once every
+        // compute unit holds three tiles; up to two tiles per unit, sixteen
+        // waves per tile hide more of the LDS and scalar-load latency.
+        S = L.total_tiles > 512 ? 4 : 2;
     }
     if (L.fused) {
         switch (S) {
