@@ -123,7 +123,7 @@ int salt_mi355_nvfp4_matmul_dev(const void *packed, const void *scales, float st
     }
     const Fp4MatmulWorkspace w = fp4_matmul_carve(workspace, R, C, B);
     hipStream_t s = (hipStream_t)stream;
-    if (hip_ok(hipMemsetAsync(w.status, 0, 4, s), "nvfp4 matmul status") != 0) return -1;
+    if (clear_words_launch(w.status, 1, s) != 0) { set_error("nvfp4 matmul: status clear failed to launch"); return -1; }
     if (fp4_qdq_launch(xs, C, B, input_global_scale, nullptr, nullptr, nullptr, w.plane, w.status, s) != 0) {
         set_error("nvfp4 matmul: activation pass failed to launch");
         return -1;

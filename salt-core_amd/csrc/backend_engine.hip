@@ -1056,7 +1056,7 @@ int salt_gpu_nvfp4_qdq(const float *input, int C, float input_global_scale, uint
     uint8_t *dq_dev = device_take(n * 4), *p_dev = device_take(n / 2), *s_dev = device_take(n / 16);
     int *st_dev = (int *)device_take(4);
     uint8_t *pin = pinned_take(n * 4 + n / 2 + n / 16 + 64);
-    if (hip_ok(hipMemsetAsync(st_dev, 0, 4, g_state.stream), "status clear") != 0 ||
+    if (clear_words_launch(st_dev, 1, g_state.stream) != 0 ||
         salt_mi355_nvfp4_qdq_dev(x_dev, C, 1, input_global_scale, p_dev, s_dev, (float *)dq_dev, st_dev, g_state.stream) != 0)
         return -1;
     int status = 0;
@@ -1096,7 +1096,7 @@ int run_fp4_jobs(std::vector<Fp4HostJob> &jobs, int C) {
     const size_t bytes = (in_floats * 2 + out_floats) * 4 + 4096 + 512 * jobs.size();
     if (staging_reserve(bytes, bytes) != 0) return -1;
     int *st_dev = (int *)device_take(4);
-    if (hip_ok(hipMemsetAsync(st_dev, 0, 4, g_state.stream), "status clear") != 0) return -1;
+    if (clear_words_launch(st_dev, 1, g_state.stream) != 0) return -1;
     std::vector<OutputCopy> copies;
     SaltGpuBatchStatsV2 &stats = e.stats;
     for (Fp4HostJob &j : jobs) {

@@ -195,6 +195,9 @@ int moe_prefill_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_
                        const int *selected, const float *weights, const float *inputs, float *outputs,
                        int *group_rows, int *row_pairs, int *status_dev, void *workspace, hipStream_t stream);
 
+// Zero `words` 32-bit words at dst with a kernel on `stream` (safe under graph capture, unlike a memset node).
+int clear_words_launch(void *dst, size_t words, hipStream_t stream);
+
 // ---------------------------------------------------------------- probes
 
 // Decodes all 256 byte values through the fp8 and fp4 converters (device

@@ -659,6 +659,21 @@ __global__ void probe_converters_kernel(float *fp8_values, float *fp4_values) {
 }
 }  // namespace
 
+namespace {
+__global__ __launch_bounds__(256) void clear_words_kernel(uint32_t *dst, size_t words) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < words) dst[i] = 0u;
+}
+}  // namespace
+
+// Zero fill by a kernel: a memset node recorded into a caller's graph capture is not reliable on replay here.
+int clear_words_launch(void *dst, size_t words, hipStream_t stream) {
+    if (words == 0) return 0;
+    hipLaunchKernelGGL(clear_words_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream, (uint32_t *)dst,
+                       words);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
 int probe_converters_launch(float *fp8_values, float *fp4_values, hipStream_t stream) {
     hipLaunchKernelGGL(probe_converters_kernel, dim3(1), dim3(256), 0, stream, fp8_values, fp4_values);
     return hipGetLastError() == hipSuccess ? 0 : -1;
