@@ -158,8 +158,8 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
     constexpr int M_STAGE = TILE_ROWS * M_PITCH;
     constexpr int WAVES = 32 / S;
     constexpr int THREADS = WAVES * 64;
-    constexpr int PIECES = (TILE_ROWS * CHUNK_BLOCKS) / THREADS;              // 16-byte pieces per thread
-    constexpr int META_ITEMS = (TILE_ROWS * CHUNK_GROUPS + THREADS - 1) / THREADS;
+    // A staging item is one scale group of one row: 32 bytes of codes (two blocks) and its (scale, bias).
+    constexpr int ITEMS = (TILE_ROWS * CHUNK_GROUPS + THREADS - 1) / THREADS;
     constexpr int FOLD_BYTES = NB * TILE_ROWS * FOLD_PITCH * 4;
     constexpr int W_BYTES = 2 * W_STAGE > FOLD_BYTES ? 2 * W_STAGE : FOLD_BYTES;
     constexpr int XG = x_batch_groups(S, NB);
@@ -241,67 +241,80 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
     const global_f32_out_ptr y = (global_f32_out_ptr)(uintptr_t)job.y;
     const uniform_f32_ptr xbase = as_uniform(job.x) + S * wave;
 
-    // Per-thread staging geometry, fixed for the whole tile.  Piece i of a
-    // thread lies (THREADS / 16) rows below piece 0 in the same 16-byte column,
-    // so only the clamped source row offsets need registers.
-    constexpr int W_ROW_STEP = THREADS / CHUNK_BLOCKS, M_ROW_STEP = THREADS / CHUNK_GROUPS;
-    const uint32_t w_seg = tid % CHUNK_BLOCKS;
-    const uint32_t w_dst0 = (tid / CHUNK_BLOCKS) * W_PITCH + w_seg * 16;
-    uint32_t w_src[PIECES];
+    // Per-thread staging geometry, fixed for the whole tile: item i of a thread
+    // is group (tid % CHUNK_GROUPS) of row (tid / CHUNK_GROUPS + i * ROW_STEP), so
+    // consecutive threads read consecutive 32-byte pieces of a row.  In LDS the
+    // two blocks of a group are interleaved 16 bits at a time: dword t of the
+    // group holds bytes 2t, 2t+1 of the first block and of the second, which is
+    // exactly the pair of two-byte slices a four-chain wave consumes.
+    constexpr int ROW_STEP = THREADS / CHUNK_GROUPS;
+    const bool has_item = tid < TILE_ROWS * CHUNK_GROUPS;    // only narrower than the block when THREADS == 1024
+    const uint32_t it_grp = tid % CHUNK_GROUPS;
+    const uint32_t w_dst0 = ((tid / CHUNK_GROUPS) & (TILE_ROWS - 1)) * W_PITCH + it_grp * 32;
+    const uint32_t m_dst0 = ((tid / CHUNK_GROUPS) & (TILE_ROWS - 1)) * M_PITCH + 2 * it_grp;
+    uint32_t w_off[ITEMS], m_off[ITEMS];                     // source offsets of the item in step 0
 #pragma unroll
-    for (int i = 0; i < PIECES; ++i) {
-        const int row = (tid / CHUNK_BLOCKS) + i * W_ROW_STEP;
-        w_src[i] = (uint32_t)(row < rows_here ? row : rows_here - 1) * row_bytes;
-    }
-    const bool has_meta = tid < TILE_ROWS * CHUNK_GROUPS;    // only narrower than the block when THREADS == 1024
-    const uint32_t m_grp = tid % CHUNK_GROUPS;
-    const uint32_t m_dst0 = ((tid / CHUNK_GROUPS) & (TILE_ROWS - 1)) * M_PITCH + 2 * m_grp;
-    uint32_t m_src[META_ITEMS];
-#pragma unroll
-    for (int i = 0; i < META_ITEMS; ++i) {
-        const int row = ((tid / CHUNK_GROUPS) + i * M_ROW_STEP) & (TILE_ROWS - 1);
-        m_src[i] = (uint32_t)(row < rows_here ? row : rows_here - 1) * ngrp;
+    for (int i = 0; i < ITEMS; ++i) {
+        const int row = ((tid / CHUNK_GROUPS) + i * ROW_STEP) & (TILE_ROWS - 1);
+        const uint32_t rc = (uint32_t)(row < rows_here ? row : rows_here - 1);
+        w_off[i] = rc * row_bytes + it_grp * 32;
+        m_off[i] = rc * ngrp + it_grp;
     }
 
-    u32x4 wreg[PIECES];
-    uint32_t sreg[META_ITEMS], breg[META_ITEMS];     // raw bf16 bits; nothing may consume them before commit
+    u32x4 wreg[ITEMS][2];
+    uint32_t sreg[ITEMS], breg[ITEMS];               // raw bf16 bits; nothing may consume them before commit
 
-    // Loads of step ck into registers.  Block and group indices past the end
-    // of the row (last step only) are clamped: the data is staged but never
-    // consumed.
+    // Loads of step ck into registers.  In every step but a partial last one
+    // the address is a wave-uniform base plus the fixed per-thread offset; in
+    // the last one group indices past the end of the row are clamped (the data
+    // is staged but never consumed).
     auto issue = [&](int ck) {
+        if (!has_item) return;
+        const bool tail = (ck + 1) * CHUNK_GROUPS > ngrp;
+        if (!tail) {
+            const global_u8_ptr v = vals + (size_t)ck * (CHUNK_GROUPS * 32);
+            const global_u16_ptr sp = scales16 + (size_t)ck * CHUNK_GROUPS;
+            const global_u16_ptr bp = biases16 ? biases16 + (size_t)ck * CHUNK_GROUPS : (global_u16_ptr)0;
 #pragma unroll
-        for (int i = 0; i < PIECES; ++i) {
-            int blk = ck * CHUNK_BLOCKS + (int)w_seg;
-            blk = blk < nblk ? blk : nblk - 1;
-            wreg[i] = *(global_u128_ptr)(vals + (w_src[i] + (uint32_t)blk * 16u));
-        }
+            for (int i = 0; i < ITEMS; ++i) {
+                wreg[i][0] = *(global_u128_ptr)(v + w_off[i]);
+                wreg[i][1] = *(global_u128_ptr)(v + w_off[i] + 16);
+                sreg[i] = sp[m_off[i]];
+                breg[i] = bp ? (uint32_t)bp[m_off[i]] : 0u;
+            }
+        } else {
 #pragma unroll
-        for (int i = 0; i < META_ITEMS; ++i) {
-            int g = ck * CHUNK_GROUPS + (int)m_grp;
-            g = g < ngrp ? g : ngrp - 1;
-            const uint32_t at = m_src[i] + (uint32_t)g;
-            sreg[i] = scales16[at];
-            breg[i] = biases16 ? (uint32_t)biases16[at] : 0u;
+            for (int i = 0; i < ITEMS; ++i) {
+                int g = ck * CHUNK_GROUPS + (int)it_grp;
+                const uint32_t back = g < ngrp ? 0u : (uint32_t)(g - (ngrp - 1));     // groups to step back to the last one
+                const global_u8_ptr v = vals + (size_t)ck * (CHUNK_GROUPS * 32);
+                wreg[i][0] = *(global_u128_ptr)(v + (w_off[i] - back * 32));
+                wreg[i][1] = *(global_u128_ptr)(v + (w_off[i] - back * 32) + 16);
+                const uint32_t at = m_off[i] + (uint32_t)ck * CHUNK_GROUPS - back;
+                sreg[i] = scales16[at];
+                breg[i] = biases16 ? (uint32_t)biases16[at] : 0u;
+            }
         }
     };
 
     auto commit = [&](int stage) {
+        if (!has_item) return;
 #pragma unroll
-        for (int i = 0; i < PIECES; ++i) {
-            uint32_t *dst = reinterpret_cast<uint32_t *>(w_lds + stage * W_STAGE + w_dst0 + i * W_ROW_STEP * W_PITCH);
-            dst[0] = wreg[i].x; dst[1] = wreg[i].y; dst[2] = wreg[i].z; dst[3] = wreg[i].w;
-        }
-        if (has_meta) {
+        for (int i = 0; i < ITEMS; ++i) {
+            uint32_t *dst = reinterpret_cast<uint32_t *>(w_lds + stage * W_STAGE + w_dst0 + i * ROW_STEP * W_PITCH);
+            const uint32_t a[4] = {wreg[i][0].x, wreg[i][0].y, wreg[i][0].z, wreg[i][0].w};
+            const uint32_t b[4] = {wreg[i][1].x, wreg[i][1].y, wreg[i][1].z, wreg[i][1].w};
 #pragma unroll
-            for (int i = 0; i < META_ITEMS; ++i) {
-                const float sc = bf16_to_f32(sreg[i]);
-                const float bi = bf16_to_f32(breg[i]);
-                if (!(__builtin_fabsf(sc) < BIG_SCALE)) slow_flag = 1;
-                float *dst = m_lds + stage * M_STAGE + m_dst0 + i * M_ROW_STEP * M_PITCH;
-                dst[0] = sc * L.code_scale;
-                dst[1] = bi;
+            for (int d = 0; d < 4; ++d) {
+                dst[2 * d] = __builtin_amdgcn_perm(b[d], a[d], 0x05040100u);          // low halves of a and b
+                dst[2 * d + 1] = __builtin_amdgcn_perm(b[d], a[d], 0x07060302u);      // high halves
             }
+            const float sc = bf16_to_f32(sreg[i]);
+            const float bi = bf16_to_f32(breg[i]);
+            if (!(__builtin_fabsf(sc) < BIG_SCALE)) slow_flag = 1;
+            float *mdst = m_lds + stage * M_STAGE + m_dst0 + i * ROW_STEP * M_PITCH;
+            mdst[0] = sc * L.code_scale;
+            mdst[1] = bi;
         }
     };
 
@@ -351,7 +364,9 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
         if (ck + 1 < nchunk) issue(ck + 1);
 
         const int slow = __builtin_amdgcn_readfirstlane(slow_flag);
-        const uint8_t *wrow = w_lds + stage * W_STAGE + lane * W_PITCH + wave * (S / 2);
+        // wave t reads dword t (S == 4), dwords 2t and 2t+1 (S == 8) or dword t / 2 (S == 2) of every group
+        const uint8_t *wrow = w_lds + stage * W_STAGE + lane * W_PITCH + (S == 2 ? (wave >> 1) * 4 : wave * S);
+        const uint32_t byte_pick = 0x0C0C0000u | (uint32_t)((2 + (wave & 1)) << 8) | (uint32_t)(wave & 1);
         const float *mrow = m_lds + stage * M_STAGE + lane * M_PITCH;
 
         // LDS operands of group g of this step: the lane's nibbles and (scale', bias)
@@ -359,17 +374,16 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
             scale = mrow[2 * g];
             bias = mrow[2 * g + 1];
             w1 = 0;
-            if (S == 8) {
-                w0 = *reinterpret_cast<const uint32_t *>(wrow + (2 * g) * 16);
-                w1 = *reinterpret_cast<const uint32_t *>(wrow + (2 * g + 1) * 16);
-            } else if (S == 4) {
-                const uint32_t a = *reinterpret_cast<const uint16_t *>(wrow + (2 * g) * 16);
-                const uint32_t b = *reinterpret_cast<const uint16_t *>(wrow + (2 * g + 1) * 16);
-                w0 = a | (b << 16);
-            } else {
-                const uint32_t a = wrow[(2 * g) * 16];
-                const uint32_t b = wrow[(2 * g + 1) * 16];
-                w0 = a | (b << 8);
+            if (S == 8) {            // dwords 2t, 2t+1: (a01 b01), (a23 b23) -> the wave's four bytes of each block
+                const uint32_t d0 = *reinterpret_cast<const uint32_t *>(wrow + g * 32);
+                const uint32_t d1 = *reinterpret_cast<const uint32_t *>(wrow + g * 32 + 4);
+                w0 = __builtin_amdgcn_perm(d1, d0, 0x05040100u);
+                w1 = __builtin_amdgcn_perm(d1, d0, 0x07060302u);
+            } else if (S == 4) {     // dword t: two bytes of the first block, two of the second
+                w0 = *reinterpret_cast<const uint32_t *>(wrow + g * 32);
+            } else {                 // S == 2: byte (t & 1) of each half of dword t / 2
+                const uint32_t d = *reinterpret_cast<const uint32_t *>(wrow + g * 32);
+                w0 = __builtin_amdgcn_perm(0u, d, byte_pick);
             }
         };
 
