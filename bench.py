@@ -141,6 +141,54 @@ def cpu_baseline(synth, budget_s: float = 12.0):
     }
 
 
+def cpu_other_configs(synth, pool, cores: int, budget_s: float = 3.0):
+    """The other configurations on the host cores, each on a bounded sample."""
+    import ctypes as C
+    from oracle_lib import ExpertGeometry, load_oracle, load_reference, ptr
+    oracle, ref = load_oracle(), load_reference()
+    out = {}
+
+    def rate(fn, unit_count, budget):
+        fn()
+        t0 = time.perf_counter(); fn(); once = time.perf_counter() - t0
+        reps = max(1, min(1000, int(budget / max(once, 1e-6))))
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        return unit_count * reps / (time.perf_counter() - t0), reps
+
+    # MoE decode layer-step (port of the reference's step, experts run on `cores` threads)
+    E, K, H, F = 128, 8, 2816, 704
+    g = ExpertGeometry(H, F)
+    logits, scale = synth.router_logits(E, 900), np.ones(E, np.float32)
+    x = synth.activations(H, 1, 950)[0]
+    sel, w = np.zeros(K, np.int32), np.zeros(K, np.float32)
+    eo, y = np.zeros((K, H), np.float32), np.zeros(H, np.float32)
+    steps_per_s, reps = rate(lambda: oracle.orc_moe_decode_step(C.byref(g), ptr(pool), E, K, ptr(logits), ptr(scale), ptr(x),
+                                                                ptr(sel), ptr(w), ptr(eo), ptr(y), cores), 1, budget_s)
+    out["moe_decode_step_us"] = {"value": round(1e6 / steps_per_s, 1), "kind": "port", "cores": cores,
+                                 "sample": f"{reps} layer-steps"}
+    # MoE prefill, grouped per expert: a 32-token sample of the 2048-token workload
+    T = 32
+    psel, pw = synth.zipf_selection(T, E, K, 1.1, 60)
+    px, py = synth.activations(H, T, 61), np.zeros((T, H), np.float32)
+    tok_per_s, reps = rate(lambda: oracle.orc_moe_group(C.byref(g), ptr(pool), E, K, T, ptr(psel), ptr(pw), ptr(px), ptr(py),
+                                                        None, cores), T, budget_s)
+    out["moe_prefill_tokens_per_s"] = {"value": round(tok_per_s, 1), "kind": "port", "cores": cores,
+                                       "sample": f"{reps} passes over {T} tokens"}
+    # NVFP4 8192 x 8192, batch 1: the reference's own function (single thread)
+    R = Cc = 8192
+    packed, fscales = synth.nvfp4_tensor(R, Cc, 40)
+    fx, fy = synth.activations(Cc, 1, 41)[0], np.zeros(R, np.float32)
+    xp, xs, xd = np.zeros(Cc // 2, np.uint8), np.zeros(Cc // 16, np.uint8), np.zeros(Cc, np.float32)
+    fn = ref.salt_nvfp4_matvec_reference if ref is not None else oracle.orc_nvfp4_matvec
+    calls_per_s, reps = rate(lambda: fn(ptr(packed), ptr(fscales), 2688.0, 64.0, R, Cc, ptr(fx), ptr(fy), ptr(xp), ptr(xs),
+                                        ptr(xd)), 1, budget_s)
+    out["nvfp4_8192_matvec_us"] = {"value": round(1e6 / calls_per_s, 1), "kind": "reference" if ref is not None else "port",
+                                   "cores": 1, "sample": f"{reps} calls"}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -273,6 +321,8 @@ def main():
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(synth)
+        if not args.no_extra:
+            result["cpu_baseline"]["other_configs"] = cpu_other_configs(synth, pool, result["cpu_baseline"]["cores"])
     print(json.dumps(result))
 
 
