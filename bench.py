@@ -300,6 +300,32 @@ def main():
         extra["nvfp4_8192_b256_tflops"] = round(2.0 * R * Cc * B / (ms_mm * 1e-3) / 1e12, 1)
         extra["nvfp4_8192_b256_mfma_frac"] = round(2.0 * R * Cc * B / (ms_mm * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
         del w, xb, yb, wsb
+        # BASELINE configs[0] through the engine-facing ABI: host pointers in and out (activation upload, launch,
+        # result download and a stream sync per call); a latency figure, never a throughput claim
+        import ctypes as C
+        R0 = C0 = 4096
+        v0, s0, b0 = synth.q4_tensor(R0, C0, 0)
+        blob = np.concatenate([v0.view(np.uint8), s0.view(np.uint8), b0.view(np.uint8)])
+        base = blob.ctypes.data
+        vp = C.c_void_p
+        lib.salt_gpu_weight_resource_describe.argtypes = [C.c_uint32, C.c_uint32, vp, C.c_size_t]
+        lib.salt_gpu_weight_resource_activate.argtypes = [C.c_uint32, C.c_uint32, C.c_int]
+        lib.salt_gpu_weight_resource_deactivate.argtypes = [C.c_uint32, C.c_uint32]
+        lib.salt_gpu_q4_matvec.argtypes = [vp, vp, vp, C.c_int, C.c_int, vp, vp]
+        x0, y0 = synth.activations(C0, 1, 1)[0], np.zeros(R0, np.float32)
+        if (lib.salt_gpu_init() == 0 and lib.salt_gpu_weight_resource_describe(1, 900, base, blob.nbytes) == 0
+                and lib.salt_gpu_weight_resource_activate(1, 900, 2) == 0):
+            def abi_call():
+                if lib.salt_gpu_q4_matvec(base, base + v0.nbytes, base + v0.nbytes + s0.nbytes, R0, C0,
+                                          x0.ctypes.data, y0.ctypes.data) != 0:
+                    raise RuntimeError(lib.salt_mi355_last_error().decode())
+            for _ in range(5):
+                abi_call()
+            t0 = time.perf_counter()
+            for _ in range(200):
+                abi_call()
+            extra["abi_q4_matvec_4096_host_pointers_us"] = round((time.perf_counter() - t0) / 200 * 1e6, 1)
+            lib.salt_gpu_weight_resource_deactivate(1, 900)
         # MoE prefill, 2048 tokens through one layer (E = 128, top-8, Zipf 1.1), grouped per expert, matrix cores
         T = 2048
         sel, wts = synth.zipf_selection(T, E, K, 1.1, 60)
