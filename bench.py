@@ -263,7 +263,7 @@ def main():
         extra["moe_decode_step_gbps"] = round(step_bytes / (ms_moe * 1e-3) / 1e9, 1)
         extra["moe_decode_step_hbm_frac"] = round(step_bytes / (ms_moe * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
         del layers
-        # NVFP4 8192 x 8192, batch 1, reference semantics (activation Q/DQ + rows), 16 instances
+        # NVFP4 8192 x 8192, batch 1, reference semantics (activation Q/DQ inside the rows' launch), 16 instances
         R = Cc = 8192
         packed, fscales = synth.nvfp4_tensor(R, Cc, 40)
         G = 16
@@ -273,13 +273,13 @@ def main():
             w.upload(packed, g * per)
             w.upload(fscales, g * per + packed.nbytes)
         x = gpu.DeviceBuffer.from_host(synth.activations(Cc, 1, 41))
-        xq, y, st = gpu.DeviceBuffer(Cc * 4), gpu.DeviceBuffer(R * 4), gpu.DeviceBuffer(4, fill=0)
+        y, st = gpu.DeviceBuffer(R * 4), gpu.DeviceBuffer(4, fill=0)
 
         def fp4_step(s):
             for g in range(G):
-                lib.salt_mi355_nvfp4_qdq_dev(x.ptr, Cc, 1, 64.0, None, None, xq.ptr, st.ptr, s)
-                lib.salt_mi355_nvfp4_matvec_dev(w.at(g * per), w.at(g * per + packed.nbytes), 2688.0, R, Cc, 1,
-                                                xq.ptr, y.ptr, 0, s)
+                if lib.salt_mi355_nvfp4_matvec_qdq_dev(w.at(g * per), w.at(g * per + packed.nbytes), 2688.0, 64.0, R, Cc,
+                                                       x.ptr, y.ptr, st.ptr, 0, s) != 0:
+                    raise RuntimeError(lib.salt_mi355_last_error().decode())
 
         ms_fp4 = timed(lib, stream, events, fp4_step, 2, 10) / G
         extra["nvfp4_8192_matvec_us"] = round(ms_fp4 * 1e3, 2)

@@ -130,6 +130,18 @@ int salt_mi355_nvfp4_matvec_dev(const void *packed, const void *scales, float st
                                 int R, int C, int B, const float *xs, float *ys,
                                 int chains_per_lane, void *stream);
 
+/* The reference matvec of one token in one launch (reference
+ * salt_nvfp4_matvec_reference, nvfp4.c:228-256): every workgroup quantises
+ * and dequantises the activation x[C] itself (nvfp4.c:82-130) and computes its
+ * rows from that, bit-identical to salt_mi355_nvfp4_qdq_dev followed by
+ * salt_mi355_nvfp4_matvec_dev.  C a multiple of 32, at most 8192.  status_dev:
+ * a device int the caller has cleared; it becomes -1 when x holds a non-finite
+ * value, and y is not written then. */
+int salt_mi355_nvfp4_matvec_qdq_dev(const void *packed, const void *scales,
+                                    float stored_divisor, float input_global_scale,
+                                    int R, int C, const float *x, float *y,
+                                    int *status_dev, int chains, void *stream);
+
 /* Prefill-sized NVFP4 matmul on the matrix cores (tolerance class): every
  * token is quantised and dequantised as salt_nvfp4_quantize_input_reference
  * does (nvfp4.c:82-130) and ys[token][row] approximates the reference matvec

@@ -148,6 +148,35 @@ int salt_mi355_nvfp4_matmul_dev(const void *packed, const void *scales, float st
     return 0;
 }
 
+int salt_mi355_nvfp4_matvec_qdq_dev(const void *packed, const void *scales, float stored_divisor,
+                                    float input_global_scale, int R, int C, const float *x, float *y, int *status_dev,
+                                    int chains, void *stream) {
+    if (!g_state.ready) { set_error("nvfp4 matvec: library not initialised"); return -1; }
+    if (!g_state.fp8_is_ocp) { set_error("nvfp4: this device's fp8 converter is not OCP E4M3FN"); return -1; }
+    if (!packed || !scales || !x || !y || !status_dev || R < 1 || C < 32 || (C & 31) || C > FP4_FUSED_MAX_COLS ||
+        !isfinite(stored_divisor) || stored_divisor == 0.0f || !isfinite(input_global_scale) ||
+        input_global_scale <= 0.0f || ((uintptr_t)packed & 15) || ((uintptr_t)scales & 1) || ((uintptr_t)x & 15) ||
+        ((uintptr_t)y & 3) || (chains != 0 && chains != 8 && chains != 4 && chains != 2)) {
+        set_error("nvfp4 matvec: bad arguments (C a multiple of 32 up to %d, packed and x 16-byte aligned)",
+                  FP4_FUSED_MAX_COLS);
+        return -1;
+    }
+    Fp4Launch launch;
+    memset(&launch, 0, sizeof launch);
+    launch.one.packed = (const uint8_t *)packed;
+    launch.one.scales = (const uint8_t *)scales;
+    launch.one.x = x;
+    launch.one.y = y;
+    launch.one.weight_global_scale = 1.0f / stored_divisor;
+    launch.one.rows = R;
+    launch.one.x_stride = C;
+    launch.njobs = 1; launch.cols = C; launch.tokens = 1;
+    launch.total_tiles = (R + 63) / 64;
+    launch.qdq = 1; launch.input_global_scale = input_global_scale; launch.status = status_dev;
+    if (fp4_launch(launch, chains, (hipStream_t)stream) != 0) { set_error("nvfp4 matvec: launch failed"); return -1; }
+    return 0;
+}
+
 int salt_mi355_router_topk_dev(const float *logits, const float *per_expert_scale, int n_experts, int topk,
                                int sorted_by_id, int *selected, float *weights, int *status_dev, void *stream) {
     if (!g_state.ready) { set_error("router: library not initialised"); return -1; }

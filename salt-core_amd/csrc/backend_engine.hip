@@ -1105,11 +1105,18 @@ int run_fp4_jobs(std::vector<Fp4HostJob> &jobs, int C) {
         if (!x_dev) return -1;
         float *dq_dev = (float *)device_take(xin * 4);
         uint8_t *y_dev = device_take(yout * 4), *y_pin = pinned_take(yout * 4);
-        if (salt_mi355_nvfp4_qdq_dev(x_dev, C, j.tokens, j.tensor->input_global_scale, nullptr, nullptr, dq_dev, st_dev,
-                                     g_state.stream) != 0 ||
-            salt_mi355_nvfp4_matvec_dev(j.packed, j.scales, j.tensor->stored_divisor, j.rows, C, j.tokens, dq_dev,
-                                        (float *)y_dev, 0, g_state.stream) != 0)
+        const bool one_launch = j.tokens == 1 && C <= FP4_FUSED_MAX_COLS;   // the activation pass runs inside the rows' launch
+        if (one_launch) {
+            if (salt_mi355_nvfp4_matvec_qdq_dev(j.packed, j.scales, j.tensor->stored_divisor,
+                                                j.tensor->input_global_scale, j.rows, C, x_dev, (float *)y_dev, st_dev, 0,
+                                                g_state.stream) != 0)
+                return -1;
+        } else if (salt_mi355_nvfp4_qdq_dev(x_dev, C, j.tokens, j.tensor->input_global_scale, nullptr, nullptr, dq_dev,
+                                            st_dev, g_state.stream) != 0 ||
+                   salt_mi355_nvfp4_matvec_dev(j.packed, j.scales, j.tensor->stored_divisor, j.rows, C, j.tokens, dq_dev,
+                                               (float *)y_dev, 0, g_state.stream) != 0) {
             return -1;
+        }
         e.pending.push_back({y_pin, j.y_host, yout * 4});
         copies.push_back({y_dev, y_pin, yout * 4});
         stats.nvfp4_logical_packed_weight_bytes += (uint64_t)j.rows * C / 2;
@@ -1117,7 +1124,7 @@ int run_fp4_jobs(std::vector<Fp4HostJob> &jobs, int C) {
         stats.nvfp4_activation_input_bytes += xin * 4;
         stats.nvfp4_activation_qdq_bytes += xin * 4;
         stats.nvfp4_projection_output_bytes += yout * 4;
-        stats.nvfp4_kernel_launches += 2 + (uint64_t)((j.tokens - 1) / 4);
+        stats.nvfp4_kernel_launches += one_launch ? 1 : 2 + (uint64_t)((j.tokens - 1) / 4);
     }
     uint8_t *st_pin = pinned_take(4);
     for (const OutputCopy &c : copies)

@@ -126,7 +126,14 @@ struct Fp4Launch {
     int cols;
     int tokens;
     int total_tiles;
+    // Fused activation pass (single job, one token, cols <= FP4_FUSED_MAX_COLS): x is the raw activation, every
+    // workgroup quantises and dequantises it into LDS, *status (cleared by the caller) becomes -1 for a non-finite
+    // activation, and nothing is published then.
+    int qdq;
+    float input_global_scale;
+    int *status;
 };
+constexpr int FP4_FUSED_MAX_COLS = 8192;
 
 int fp4_launch(const Fp4Launch &launch, int chains_per_lane, hipStream_t stream);
 // activation quantise/dequantise per 16-block; any of packed/scales/dequant/plane may be null.  plane receives

@@ -67,12 +67,78 @@ __device__ __forceinline__ Fp4Job find_job(const Fp4Launch &L, int tile) {
     return job;
 }
 
+// Closed-form round-to-nearest-even E4M3FN encode of a finite, non-negative
+// value already clamped to 448.
+__device__ __forceinline__ uint32_t e4m3_encode_positive(float m) {
+    if (m < 0.015625f) return (uint32_t)__builtin_rintf(m * 512.0f);
+    uint32_t bits = __float_as_uint(m);
+    bits += 0x7FFFFu + ((bits >> 20) & 1u);
+    return (bits >> 20) - ((127u - 7u) << 3);
+}
+
+__device__ __forceinline__ uint32_t e2m1_encode(float v) {
+    const float m = __builtin_fabsf(v);
+    const uint32_t code = (uint32_t)(m > 0.25f) + (uint32_t)(m >= 0.75f) + (uint32_t)(m > 1.25f) +
+                          (uint32_t)(m >= 1.75f) + (uint32_t)(m > 2.5f) + (uint32_t)(m >= 3.5f) +
+                          (uint32_t)(m > 5.0f);
+    return code | ((__float_as_uint(v) >> 28) & 8u);
+}
+
+__device__ __forceinline__ float e2m1_decode(uint32_t code) {
+    const uint32_t m = code & 7u;
+    // 0, .5, 1, 1.5, 2, 3, 4, 6; magnitude zero is +0 whatever the sign bit
+    const float mag = m == 0 ? 0.0f : m == 1 ? 0.5f : (1.0f + 0.5f * (float)(m & 1u)) * (float)(1u << ((m >> 1) - 1u));
+    return (code & 8u) && m != 0 ? -mag : mag;
+}
+
+// Quantise and dequantise one 16-element block (reference nvfp4.c:82-130).
+// Returns false when an element is not finite (the reference rejects the call).
+__device__ __forceinline__ bool qdq_block(const float (&v)[16], float g, uint32_t &scale_code, uint32_t (&bytes)[2],
+                                          float (&out)[16], uint32_t (&halves)[8]) {
+    float top = 0.0f;
+    bool finite = true;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const float m = __builtin_fabsf(v[i]);
+        finite = finite && (m < __builtin_inff());           // false for inf and NaN
+        if (m > top) top = m;
+    }
+    if (!finite) return false;
+    const float sixth = top * (1.0f / 6.0f);
+    float raw = g * sixth;
+    if (raw > 448.0f) raw = 448.0f;
+    scale_code = e4m3_encode_positive(raw);
+    const float scale = __builtin_amdgcn_cvt_f32_fp8((int)scale_code, 0);
+    const float to_code = scale == 0.0f ? 0.0f : g / scale;
+    const float from_code = scale / g;
+    bytes[0] = 0u; bytes[1] = 0u;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        float s = v[i] * to_code;
+        if (s > 6.0f) s = 6.0f;
+        if (s < -6.0f) s = -6.0f;
+        const uint32_t code = e2m1_encode(s);
+        bytes[i >> 3] |= code << (4 * (i & 7));
+        const float value = e2m1_decode(code);
+        out[i] = value * from_code;
+        // code value * block scale: at most six significant bits, exact in bf16
+        const uint32_t h = __float_as_uint(value * scale) >> 16;
+        if (i & 1) halves[i >> 1] |= h << 16; else halves[i >> 1] = h;
+    }
+    return true;
+}
+
 constexpr int x_batch_blocks(int S, int NB) {
     const int fit = (S == 8 ? 32 : 64) / (S * NB);
     return fit >= 16 ? 16 : fit >= 8 ? 8 : fit >= 4 ? 4 : fit >= 2 ? 2 : 1;
 }
 
-template <int S, int NB>
+// QDQ: the launch's single token is quantised and dequantised by every
+// workgroup in its prologue (the activation pass of the reference matvec,
+// nvfp4.c:228-256) into LDS, and the rows read it from there through
+// v_readfirstlane; workgroup 0 reports a non-finite activation (-1 into a
+// status word the caller cleared) and nothing is published then.
+template <int S, int NB, bool QDQ = false>
 __global__ __launch_bounds__((32 / S) * 64) void fp4_tile_kernel(const Fp4Launch L) {
     constexpr int WAVES = 32 / S;
     constexpr int THREADS = WAVES * 64;
@@ -86,12 +152,38 @@ __global__ __launch_bounds__((32 / S) * 64) void fp4_tile_kernel(const Fp4Launch
 
     __shared__ __attribute__((aligned(16))) uint8_t w_lds[W_BYTES];
     __shared__ float m_lds[2 * M_STAGE];
+    __shared__ __attribute__((aligned(16))) float x_lds[QDQ ? FP4_FUSED_MAX_COLS : 4];
+    __shared__ int x_bad;
+    static_assert(!QDQ || NB == 1, "the fused activation pass serves single-token launches");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
     const Fp4Job job = find_job(L, blockIdx.x);
+    if (QDQ) {
+        if (tid == 0) x_bad = 0;
+        __syncthreads();
+        for (int blk = tid; blk < (L.cols >> 4); blk += THREADS) {
+            const float4 *src = reinterpret_cast<const float4 *>(job.x + (size_t)blk * 16);
+            float v[16];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float4 f = src[q];
+                v[4 * q] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w;
+            }
+            uint32_t scale_code, bytes[2], halves[8];
+            float out[16];
+            if (!qdq_block(v, L.input_global_scale, scale_code, bytes, out, halves)) { x_bad = 1; continue; }
+            float4 *dst = reinterpret_cast<float4 *>(x_lds + blk * 16);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) dst[q] = make_float4(out[4 * q], out[4 * q + 1], out[4 * q + 2], out[4 * q + 3]);
+        }
+        __syncthreads();
+        const int bad = x_bad;
+        if (bad && blockIdx.x == 0 && tid == 0) *L.status = -1;        // like fp4_qdq_kernel: the caller cleared it
+        if (bad) return;                                   // uniform
+    }
     const int row0 = (blockIdx.x - job.tile0) * TILE_ROWS;
     const int rows_here = job.rows - row0 < TILE_ROWS ? job.rows - row0 : TILE_ROWS;
     const int nblk = L.cols >> 5;
@@ -148,6 +240,14 @@ __global__ __launch_bounds__((32 / S) * 64) void fp4_tile_kernel(const Fp4Launch
     issue(0);
 
     auto load_x = [&](int blk0, float (&xq)[NB][XN], int blocks) {
+        if (QDQ) {                        // wave-uniform LDS reads, broadcast into scalar registers
+            const float *xl = x_lds + blk0 * 32 + S * wave;
+#pragma unroll
+            for (int k = 0; k < XN; ++k)
+                if (k < blocks * S)
+                    xq[0][k] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(xl[(k / S) * 32 + (k % S)])));
+            return;
+        }
         const uniform_f32_ptr xg = xbase + (size_t)blk0 * 32;
 #pragma unroll
         for (int t = 0; t < NB; ++t)
@@ -249,6 +349,11 @@ __global__ __launch_bounds__((32 / S) * 64) void fp4_tile_kernel(const Fp4Launch
 template <int S>
 int launch_tiles(const Fp4Launch &L, hipStream_t stream) {
     const dim3 grid(L.total_tiles), block((32 / S) * 64);
+    if (L.qdq) {
+        if (L.tokens != 1 || L.table || L.cols > FP4_FUSED_MAX_COLS || !L.status || ((uintptr_t)L.one.x & 15)) return -1;
+        hipLaunchKernelGGL((fp4_tile_kernel<S, 1, true>), grid, block, 0, stream, L);
+        return hipGetLastError() == hipSuccess ? 0 : -1;
+    }
     switch (L.tokens) {
         case 1: hipLaunchKernelGGL((fp4_tile_kernel<S, 1>), grid, block, 0, stream, L); break;
         case 2: hipLaunchKernelGGL((fp4_tile_kernel<S, 2>), grid, block, 0, stream, L); break;
@@ -260,30 +365,6 @@ int launch_tiles(const Fp4Launch &L, hipStream_t stream) {
 }
 
 // ---------------------------------------------------------------- activation Q/DQ
-
-// Closed-form round-to-nearest-even E4M3FN encode of a finite, non-negative
-// value already clamped to 448.
-__device__ __forceinline__ uint32_t e4m3_encode_positive(float m) {
-    if (m < 0.015625f) return (uint32_t)__builtin_rintf(m * 512.0f);
-    uint32_t bits = __float_as_uint(m);
-    bits += 0x7FFFFu + ((bits >> 20) & 1u);
-    return (bits >> 20) - ((127u - 7u) << 3);
-}
-
-__device__ __forceinline__ uint32_t e2m1_encode(float v) {
-    const float m = __builtin_fabsf(v);
-    const uint32_t code = (uint32_t)(m > 0.25f) + (uint32_t)(m >= 0.75f) + (uint32_t)(m > 1.25f) +
-                          (uint32_t)(m >= 1.75f) + (uint32_t)(m > 2.5f) + (uint32_t)(m >= 3.5f) +
-                          (uint32_t)(m > 5.0f);
-    return code | ((__float_as_uint(v) >> 28) & 8u);
-}
-
-__device__ __forceinline__ float e2m1_decode(uint32_t code) {
-    const uint32_t m = code & 7u;
-    // 0, .5, 1, 1.5, 2, 3, 4, 6; magnitude zero is +0 whatever the sign bit
-    const float mag = m == 0 ? 0.0f : m == 1 ? 0.5f : (1.0f + 0.5f * (float)(m & 1u)) * (float)(1u << ((m >> 1) - 1u));
-    return (code & 8u) && m != 0 ? -mag : mag;
-}
 
 // One thread per 16-element block of one token.
 __global__ __launch_bounds__(256) void fp4_qdq_kernel(const float *__restrict__ input, int cols, int tokens,
@@ -300,39 +381,11 @@ __global__ __launch_bounds__(256) void fp4_qdq_kernel(const float *__restrict__ 
         const float4 f = src[q];
         v[4 * q] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w;
     }
-    float top = 0.0f;
-    bool finite = true;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const float m = __builtin_fabsf(v[i]);
-        finite = finite && (m < __builtin_inff());           // false for inf and NaN
-        if (m > top) top = m;
-    }
-    if (!finite) {                       // the reference rejects the whole call
+    uint32_t scale_code, bytes[2], halves[8];
+    float out[16];
+    if (!qdq_block(v, g, scale_code, bytes, out, halves)) {     // the reference rejects the whole call
         *status = -1;
         return;
-    }
-    const float sixth = top * (1.0f / 6.0f);
-    float raw = g * sixth;
-    if (raw > 448.0f) raw = 448.0f;
-    const uint32_t scale_code = e4m3_encode_positive(raw);
-    const float scale = __builtin_amdgcn_cvt_f32_fp8((int)scale_code, 0);
-    const float to_code = scale == 0.0f ? 0.0f : g / scale;
-    const float from_code = scale / g;
-    uint32_t bytes[2] = {0u, 0u};
-    float out[16];
-    uint32_t halves[8];                  // code value * block scale: at most six significant bits, exact in bf16
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        float s = v[i] * to_code;
-        if (s > 6.0f) s = 6.0f;
-        if (s < -6.0f) s = -6.0f;
-        const uint32_t code = e2m1_encode(s);
-        bytes[i >> 3] |= code << (4 * (i & 7));
-        const float value = e2m1_decode(code);
-        out[i] = value * from_code;
-        const uint32_t h = __float_as_uint(value * scale) >> 16;
-        if (i & 1) halves[i >> 1] |= h << 16; else halves[i >> 1] = h;
     }
     if (scales) scales[item] = (uint8_t)scale_code;
     if (packed) reinterpret_cast<uint2 *>(packed)[item] = make_uint2(bytes[0], bytes[1]);

@@ -69,6 +69,7 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_q4_matmul_dev, i, vp, vp, vp, i, i, i, vp, vp, vp, vp)
     _sig(lib.salt_mi355_nvfp4_qdq_dev, i, vp, i, i, f, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_nvfp4_matvec_dev, i, vp, vp, f, i, i, i, vp, vp, i, vp)
+    _sig(lib.salt_mi355_nvfp4_matvec_qdq_dev, i, vp, vp, f, f, i, i, vp, vp, vp, i, vp)
     _sig(lib.salt_mi355_nvfp4_matmul_workspace_bytes, sz, i, i, i)
     _sig(lib.salt_mi355_nvfp4_matmul_dev, i, vp, vp, f, f, i, i, i, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_router_topk_dev, i, vp, vp, i, i, i, vp, vp, vp, vp)
@@ -197,6 +198,21 @@ def nvfp4_matvec(packed: np.ndarray, scales: np.ndarray, divisor: float, R: int,
           "nvfp4_matvec_dev")
     check(lib.salt_mi355_stream_sync(stream), "sync")
     return int(st.to_host(np.int32)[0]), dy.to_host(np.float32).reshape(B, R)
+
+
+def nvfp4_matvec_one_launch(packed: np.ndarray, scales: np.ndarray, divisor: float, R: int, C_: int, x: np.ndarray,
+                            input_global_scale: float = 64.0, chains: int = 0):
+    """The reference matvec of one token with the activation pass inside the
+    rows' launch.  Returns (status, y[R]); y stays 0xFF-filled when rejected."""
+    lib = init()
+    x = np.ascontiguousarray(x, np.float32).reshape(C_)
+    dw, ds, dx = DeviceBuffer.from_host(packed), DeviceBuffer.from_host(scales), DeviceBuffer.from_host(x)
+    dy, st = DeviceBuffer(R * 4, fill=0xFF), DeviceBuffer(4, fill=0)
+    stream = lib.salt_mi355_stream()
+    check(lib.salt_mi355_nvfp4_matvec_qdq_dev(dw.ptr, ds.ptr, divisor, input_global_scale, R, C_, dx.ptr, dy.ptr, st.ptr,
+                                              chains, stream), "nvfp4_matvec_qdq_dev")
+    check(lib.salt_mi355_stream_sync(stream), "sync")
+    return int(st.to_host(np.int32)[0]), dy.to_host(np.float32)
 
 
 def router_topk(logits: np.ndarray, scale: np.ndarray, topk: int, sorted_by_id: bool = False):

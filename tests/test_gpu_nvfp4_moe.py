@@ -82,6 +82,24 @@ def test_matvec_matches_checker(gpu, oracle, R, Cc, B, divisor, chains):
     assert np.array_equal(bits(got), bits(want))
 
 
+@pytest.mark.parametrize("chains", [0, 8, 4, 2])
+@pytest.mark.parametrize("R,Cc,g", [(64, 64, 64.0), (130, 2816, 8.0), (65, 8192, 64.0), (1, 32, 1.0), (704, 704, 100.0)])
+def test_matvec_with_activation_pass_in_one_launch(gpu, oracle, R, Cc, g, chains):
+    print(f"nvfp4 one launch R={R} C={Cc} g={g} chains={chains}", flush=True)
+    packed, scales = synth.nvfp4_tensor(R, Cc, R * 7 + Cc)
+    x = synth.activations(Cc, 1, R + 11)[0]
+    x[:3] = [0.0, -0.0, 1e-30]
+    want = np.zeros(R, np.float32)
+    xp = np.zeros(Cc // 2, np.uint8); xsc = np.zeros(Cc // 16, np.uint8); xd = np.zeros(Cc, np.float32)
+    assert oracle.orc_nvfp4_matvec(ptr(packed), ptr(scales), 2688.0, g, R, Cc, ptr(x), ptr(want), ptr(xp), ptr(xsc),
+                                   ptr(xd)) == 0
+    st, got = gpu.nvfp4_matvec_one_launch(packed, scales, 2688.0, R, Cc, x, g, chains)
+    assert st == 0 and np.array_equal(bits(got), bits(want))
+    bad = x.copy(); bad[Cc - 1] = np.inf
+    st, got = gpu.nvfp4_matvec_one_launch(packed, scales, 2688.0, R, Cc, bad, g, chains)
+    assert st == -1 and (got.view(np.uint32) == 0xFFFFFFFF).all()
+
+
 def test_matvec_nan_scale_codes_and_negative_divisor(gpu, oracle):
     R, Cc = 64, 128
     packed, scales = synth.nvfp4_tensor(R, Cc, 5)
