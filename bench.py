@@ -38,7 +38,7 @@ SWEEP = [(2816, 2816), (16384, 2816), (2816, 8192)]        # (R, C) = (N, K)
 INSTANCE_BYTES = 640e6                                      # distinct weight bytes per launch
 # HBM bytes one launch of the default workload moves, from FETCH_SIZE / WRITE_SIZE counter runs scaled by a copy of
 # known size (profiles/q4_tile_kernel_decode_sweep_b1.md); valid for the default instance counts only.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 663_509_000
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 661_320_000
 
 
 class Events:
