@@ -241,6 +241,7 @@ int moe_prefill_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_
     const int nt_up = (g.routed + tn_up - 1) / tn_up, nt_down = (g.hidden + tn_down - 1) / tn_down;
     // plan and counts are adjacent 256-byte aligned pieces of the workspace: one clear covers both
     static_assert(sizeof(PrefillPlan) <= 256, "the plan fits the first aligned piece");
+    if ((uint8_t *)w.counts != (uint8_t *)w.plan + 256) return -1;
     if (clear_words_launch(w.plan, 64 + (size_t)g.n_experts, stream) != 0) return -1;
     hipLaunchKernelGGL(group_count_kernel, dim3((tokens + 255) / 256), dim3(256), 0, stream, selected, weights, tokens,
                        g.topk, g.n_experts, w.counts, w.plan);

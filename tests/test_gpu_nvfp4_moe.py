@@ -213,3 +213,26 @@ def test_moe_decode_step_fresh_logits_and_rejection(gpu, oracle):
         assert np.array_equal(bits(eo), bits(oeo)) and np.array_equal(bits(y), bits(oy))
     logits = synth.router_logits(E, 1).copy(); logits[3] = np.inf
     assert layer.step(logits, scale, x)[0] == -1
+
+
+@pytest.mark.parametrize("E,K,H,F,why", [
+    (520, 4, 128, 64, "more experts than the fused prologue holds: router, gate/up, activate, down, reduce as five launches"),
+    (16, 16, 2816, 2048, "more than two tiles per compute unit: eight waves per tile in both fused launches"),
+    (24, 5, 192, 4160, "d_ff beyond the LDS activation buffer of the fused down launch: five launches"),
+])
+def test_moe_decode_step_other_launch_shapes(gpu, oracle, E, K, H, F, why):
+    print(f"moe step E={E} K={K} H={H} F={F}: {why}", flush=True)
+    pool = synth.expert_pool(E, H, F, E + K)
+    layer = gpu.MoeLayer(pool, E, H, F, K)
+    g = ExpertGeometry(H, F)
+    scale = synth.rng(2).uniform(0.5, 2.0, E).astype(np.float32)
+    logits = synth.router_logits(E, 40 + E); x = synth.activations(H, 1, 41 + E)[0]
+    st, sel, w, eo, y = layer.step(logits, scale, x)
+    osel = np.zeros(K, np.int32); ow = np.zeros(K, np.float32)
+    oeo = np.zeros((K, H), np.float32); oy = np.zeros(H, np.float32)
+    assert oracle.orc_moe_decode_step(C.byref(g), ptr(pool), E, K, ptr(logits), ptr(scale), ptr(x), ptr(osel),
+                                      ptr(ow), ptr(oeo), ptr(oy), host_threads()) == 0
+    assert st == 0 and np.array_equal(sel, osel) and np.array_equal(bits(w), bits(ow))
+    assert np.array_equal(bits(eo), bits(oeo)) and np.array_equal(bits(y), bits(oy))
+    logits[E - 1] = np.nan
+    assert layer.step(logits, scale, x)[0] == -1
