@@ -139,28 +139,34 @@ __global__ __launch_bounds__(MAX_EXPERTS) void group_scan_kernel(const ScanArgs 
     }
 }
 
-// one workgroup per expert: its (token, rank) pairs in token-major order.  A
-// thread owns a contiguous run of pairs, so the rank of a match is the number
-// of matches in earlier runs plus those before it in its own.
+// one wave per expert: its (token, rank) pairs in token-major order.  The wave
+// walks the selection 64 pairs at a time (one coalesced load); a match's place
+// is the matches before the chunk plus the matching lanes below it, so no
+// workgroup barrier is needed.
 __global__ __launch_bounds__(256) void group_fill_kernel(const int *__restrict__ selected, int pairs, int topk,
-                                                         const int *__restrict__ offsets,
+                                                         const int *__restrict__ offsets, int n_experts,
                                                          const PrefillPlan *__restrict__ plan,
                                                          int *__restrict__ row_pairs, int *__restrict__ pair_rows) {
-    __shared__ int s_wave[4];
     if (plan->status != 0) {            // keep the gather in range: every grouped row reads token 0
         for (int p = blockIdx.x * 256 + threadIdx.x; p < pairs; p += gridDim.x * 256) row_pairs[p] = 0;
         return;
     }
-    const int e = blockIdx.x;
-    const int n = offsets[e + 1] - offsets[e];
-    if (n == 0) return;                 // uniform
-    const int run = (pairs + 255) / 256;
-    const int first = threadIdx.x * run, last = first + run < pairs ? first + run : pairs;
-    int mine = 0;
-    for (int p = first; p < last; ++p) mine += selected[p] == e;
-    int at = offsets[e] + block_exclusive_scan(mine, s_wave, nullptr);
-    for (int p = first; p < last && mine > 0; ++p)
-        if (selected[p] == e) { row_pairs[at] = p; pair_rows[p] = at; ++at; --mine; }
+    const int lane = threadIdx.x & 63;
+    const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (e >= n_experts) return;         // uniform per wave
+    int at = offsets[e];
+    if (offsets[e + 1] == at) return;
+    for (int first = 0; first < pairs; first += 64) {
+        const int p = first + lane;
+        const bool hit = p < pairs && selected[p] == e;
+        const unsigned long long mask = __ballot(hit);
+        if (hit) {
+            const int row = at + __popcll(mask & ((1ull << lane) - 1ull));
+            row_pairs[row] = p;
+            pair_rows[p] = row;
+        }
+        at += __popcll(mask);
+    }
 }
 
 // out[token][d] = sum over rank of down[row(token, rank)][d] * weight, from +0, rank ascending
@@ -254,8 +260,8 @@ int moe_prefill_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_
     a.gate = w.gate; a.up = w.up; a.down = w.down;
     hipLaunchKernelGGL(group_scan_kernel, dim3(1), dim3(MAX_EXPERTS), 0, stream, a);
     int *rp = row_pairs ? row_pairs : w.row_pairs;
-    hipLaunchKernelGGL(group_fill_kernel, dim3(g.n_experts), dim3(256), 0, stream, selected, rows, g.topk, w.offsets,
-                       w.plan, rp, w.pair_rows);
+    hipLaunchKernelGGL(group_fill_kernel, dim3((g.n_experts + 3) / 4), dim3(256), 0, stream, selected, rows, g.topk,
+                       w.offsets, g.n_experts, w.plan, rp, w.pair_rows);
     if (hipGetLastError() != hipSuccess) return -1;
 
     // The inputs are split once per token; the matmul gathers the rows of an
