@@ -284,6 +284,21 @@ def main():
         ms_fp4 = timed(lib, stream, events, fp4_step, 2, 10) / G
         extra["nvfp4_8192_matvec_us"] = round(ms_fp4 * 1e3, 2)
         extra["nvfp4_8192_gbps"] = round(synth.nvfp4_bytes(R, Cc, 1) / (ms_fp4 * 1e-3) / 1e9, 1)
+        # the same 16 instances as ONE multi-matrix launch after one activation pass: the kernel's streaming rate
+        xq = gpu.DeviceBuffer(Cc * 4)
+        ys16 = gpu.DeviceBuffer(G * R * 4)
+        fjobs = (gpu.Fp4Job * G)()
+        for g in range(G):
+            fjobs[g] = gpu.Fp4Job(w.at(g * per), w.at(g * per + packed.nbytes), 2688.0, xq.ptr, ys16.at(g * R * 4), R)
+
+        def fp4_sweep_step(s):
+            lib.salt_mi355_nvfp4_qdq_dev(x.ptr, Cc, 1, 64.0, None, None, xq.ptr, st.ptr, s)
+            if lib.salt_mi355_nvfp4_jobs_dev(fjobs, G, Cc, 1, 0, s) != 0:
+                raise RuntimeError(lib.salt_mi355_last_error().decode())
+
+        ms_sw = timed(lib, stream, events, fp4_sweep_step, 2, 10)
+        extra["nvfp4_8192_x16_one_launch_gbps"] = round(G * synth.nvfp4_bytes(R, Cc, 1) / (ms_sw * 1e-3) / 1e9, 1)
+        del xq, ys16
         # NVFP4 8192 x 8192, batch 256, on the matrix cores (tolerance class); activation pass included
         B = 256
         xb = gpu.DeviceBuffer.from_host(synth.activations(Cc, B, 42))

@@ -130,6 +130,22 @@ int salt_mi355_nvfp4_matvec_dev(const void *packed, const void *scales, float st
                                 int R, int C, int B, const float *xs, float *ys,
                                 int chains_per_lane, void *stream);
 
+/* Many NVFP4 matrices in one launch (the shape of reference
+ * salt_gpu_nvfp4_mixed_batch, gpu.h:55-59): job j multiplies its own
+ * R_j x C matrix with its own tokens, the activation used as given (pass the
+ * dequantised output of salt_mi355_nvfp4_qdq_dev for the reference matvec).
+ * `jobs` is a HOST array; the library copies it to the device on `stream`. */
+typedef struct SaltMi355Fp4Job {
+    const void *packed;
+    const void *scales;
+    float stored_divisor;
+    const float *xs;         /* device, [tokens][C] */
+    float *ys;               /* device, [tokens][rows] */
+    int rows;
+} SaltMi355Fp4Job;
+int salt_mi355_nvfp4_jobs_dev(const SaltMi355Fp4Job *jobs, int njobs, int C, int tokens,
+                              int chains_per_lane, void *stream);
+
 /* The reference matvec of one token in one launch (reference
  * salt_nvfp4_matvec_reference, nvfp4.c:228-256): every workgroup quantises
  * and dequantises the activation x[C] itself (nvfp4.c:82-130) and computes its

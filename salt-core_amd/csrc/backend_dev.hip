@@ -4,6 +4,8 @@
 #include <math.h>
 #include <string.h>
 
+#include <vector>
+
 using namespace mi355;
 
 extern "C" {
@@ -145,6 +147,56 @@ int salt_mi355_nvfp4_matmul_dev(const void *packed, const void *scales, float st
         hip_ok(hipStreamSynchronize(s), "nvfp4 matmul sync") != 0)
         return -1;
     if (status != 0) { set_error("nvfp4 matmul: non-finite activation"); return -1; }
+    return 0;
+}
+
+int salt_mi355_nvfp4_jobs_dev(const SaltMi355Fp4Job *jobs, int njobs, int C, int tokens, int chains, void *stream_handle) {
+    hipStream_t stream = (hipStream_t)stream_handle;
+    if (!g_state.ready) { set_error("nvfp4 jobs: library not initialised"); return -1; }
+    if (!g_state.fp8_is_ocp) { set_error("nvfp4: this device's fp8 converter is not OCP E4M3FN"); return -1; }
+    if (!jobs || njobs < 1 || C < 32 || (C & 31) || tokens < 1 ||
+        (chains != 0 && chains != 8 && chains != 4 && chains != 2)) {
+        set_error("nvfp4 jobs: bad arguments (C must be a multiple of 32)");
+        return -1;
+    }
+    for (int j = 0; j < njobs; ++j)
+        if (!jobs[j].packed || !jobs[j].scales || !jobs[j].xs || !jobs[j].ys || jobs[j].rows < 1 ||
+            !isfinite(jobs[j].stored_divisor) || jobs[j].stored_divisor == 0.0f || ((uintptr_t)jobs[j].packed & 15) ||
+            ((uintptr_t)jobs[j].scales & 1) || ((uintptr_t)jobs[j].xs & 3) || ((uintptr_t)jobs[j].ys & 3)) {
+            set_error("nvfp4 jobs: job %d is malformed (packed 16-byte aligned, non-zero finite divisor)", j);
+            return -1;
+        }
+    std::vector<Fp4Job> table((size_t)njobs);
+    for (int first = 0; first < tokens; first += 4) {
+        int tiles = 0;
+        for (int j = 0; j < njobs; ++j) {
+            Fp4Job &f = table[(size_t)j];
+            f.packed = (const uint8_t *)jobs[j].packed;
+            f.scales = (const uint8_t *)jobs[j].scales;
+            f.x = jobs[j].xs + (size_t)first * C;
+            f.y = jobs[j].ys + (size_t)first * jobs[j].rows;
+            f.weight_global_scale = 1.0f / jobs[j].stored_divisor;
+            f.rows = jobs[j].rows;
+            f.tile0 = tiles;
+            f.x_stride = C;
+            tiles += (jobs[j].rows + 63) / 64;
+        }
+        Fp4Launch launch;
+        memset(&launch, 0, sizeof launch);
+        launch.njobs = njobs; launch.cols = C; launch.total_tiles = tiles;
+        launch.tokens = tokens - first < 4 ? tokens - first : 4;
+        State::TableSlot *slot = nullptr;
+        if (njobs == 1) {
+            launch.one = table[0];
+        } else {
+            slot = table_acquire(table.data(), table.size() * sizeof(Fp4Job), stream);
+            if (!slot) return -1;
+            launch.table = (const Fp4Job *)slot->device;
+        }
+        const int rc = fp4_launch(launch, chains, stream);
+        table_release(slot, stream);
+        if (rc != 0) { set_error("nvfp4 jobs: kernel launch failed"); return -1; }
+    }
     return 0;
 }
 

@@ -1099,23 +1099,37 @@ int run_fp4_jobs(std::vector<Fp4HostJob> &jobs, int C) {
     if (clear_words_launch(st_dev, 1, g_state.stream) != 0) return -1;
     std::vector<OutputCopy> copies;
     SaltGpuBatchStatsV2 &stats = e.stats;
+    // Several single-token jobs: one activation pass per job, then all rows in ONE multi-matrix launch (streaming
+    // rate instead of one latency-bound launch per matrix).  Otherwise job by job; a single token of a single job
+    // runs its activation pass inside the rows' launch.
+    bool all_single = jobs.size() > 1;
+    for (const Fp4HostJob &j : jobs) all_single = all_single && j.tokens == 1;
+    std::vector<SaltMi355Fp4Job> table;
     for (Fp4HostJob &j : jobs) {
         const size_t xin = (size_t)j.tokens * C, yout = (size_t)j.tokens * j.rows;
         float *x_dev = upload_activations(j.x_host, xin);
         if (!x_dev) return -1;
         float *dq_dev = (float *)device_take(xin * 4);
         uint8_t *y_dev = device_take(yout * 4), *y_pin = pinned_take(yout * 4);
-        const bool one_launch = j.tokens == 1 && C <= FP4_FUSED_MAX_COLS;   // the activation pass runs inside the rows' launch
+        const bool one_launch = !all_single && j.tokens == 1 && C <= FP4_FUSED_MAX_COLS;
         if (one_launch) {
             if (salt_mi355_nvfp4_matvec_qdq_dev(j.packed, j.scales, j.tensor->stored_divisor,
                                                 j.tensor->input_global_scale, j.rows, C, x_dev, (float *)y_dev, st_dev, 0,
                                                 g_state.stream) != 0)
                 return -1;
-        } else if (salt_mi355_nvfp4_qdq_dev(x_dev, C, j.tokens, j.tensor->input_global_scale, nullptr, nullptr, dq_dev,
-                                            st_dev, g_state.stream) != 0 ||
-                   salt_mi355_nvfp4_matvec_dev(j.packed, j.scales, j.tensor->stored_divisor, j.rows, C, j.tokens, dq_dev,
-                                               (float *)y_dev, 0, g_state.stream) != 0) {
-            return -1;
+        } else {
+            if (salt_mi355_nvfp4_qdq_dev(x_dev, C, j.tokens, j.tensor->input_global_scale, nullptr, nullptr, dq_dev,
+                                         st_dev, g_state.stream) != 0)
+                return -1;
+            if (all_single) {
+                SaltMi355Fp4Job t;
+                t.packed = j.packed; t.scales = j.scales; t.stored_divisor = j.tensor->stored_divisor;
+                t.xs = dq_dev; t.ys = (float *)y_dev; t.rows = j.rows;
+                table.push_back(t);
+            } else if (salt_mi355_nvfp4_matvec_dev(j.packed, j.scales, j.tensor->stored_divisor, j.rows, C, j.tokens,
+                                                   dq_dev, (float *)y_dev, 0, g_state.stream) != 0) {
+                return -1;
+            }
         }
         e.pending.push_back({y_pin, j.y_host, yout * 4});
         copies.push_back({y_dev, y_pin, yout * 4});
@@ -1124,7 +1138,11 @@ int run_fp4_jobs(std::vector<Fp4HostJob> &jobs, int C) {
         stats.nvfp4_activation_input_bytes += xin * 4;
         stats.nvfp4_activation_qdq_bytes += xin * 4;
         stats.nvfp4_projection_output_bytes += yout * 4;
-        stats.nvfp4_kernel_launches += one_launch ? 1 : 2 + (uint64_t)((j.tokens - 1) / 4);
+        stats.nvfp4_kernel_launches += one_launch ? 1 : all_single ? 1 : 2 + (uint64_t)((j.tokens - 1) / 4);
+    }
+    if (all_single) {
+        if (salt_mi355_nvfp4_jobs_dev(table.data(), (int)table.size(), C, 1, 0, g_state.stream) != 0) return -1;
+        stats.nvfp4_kernel_launches += 1;
     }
     uint8_t *st_pin = pinned_take(4);
     for (const OutputCopy &c : copies)

@@ -16,6 +16,11 @@ class Q4Job(C.Structure):
     _fields_ = [("vals", vp), ("scales", vp), ("biases", vp), ("xs", vp), ("ys", vp), ("rows", C.c_int)]
 
 
+class Fp4Job(C.Structure):
+    _fields_ = [("packed", vp), ("scales", vp), ("stored_divisor", C.c_float), ("xs", vp), ("ys", vp),
+                ("rows", C.c_int)]
+
+
 _lib = None
 
 INCLUDE_DIR = Path(__file__).resolve().parent.parent / "include"
@@ -69,6 +74,7 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_q4_matmul_dev, i, vp, vp, vp, i, i, i, vp, vp, vp, vp)
     _sig(lib.salt_mi355_nvfp4_qdq_dev, i, vp, i, i, f, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_nvfp4_matvec_dev, i, vp, vp, f, i, i, i, vp, vp, i, vp)
+    _sig(lib.salt_mi355_nvfp4_jobs_dev, i, C.POINTER(Fp4Job), i, i, i, i, vp)
     _sig(lib.salt_mi355_nvfp4_matvec_qdq_dev, i, vp, vp, f, f, i, i, vp, vp, vp, i, vp)
     _sig(lib.salt_mi355_nvfp4_matmul_workspace_bytes, sz, i, i, i)
     _sig(lib.salt_mi355_nvfp4_matmul_dev, i, vp, vp, f, f, i, i, i, vp, vp, vp, vp, vp)

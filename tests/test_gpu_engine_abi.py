@@ -394,6 +394,7 @@ def test_nvfp4_engine_entry_points(eng, oracle, pkg):
         return out
 
     xs = synth.activations(Cc, 5, 62)
+    bad_row = xs[0:1].copy(); bad_row[0, 5] = np.nan
     y = np.zeros(R, np.float32)
     assert eng.salt_gpu_nvfp4_matvec(key, R, Cc, ptr(xs[0]), ptr(y)) == 0, err(pkg)
     assert np.array_equal(bits(y), bits(want(xs[:1])[0]))
@@ -405,6 +406,17 @@ def test_nvfp4_engine_entry_points(eng, oracle, pkg):
                                   abi.ptr_array([y1, y2]), (C.c_int * 2)(2, 1), R, Cc, 2)
     assert rc == 0, err(pkg)
     assert np.array_equal(bits(y1), bits(want(xs[0:2]))) and np.array_equal(bits(y2), bits(want(xs[4:5])))
+    # three single-token jobs: one multi-matrix launch behind the same entry point
+    ys3 = [np.zeros((1, R), np.float32) for _ in range(3)]
+    rc = eng.salt_gpu_nvfp4_batch(abi.ptr_array([key, key, key]), abi.ptr_array([xs[1:2], xs[3:4], xs[2:3]]),
+                                  abi.ptr_array(ys3), (C.c_int * 3)(1, 1, 1), R, Cc, 3)
+    assert rc == 0, err(pkg)
+    for got, t in zip(ys3, (1, 3, 2)):
+        assert np.array_equal(bits(got), bits(want(xs[t:t + 1])))
+    ys3[1][:] = 5.0
+    rc = eng.salt_gpu_nvfp4_batch(abi.ptr_array([key, key, key]), abi.ptr_array([xs[1:2], bad_row, xs[2:3]]),
+                                  abi.ptr_array(ys3), (C.c_int * 3)(1, 1, 1), R, Cc, 3)
+    assert rc == -1 and (ys3[1] == 5.0).all()                                            # nothing published
     assert eng.salt_gpu_nvfp4_matvec(0x9999, R, Cc, ptr(xs[0]), ptr(y)) == -1            # unknown key
     assert eng.salt_gpu_nvfp4_matvec(key, R + 1, Cc, ptr(xs[0]), ptr(y)) == -1           # geometry mismatch
     bad = xs[0].copy(); bad[17] = np.inf

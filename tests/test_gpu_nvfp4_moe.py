@@ -100,6 +100,35 @@ def test_matvec_with_activation_pass_in_one_launch(gpu, oracle, R, Cc, g, chains
     assert st == -1 and (got.view(np.uint32) == 0xFFFFFFFF).all()
 
 
+@pytest.mark.parametrize("tokens", [1, 3, 6])
+def test_many_matrices_in_one_launch(gpu, oracle, tokens):
+    print(f"nvfp4 jobs tokens={tokens}", flush=True)
+    Cc = 704
+    rows = [64, 130, 1, 700, 65]
+    lib = gpu.init()
+    stream = lib.salt_mi355_stream()
+    jobs = (gpu.Fp4Job * len(rows))()
+    keep, wants = [], []
+    for j, R in enumerate(rows):
+        packed, scales = synth.nvfp4_tensor(R, Cc, 50 + j)
+        xs = synth.activations(Cc, tokens, 60 + j)
+        divisor = [1.0, 2688.0, -3.0, 0.5, 7.0][j]
+        want = np.zeros((tokens, R), np.float32)
+        for t in range(tokens):
+            assert oracle.orc_nvfp4_matvec_weights_only(ptr(packed), ptr(scales), divisor, R, Cc, ptr(xs[t]),
+                                                        ptr(want[t])) == 0
+        dp, ds, dx = (gpu.DeviceBuffer.from_host(a) for a in (packed, scales, xs))
+        dy = gpu.DeviceBuffer(tokens * R * 4, fill=0xFF)
+        keep.append((dp, ds, dx, dy)); wants.append(want)
+        jobs[j] = gpu.Fp4Job(dp.ptr, ds.ptr, divisor, dx.ptr, dy.ptr, R)
+    assert lib.salt_mi355_nvfp4_jobs_dev(jobs, len(rows), Cc, tokens, 0, stream) == 0
+    assert lib.salt_mi355_stream_sync(stream) == 0
+    for (dp, ds, dx, dy), want in zip(keep, wants):
+        assert np.array_equal(bits(dy.to_host(np.float32).reshape(want.shape)), bits(want))
+    jobs[1].stored_divisor = 0.0
+    assert lib.salt_mi355_nvfp4_jobs_dev(jobs, len(rows), Cc, tokens, 0, stream) == -1
+
+
 def test_matvec_nan_scale_codes_and_negative_divisor(gpu, oracle):
     R, Cc = 64, 128
     packed, scales = synth.nvfp4_tensor(R, Cc, 5)
