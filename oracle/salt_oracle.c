@@ -12,6 +12,10 @@
  *   orc_e2m1 / orc_e4m3fn / encoders / orc_nvfp4_qdq / orc_nvfp4_matvec
  *       reference golden bytes and bit patterns (tests/test_nvfp4.c:28-117),
  *       OCP FP8/FP4 tables from torch, the compiled reference and fixtures.
+ *   orc_bf16_matvec / orc_q8_matvec   the compiled reference in both its
+ *       scalar and SIMD realisation, a step-by-step numpy float32
+ *       emulation, exact closed forms (powers of two against the column
+ *       index; byte sums; a single left-to-right chain).
  *   orc_expf / orc_tanhf / orc_gelu_tanh   no vectors exist in the reference
  *       tree; pinned by fixtures generated from the compiled reference and by
  *       closeness to libm (a dropped Horner term or a wrong constant fails).
@@ -369,6 +373,52 @@ int orc_nvfp4_matvec_weights_only(const uint8_t *packed,
     for (int r = 0; r < R; r++)
         output[r] = orc_nvfp4_row(packed, scales, wg, r, C, x);
     return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* bf16 and 8-bit affine matvecs                                       */
+/* ------------------------------------------------------------------ */
+
+void orc_bf16_matvec(const uint16_t *W, int R, int C, const float *x,
+                     const float *bias, float *y) {
+    for (int r = 0; r < R; r++) {
+        const uint16_t *row = W + (size_t)r * (size_t)C;
+        float a[8];
+        for (int j = 0; j < 8; j++) a[j] = 0.0f;
+        int c = 0;
+        for (; c + 7 < C; c += 8)
+            for (int j = 0; j < 8; j++) {
+                float p = orc_bf16(row[c + j]) * x[c + j];
+                a[j] = a[j] + p;
+            }
+        float even = (a[0] + a[2]) + (a[4] + a[6]);
+        float odd = (a[1] + a[3]) + (a[5] + a[7]);
+        float s = even + odd;
+        for (; c < C; c++) {
+            float p = orc_bf16(row[c]) * x[c];
+            s = s + p;
+        }
+        y[r] = s + (bias ? bias[r] : 0.0f);
+    }
+}
+
+void orc_q8_matvec(const void *vals, const void *scales, const void *biases,
+                   int R, int C, const float *x, float *y) {
+    const unsigned char *bytes = (const unsigned char *)vals;
+    for (int r = 0; r < R; r++) {
+        float acc = 0.0f;
+        for (int c = 0; c < C; c++) {
+            size_t k = (size_t)r * (size_t)C + (size_t)c;
+            size_t g = k / ORC_GROUP;
+            float s = orc_bf16(ld16(scales, g));
+            float b = biases ? orc_bf16(ld16(biases, g)) : 0.0f;
+            float w = (float)bytes[k] * s;
+            w = w + b;
+            float p = w * x[c];
+            acc = acc + p;
+        }
+        y[r] = acc;
+    }
 }
 
 /* ------------------------------------------------------------------ */

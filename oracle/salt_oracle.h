@@ -46,6 +46,21 @@ int orc_q4_matvec_threads(const void *vals, const void *scales,
                           const void *biases, int R, int C, const float *x,
                           float *y, int threads);
 
+/* ---- bf16 and 8-bit affine matvecs (the LM head and the router gates) */
+
+/* reference src/kernels.c:139-174 (salt_bf16_matvec, scalar body): eight
+ * chains a[c % 8] over the 8-aligned part of the row, each p = fl(w*x),
+ * a = fl(a + p); s = ((a0+a2)+(a4+a6)) + ((a1+a3)+(a5+a7)); the columns past
+ * the last multiple of eight are added to s in order; y = s + (bias ? bias[r]
+ * : 0.0f). */
+void orc_bf16_matvec(const uint16_t *W, int R, int C, const float *x,
+                     const float *bias, float *y);
+/* reference src/kernels.c:343-370 (salt_q8_matvec): one chain per row,
+ * acc = fl(acc + fl(fl(fl(q*s) + b) * x[c])) over all columns in order; the
+ * value of flat element k is byte k of vals, its scale group k / 64. */
+void orc_q8_matvec(const void *vals, const void *scales, const void *biases,
+                   int R, int C, const float *x, float *y);
+
 /* ---- NVFP4: packed E2M1 codes, E4M3FN block scale per 16, fp32 divisor */
 
 /* reference src/nvfp4.c:19-23 */

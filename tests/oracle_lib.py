@@ -51,6 +51,8 @@ def load_oracle() -> C.CDLL:
     _sig(lib.orc_q4_matvec_rows, i, vp, vp, vp, i, i, vp, vp, i, i)
     _sig(lib.orc_q4_matvec_batch, i, vp, vp, vp, i, i, i, vp, vp)
     _sig(lib.orc_q4_matvec_threads, i, vp, vp, vp, i, i, vp, vp, i)
+    _sig(lib.orc_bf16_matvec, None, vp, i, i, vp, vp, vp)
+    _sig(lib.orc_q8_matvec, None, vp, vp, vp, i, i, vp, vp)
     _sig(lib.orc_e2m1, f, C.c_uint8)
     _sig(lib.orc_e4m3fn, f, C.c_uint8)
     _sig(lib.orc_e4m3fn_encode, i, f, c_u8p)
@@ -91,6 +93,8 @@ def load_reference() -> C.CDLL | None:
     _sig(lib.salt_q4_matvec_status, i, vp, vp, vp, i, i, vp, vp)
     _sig(lib.salt_q4_matvec_rows_status, i, vp, vp, vp, i, i, vp, vp, i, i)
     _sig(lib.salt_q4_matvec_batch_rows, i, vp, vp, vp, i, i, i, vp, vp, i, i)
+    _sig(lib.salt_bf16_matvec, None, vp, i, i, vp, vp, vp)
+    _sig(lib.salt_q8_matvec, None, vp, vp, vp, i, i, vp, vp)
     _sig(lib.salt_kernels_set_simd, None, i)
     _sig(lib.salt_kernels_set_in_expert, None, i)
     _sig(lib.salt_nvfp4_e2m1, f, C.c_uint8)
