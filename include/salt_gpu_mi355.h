@@ -173,6 +173,27 @@ int salt_mi355_nvfp4_matmul_dev(const void *packed, const void *scales,
                                 int R, int C, int B, const float *xs, float *ys,
                                 int *status_dev, void *workspace, void *stream);
 
+/* ---- bf16 and 8-bit affine matvecs, device-resident --------------------- */
+
+/* reference salt_bf16_matvec (src/kernels.c:139-174), the arithmetic behind
+ * salt_gpu_bf16_matvec (include/salt/gpu.h:63-65, src/gpu_hip.cpp:1308-1341,
+ * 4591-4622): the language-model head.  weights is [R][C] bf16, xs [B][C],
+ * ys [B][R], bias [R] or NULL.  Eight column chains per row, the reference's
+ * fold tree, separately rounded products and sums: bit-exact.  Any C and any
+ * weight address are accepted; C % 8 == 0 with 16-byte aligned weights runs
+ * the streaming kernel. */
+int salt_mi355_bf16_matvec_dev(const void *weights, int R, int C, int B,
+                               const float *xs, const float *bias, float *ys,
+                               void *stream);
+
+/* reference salt_q8_matvec (src/kernels.c:343-370), the arithmetic behind
+ * salt_gpu_q8_matvec / salt_gpu_q8_batch (include/salt/gpu.h:37-39, 89-94):
+ * router gates.  vals is [R][C] bytes, scales and biases (or NULL) one bf16
+ * per 64 flat elements.  One left-to-right chain per row: bit-exact. */
+int salt_mi355_q8_matvec_dev(const void *vals, const void *scales,
+                             const void *biases, int R, int C, int B,
+                             const float *xs, float *ys, void *stream);
+
 /* ---- MoE decode layer-step, device-resident ----------------------------- */
 
 /* reference salt_gemma4_router_topk (gemma4.c:132-186).  sorted_by_id = 0

@@ -229,6 +229,40 @@ int salt_mi355_nvfp4_matvec_qdq_dev(const void *packed, const void *scales, floa
     return 0;
 }
 
+int salt_mi355_bf16_matvec_dev(const void *weights, int R, int C, int B, const float *xs, const float *bias, float *ys,
+                                void *stream) {
+    if (!g_state.ready) { set_error("bf16 matvec: library not initialised"); return -1; }
+    if (!weights || !xs || !ys || R < 1 || C < 1 || B < 1 || ((uintptr_t)xs & 3) || ((uintptr_t)ys & 3) ||
+        ((uintptr_t)bias & 3)) {
+        set_error("bf16 matvec: bad arguments");
+        return -1;
+    }
+    Bf16Launch launch;
+    launch.weights = (const uint16_t *)weights;
+    launch.x = xs; launch.bias = bias; launch.y = ys;
+    launch.rows = R; launch.cols = C; launch.tokens = B;
+    launch.x_stride = C; launch.y_stride = R;
+    if (bf16_launch(launch, (hipStream_t)stream) != 0) { set_error("bf16 matvec: launch failed"); return -1; }
+    return 0;
+}
+
+int salt_mi355_q8_matvec_dev(const void *vals, const void *scales, const void *biases, int R, int C, int B,
+                              const float *xs, float *ys, void *stream) {
+    if (!g_state.ready) { set_error("q8 matvec: library not initialised"); return -1; }
+    if (!vals || !scales || !xs || !ys || R < 1 || C < 1 || B < 1 || B > 65535 || ((uintptr_t)xs & 3) ||
+        ((uintptr_t)ys & 3)) {
+        set_error("q8 matvec: bad arguments");
+        return -1;
+    }
+    Q8Launch launch;
+    launch.vals = (const uint8_t *)vals; launch.scales = (const uint8_t *)scales; launch.biases = (const uint8_t *)biases;
+    launch.x = xs; launch.y = ys;
+    launch.rows = R; launch.cols = C; launch.tokens = B;
+    launch.x_stride = C; launch.y_stride = R;
+    if (q8_launch(launch, (hipStream_t)stream) != 0) { set_error("q8 matvec: launch failed"); return -1; }
+    return 0;
+}
+
 int salt_mi355_router_topk_dev(const float *logits, const float *per_expert_scale, int n_experts, int topk,
                                int sorted_by_id, int *selected, float *weights, int *status_dev, void *stream) {
     if (!g_state.ready) { set_error("router: library not initialised"); return -1; }

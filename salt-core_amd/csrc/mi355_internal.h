@@ -156,6 +156,34 @@ struct Fp4MfmaLaunch {
 int fp4_mfma_splits(int rows, int cols, int tokens);
 int fp4_mfma_launch(const Fp4MfmaLaunch &launch, hipStream_t stream);
 
+// ---------------------------------------------------------------- bf16 and 8-bit affine matvecs
+
+// y[t][r] = bf16 row r of `weights` times x[t], eight column chains per row folded in the reference's tree
+// (src/kernels.c:139-174), plus bias[r] (or 0.0f).  All pointers are device pointers.
+struct Bf16Launch {
+    const uint16_t *weights;  // [rows][cols]
+    const float *x;           // [tokens][x_stride]
+    const float *bias;        // [rows] or null
+    float *y;                 // [tokens][y_stride]
+    int rows, cols, tokens;
+    int x_stride, y_stride;
+};
+bool bf16_is_tileable(const Bf16Launch &launch);
+int bf16_launch(const Bf16Launch &launch, hipStream_t stream);
+
+// y[t][r] = sum over c, one left-to-right chain, of ((float)byte * scale + bias) * x[t][c] with the scale and bias
+// of the 64-element group that holds flat element r * cols + c (src/kernels.c:343-370).
+struct Q8Launch {
+    const uint8_t *vals;      // [rows][cols] bytes
+    const uint8_t *scales;    // bf16 per 64 flat elements
+    const uint8_t *biases;    // bf16 per 64 flat elements, or null (0.0f)
+    const float *x;           // [tokens][x_stride]
+    float *y;                 // [tokens][y_stride]
+    int rows, cols, tokens;
+    int x_stride, y_stride;
+};
+int q8_launch(const Q8Launch &launch, hipStream_t stream);
+
 // ---------------------------------------------------------------- MoE
 
 struct MoeGeometry {

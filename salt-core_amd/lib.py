@@ -78,6 +78,8 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_nvfp4_matvec_qdq_dev, i, vp, vp, f, f, i, i, vp, vp, vp, i, vp)
     _sig(lib.salt_mi355_nvfp4_matmul_workspace_bytes, sz, i, i, i)
     _sig(lib.salt_mi355_nvfp4_matmul_dev, i, vp, vp, f, f, i, i, i, vp, vp, vp, vp, vp)
+    _sig(lib.salt_mi355_bf16_matvec_dev, i, vp, i, i, i, vp, vp, vp, vp)
+    _sig(lib.salt_mi355_q8_matvec_dev, i, vp, vp, vp, i, i, i, vp, vp, vp)
     _sig(lib.salt_mi355_router_topk_dev, i, vp, vp, i, i, i, vp, vp, vp, vp)
     _sig(lib.salt_mi355_moe_workspace_bytes, sz, i, i, i, i)
     _sig(lib.salt_mi355_moe_decode_step_dev, i, vp, sz, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, vp, vp)
@@ -219,6 +221,42 @@ def nvfp4_matvec_one_launch(packed: np.ndarray, scales: np.ndarray, divisor: flo
                                               chains, stream), "nvfp4_matvec_qdq_dev")
     check(lib.salt_mi355_stream_sync(stream), "sync")
     return int(st.to_host(np.int32)[0]), dy.to_host(np.float32)
+
+
+def bf16_matvec(weights: np.ndarray, R: int, C_: int, xs: np.ndarray, bias: np.ndarray | None = None,
+                weight_offset: int = 0) -> np.ndarray:
+    """weights: uint16 [R*C]; xs: float32 [B, C]; returns float32 [B, R].  weight_offset shifts the matrix by that
+    many bytes inside its device allocation (the kernels' alignment cases)."""
+    lib = init()
+    xs = np.ascontiguousarray(xs, np.float32).reshape(-1, C_)
+    B = xs.shape[0]
+    dw = DeviceBuffer(weights.nbytes + weight_offset + 16, fill=0)
+    dw.upload(weights, weight_offset)
+    dx, dy = DeviceBuffer.from_host(xs), DeviceBuffer(B * R * 4, fill=0xFF)
+    db = DeviceBuffer.from_host(np.ascontiguousarray(bias, np.float32)) if bias is not None else None
+    stream = lib.salt_mi355_stream()
+    check(lib.salt_mi355_bf16_matvec_dev(dw.at(weight_offset), R, C_, B, dx.ptr, db.ptr if db else None, dy.ptr, stream),
+          "bf16_matvec_dev")
+    check(lib.salt_mi355_stream_sync(stream), "sync")
+    return dy.to_host(np.float32).reshape(B, R)
+
+
+def q8_matvec(vals: np.ndarray, scales: np.ndarray, biases: np.ndarray | None, R: int, C_: int, xs: np.ndarray,
+              value_offset: int = 0) -> np.ndarray:
+    """vals: uint8 [R*C]; scales / biases: uint16 per 64 flat elements; xs: float32 [B, C]; returns [B, R]."""
+    lib = init()
+    xs = np.ascontiguousarray(xs, np.float32).reshape(-1, C_)
+    B = xs.shape[0]
+    dv = DeviceBuffer(vals.nbytes + value_offset + 16, fill=0)
+    dv.upload(vals, value_offset)
+    ds = DeviceBuffer.from_host(scales)
+    dbi = DeviceBuffer.from_host(biases) if biases is not None else None
+    dx, dy = DeviceBuffer.from_host(xs), DeviceBuffer(B * R * 4, fill=0xFF)
+    stream = lib.salt_mi355_stream()
+    check(lib.salt_mi355_q8_matvec_dev(dv.at(value_offset), ds.ptr, dbi.ptr if dbi else None, R, C_, B, dx.ptr, dy.ptr,
+                                       stream), "q8_matvec_dev")
+    check(lib.salt_mi355_stream_sync(stream), "sync")
+    return dy.to_host(np.float32).reshape(B, R)
 
 
 def router_topk(logits: np.ndarray, scale: np.ndarray, topk: int, sorted_by_id: bool = False):
