@@ -47,7 +47,7 @@ struct Resource {
 struct Tensor {
     int resource = -1;                // index into resources
     const uint8_t *vals = nullptr, *scales = nullptr, *biases = nullptr;   // host addresses as registered
-    int bits = 0;                     // 4 = affine Q4, 40 = NVFP4
+    int bits = 0;                     // 4 = affine Q4, 8 = affine 8-bit, 16 = bf16, 40 = NVFP4
     int R = 0, C = 0;
     float stored_divisor = 0.0f, input_global_scale = 0.0f;
 };
@@ -205,6 +205,7 @@ int release_resource_memory(Resource &r) {
 struct Q4Weights { const uint8_t *vals, *scales, *biases; };
 
 size_t q4_vals_bytes(int R, int C) { return ((size_t)R * C + 7) / 8 * 4; }
+size_t q8_vals_bytes(int R, int C) { return ((size_t)R * C + 3) / 4 * 4; }
 size_t q4_meta_bytes(int R, int C) { return ((size_t)R * C + 63) / 64 * 2; }
 
 int legacy_reserve(size_t nbytes) {
@@ -234,8 +235,9 @@ const uint8_t *legacy_upload(const void *host, size_t nbytes) {
 
 // Maps the host pointers of one affine-Q4 tensor to device addresses.
 // *legacy is set when the weights had to be copied for this call.
-int locate_q4(const void *vals, const void *scales, const void *biases, int R, int C, Q4Weights *out, int *legacy) {
-    const size_t vb = q4_vals_bytes(R, C), mb = q4_meta_bytes(R, C);
+int locate_q4(const void *vals, const void *scales, const void *biases, int R, int C, Q4Weights *out, int *legacy,
+              int bits = 4) {
+    const size_t vb = bits == 8 ? q8_vals_bytes(R, C) : q4_vals_bytes(R, C), mb = q4_meta_bytes(R, C);
     out->vals = resident_address(vals, vb);
     out->scales = resident_address(scales, mb);
     out->biases = biases ? resident_address(biases, mb) : nullptr;
@@ -256,12 +258,12 @@ int locate_q4(const void *vals, const void *scales, const void *biases, int R, i
 
 // A registered key must agree with the pointers the call carries (the
 // reference re-validates this on every batch, gpu_hip.cpp:4973-4986).
-int key_agrees(const void *key, const void *vals, const void *scales, const void *biases, int R, int C) {
+int key_agrees(const void *key, const void *vals, const void *scales, const void *biases, int R, int C, int bits = 4) {
     if (!key) return 1;
     auto it = g_engine.tensors.find(key);
     if (it == g_engine.tensors.end()) return 1;          // unknown keys fall through to pointer lookup
     const Tensor &t = it->second;
-    return t.bits == 4 && t.vals == vals && t.scales == scales && t.biases == biases && t.R == R && t.C == C;
+    return t.bits == bits && t.vals == vals && t.scales == scales && t.biases == biases && t.R == R && t.C == C;
 }
 
 void count_batch(const void *vals, int legacy) {
@@ -284,9 +286,9 @@ int ready_or_fail(const char *who) {
 int register_tensor(uint32_t kind, uint32_t id, const void *key, const void *vals, size_t vals_bytes,
                     const void *scales, size_t scales_bytes, const void *biases, size_t biases_bytes, Tensor proto) {
     const int ri = find_resource(kind, id);
-    if (ri < 0 || !key || !vals || !scales) { set_error("tensor slot: unknown resource or null argument"); return -1; }
+    if (ri < 0 || !key || !vals || (!scales && scales_bytes)) { set_error("tensor slot: unknown resource or null argument"); return -1; }
     const Resource &r = g_engine.resources[(size_t)ri];
-    if (!inside(r.host, r.nbytes, vals, vals_bytes) || !inside(r.host, r.nbytes, scales, scales_bytes) ||
+    if (!inside(r.host, r.nbytes, vals, vals_bytes) || (scales && !inside(r.host, r.nbytes, scales, scales_bytes)) ||
         (biases && !inside(r.host, r.nbytes, biases, biases_bytes))) {
         set_error("tensor slot: tensor bytes lie outside resource (%u, %u)", kind, id);
         return -1;
@@ -574,12 +576,12 @@ int salt_gpu_weight_resource_usage(SaltGpuWeightResourceUsage *usage, size_t usa
 int salt_gpu_weight_resource_slot(uint32_t kind, uint32_t resource_id, const void *key, const uint32_t *vals,
                                   const uint16_t *scales, const uint16_t *biases, int bits, int R, int C) {
     if (ready_or_fail("weight_resource_slot") != 0) return -1;
-    if (bits != 4) { set_error("weight_resource_slot: only 4-bit tensors are on this backend's path (bits %d)", bits); return -1; }
+    if (bits != 4 && bits != 8) { set_error("weight_resource_slot: only 4-bit and 8-bit tensors are on this backend's path (bits %d)", bits); return -1; }
     if (R < 1 || C < 1 || C > MAX_C) { set_error("weight_resource_slot: bad geometry"); return -1; }
     Tensor t;
-    t.bits = 4; t.R = R; t.C = C;
-    return register_tensor(kind, resource_id, key, vals, q4_vals_bytes(R, C), scales, q4_meta_bytes(R, C), biases,
-                           q4_meta_bytes(R, C), t);
+    t.bits = bits; t.R = R; t.C = C;
+    return register_tensor(kind, resource_id, key, vals, bits == 8 ? q8_vals_bytes(R, C) : q4_vals_bytes(R, C), scales,
+                           q4_meta_bytes(R, C), biases, q4_meta_bytes(R, C), t);
 }
 
 int salt_gpu_nvfp4_resource_slot(uint32_t kind, uint32_t resource_id, const void *key, const uint8_t *packed,
@@ -1228,6 +1230,107 @@ int salt_gpu_nvfp4_batch(const void *const *keys, const float *const *inputs, fl
     return salt_gpu_nvfp4_mixed_batch(keys, inputs, outputs, batches, rows.data(), C, njobs);
 }
 
+// ================================================================ 8-bit affine (router gates) and bf16 (head)
+
+int salt_gpu_q8_batch(const uint32_t *const *vals, const uint16_t *const *scales, const uint16_t *const *biases,
+                      const float *const *xs, float *const *ys, const void *const *ids, const int *Rj, int C,
+                      int njobs) {
+    if (ready_or_fail("q8_batch") != 0) return -1;
+    if (!vals || !scales || !xs || !ys || !Rj || njobs < 1 || (uint32_t)njobs > MAX_BATCH_JOBS || C < 1 || C > MAX_C) {
+        set_error("q8_batch: bad arguments");
+        return -1;
+    }
+    std::vector<HostJob> jobs;
+    int any_legacy = 0;
+    size_t in_bytes = 0, out_bytes = 0;
+    for (int j = 0; j < njobs; ++j) {
+        const uint16_t *bias = biases ? biases[j] : nullptr;
+        if (!vals[j] || !scales[j] || !xs[j] || !ys[j] || Rj[j] < 1) { set_error("q8_batch: job %d is malformed", j); return -1; }
+        if (!key_agrees(ids ? ids[j] : nullptr, vals[j], scales[j], bias, Rj[j], C, 8)) {
+            set_error("q8_batch: job %d does not match the tensor registered under its key", j);
+            return -1;
+        }
+        // the engine sends one job per token of the same gate: contiguous rows of x and y become one job
+        if (!jobs.empty()) {
+            HostJob &prev = jobs.back();
+            if (prev.rows == Rj[j] && vals[j] == vals[j - 1] && scales[j] == scales[j - 1] &&
+                prev.x_host + (size_t)prev.tokens * C == xs[j] && prev.y_host + (size_t)prev.tokens * prev.rows == ys[j]) {
+                prev.tokens++;
+                continue;
+            }
+        }
+        HostJob job = {};
+        int legacy = 0;
+        if (locate_q4(vals[j], scales[j], bias, Rj[j], C, &job.w, &legacy, 8) != 0) return -1;
+        any_legacy |= legacy;
+        job.x_host = xs[j]; job.y_host = ys[j]; job.rows = Rj[j]; job.tokens = 1;
+        jobs.push_back(job);
+    }
+    for (const HostJob &j : jobs) {
+        in_bytes += align_up((size_t)j.tokens * C * 4, 256);
+        out_bytes += align_up((size_t)j.tokens * j.rows * 4, 256);
+    }
+    if (staging_reserve(in_bytes + out_bytes, in_bytes + out_bytes) != 0) return -1;
+    std::vector<OutputCopy> copies;
+    for (HostJob &j : jobs) {
+        const float *x_dev = upload_activations(j.x_host, (size_t)j.tokens * C);
+        if (!x_dev) { (void)salt_gpu_sync(); return -1; }
+        const size_t count = (size_t)j.tokens * j.rows;
+        uint8_t *dev = device_take(count * 4), *pin = pinned_take(count * 4);
+        g_engine.pending.push_back({pin, j.y_host, count * 4});
+        copies.push_back({dev, pin, count * 4});
+        if (salt_mi355_q8_matvec_dev(j.w.vals, j.w.scales, j.w.biases, j.rows, C, j.tokens, x_dev, (float *)dev,
+                                     g_state.stream) != 0) { (void)salt_gpu_sync(); return -1; }
+    }
+    count_batch(vals[0], any_legacy);
+    return finish_call(copies);
+}
+
+int salt_gpu_q8_matvec(const uint32_t *vals, const uint16_t *scales, const uint16_t *biases, int R, int C,
+                       const float *x, float *y) {
+    const void *id = vals;
+    return salt_gpu_q8_batch(&vals, &scales, &biases, &x, &y, &id, &R, C, 1);
+}
+
+int salt_gpu_bf16_resource_slot(uint32_t kind, uint32_t resource_id, const void *key, const uint16_t *weights, int R,
+                                int C) {
+    if (ready_or_fail("bf16_resource_slot") != 0) return -1;
+    if (R < 1 || C < 8 || (C & 7) != 0) { set_error("bf16_resource_slot: the column count must be a multiple of 8"); return -1; }
+    Tensor t;
+    t.bits = 16; t.R = R; t.C = C;
+    return register_tensor(kind, resource_id, key, weights, (size_t)R * C * 2, nullptr, 0, nullptr, 0, t);
+}
+
+int salt_gpu_bf16_matvec(const void *key, int R, int C, const float *input, float *output) {
+    if (ready_or_fail("bf16_matvec") != 0) return -1;
+    auto it = g_engine.tensors.find(key);
+    if (!key || it == g_engine.tensors.end() || it->second.bits != 16 || it->second.R != R || it->second.C != C ||
+        R < 1 || C < 8 || (C & 7) != 0 || (size_t)R > MAX_OUTPUT_FLOATS || !input || !output) {
+        g_engine.stats.mapped_only_misses += g_engine.mapped_only ? 1 : 0;
+        set_error("bf16_matvec: no bf16 tensor of %d x %d is registered under this key, or bad arguments", R, C);
+        return -1;
+    }
+    const Tensor &t = it->second;
+    const uint8_t *weights = resident_address(t.vals, (size_t)R * C * 2);
+    if (!weights) { set_error("bf16_matvec: the tensor's resource is not active"); return -1; }
+    const size_t in_bytes = align_up((size_t)C * 4, 256), out_bytes = align_up((size_t)R * 4, 256);
+    if (staging_reserve(in_bytes + out_bytes, in_bytes + out_bytes) != 0) return -1;
+    const float *x_dev = upload_activations(input, (size_t)C);
+    if (!x_dev) { (void)salt_gpu_sync(); return -1; }
+    uint8_t *dev = device_take((size_t)R * 4), *pin = pinned_take((size_t)R * 4);
+    g_engine.pending.push_back({pin, output, (size_t)R * 4});
+    std::vector<OutputCopy> copies(1, OutputCopy{dev, pin, (size_t)R * 4});
+    if (salt_mi355_bf16_matvec_dev(weights, R, C, 1, x_dev, nullptr, (float *)dev, g_state.stream) != 0) {
+        (void)salt_gpu_sync();
+        return -1;
+    }
+    const Resource &r = g_engine.resources[(size_t)t.resource];
+    if (r.kind == KIND_EXPERT_LAYER) g_engine.stats.expert_layer_batches++; else g_engine.stats.trunk_batches++;
+    g_engine.stats.direct_output_batches++;
+    g_engine.stats.direct_output_jobs++;
+    return finish_call(copies);
+}
+
 // ================================================================ residency operations
 
 static int res_create(void *, const SaltGpuResidencyPlan *plan) {
@@ -1367,11 +1470,8 @@ const SaltGpuResidencyBackendOps *salt_gpu_residency_backend_ops(void) { return 
 
 // ================================================================ off-path entry points (null-backend answers)
 
-int salt_gpu_q8_matvec(const uint32_t *, const uint16_t *, const uint16_t *, int, int, const float *, float *) { return -1; }
-int salt_gpu_q8_batch(const uint32_t *const *, const uint16_t *const *, const uint16_t *const *, const float *const *,
-                      float *const *, const void *const *, const int *, int, int) { return -1; }
-int salt_gpu_bf16_resource_slot(uint32_t, uint32_t, const void *, const uint16_t *, int, int) { return -1; }
-int salt_gpu_bf16_matvec(const void *, int, int, const float *, float *) { return -1; }
+// The ROCm backend of the reference leaves the batched bf16 matvec to the CPU (src/gpu_hip.cpp:4624-4628); its CUDA
+// counterpart computes a different, single-chain order for the vision tower.
 int salt_gpu_bf16_matvec_batch(const void *, int, int, int, const float *, float *) { return -1; }
 int salt_gpu_exact_cells(const struct SaltGpuExactCell *, int) { return -1; }
 const struct SaltGpuDispatch *salt_dispatch_get(void) { return nullptr; }

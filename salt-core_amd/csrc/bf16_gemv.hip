@@ -39,7 +39,7 @@ __device__ __forceinline__ void wait_loads() {
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-// NB activation rows (1..4), STAGES chunks of LDS per wave, WAVES independent waves per workgroup.
+// NB activation rows (1 or 2), STAGES chunks of LDS per wave, WAVES independent waves per workgroup.
 template <int NB, int STAGES, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void bf16_tile_kernel(Bf16Launch L) {
     static_assert(STAGES >= 2 && STAGES <= 5, "the wait below knows up to four chunks in flight");
@@ -89,23 +89,34 @@ __global__ __launch_bounds__(WAVES * 64) void bf16_tile_kernel(Bf16Launch L) {
 
     const uniform_f32_ptr xbase = (uniform_f32_ptr)(uintptr_t)L.x;
 
+    // Activations of XS segments (for all NB rows at most 64 scalar registers) are requested together, so one wait
+    // covers them instead of one wait per segment.
+    constexpr int XS = NB == 1 ? 8 : 4;
     auto consume = [&](int ck, int segs) {
         const u32x4 *stage = mine + (ck % STAGES) * SLOTS + lane * 8;
         const uniform_f32_ptr xc = xbase + (size_t)ck * CHUNK;
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            if (s >= segs) break;
-            const u32x4 v = stage[s ^ my_swz];
-            const uint32_t word[4] = {v.x, v.y, v.z, v.w};
+        for (int s0 = 0; s0 < 8; s0 += XS) {
+            if (s0 >= segs) break;
+            float xq[NB][XS * 8];
 #pragma unroll
-            for (int t = 0; t < NB; ++t) {
-                const uniform_f32_ptr xs = xc + (size_t)t * L.x_stride + s * 8;
+            for (int t = 0; t < NB; ++t)
 #pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    const float lo = __uint_as_float(word[p] << 16), hi = __uint_as_float(word[p] & 0xffff0000u);
-                    acc[t][2 * p] = acc[t][2 * p] + lo * xs[2 * p];
-                    acc[t][2 * p + 1] = acc[t][2 * p + 1] + hi * xs[2 * p + 1];
-                }
+                for (int k = 0; k < XS * 8; ++k)
+                    if (s0 * 8 + k < segs * 8) xq[t][k] = xc[(size_t)t * L.x_stride + s0 * 8 + k];
+#pragma unroll
+            for (int s = s0; s < s0 + XS; ++s) {
+                if (s >= segs) break;
+                const u32x4 v = stage[s ^ my_swz];
+                const uint32_t word[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int t = 0; t < NB; ++t)
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) {
+                        const float lo = __uint_as_float(word[p] << 16), hi = __uint_as_float(word[p] & 0xffff0000u);
+                        acc[t][2 * p] = acc[t][2 * p] + lo * xq[t][(s - s0) * 8 + 2 * p];
+                        acc[t][2 * p + 1] = acc[t][2 * p + 1] + hi * xq[t][(s - s0) * 8 + 2 * p + 1];
+                    }
             }
         }
     };
@@ -178,10 +189,9 @@ template <int NB>
 void launch_shape(const Bf16Launch &L, hipStream_t stream) {
     switch (env_shape()) {
     case 1: launch_tiles<NB, 2, 1>(L, stream); break;
-    case 2: launch_tiles<NB, 4, 1>(L, stream); break;
-    case 3: launch_tiles<NB, 4, 2>(L, stream); break;
-    case 4: launch_tiles<NB, 2, 4>(L, stream); break;
-    default: launch_tiles<NB, 3, 1>(L, stream); break;
+    case 2: launch_tiles<NB, 3, 1>(L, stream); break;
+    case 3: launch_tiles<NB, 2, 2>(L, stream); break;
+    default: launch_tiles<NB, 2, 4>(L, stream); break;
     }
 }
 
@@ -198,17 +208,14 @@ int bf16_launch(const Bf16Launch &L, hipStream_t stream) {
         bf16_generic_kernel<<<dim3((L.rows + 63) / 64), dim3(64), 0, stream>>>(L);
         return hipGetLastError() == hipSuccess ? 0 : -1;
     }
-    for (int first = 0; first < L.tokens; first += 4) {
+    // two activation rows per pass: the pass stays bound by the matrix stream, which wider passes do not
+    for (int first = 0; first < L.tokens; first += 2) {
         Bf16Launch part = L;
         part.x = L.x + (size_t)first * L.x_stride;
         part.y = L.y + (size_t)first * L.y_stride;
-        part.tokens = L.tokens - first < 4 ? L.tokens - first : 4;
-        switch (part.tokens) {
-        case 1: launch_shape<1>(part, stream); break;
-        case 2: launch_shape<2>(part, stream); break;
-        case 3: launch_shape<3>(part, stream); break;
-        default: launch_shape<4>(part, stream); break;
-        }
+        part.tokens = L.tokens - first < 2 ? L.tokens - first : 2;
+        if (part.tokens == 1) launch_shape<1>(part, stream);
+        else launch_shape<2>(part, stream);
         if (hipGetLastError() != hipSuccess) return -1;
     }
     return 0;

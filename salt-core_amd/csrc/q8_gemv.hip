@@ -2,8 +2,9 @@
 // reference src/kernels.c:343-370): one accumulator per row walks the columns left to right,
 //     acc = acc + ((float)byte * scale + bias) * x[c]
 // with every operation rounded separately and the scale and bias of the 64-element group that holds the flat element
-// row * cols + c.  The chain of one row cannot be split, so a lane owns a row; lanes of a wave own 64 consecutive
-// rows and the activations reach them as scalar operands.
+// row * cols + c.  The chain of one row cannot be split, and a dependent fp32 addition issues only every dozen clocks
+// from a lone wave, so the chain itself bounds the time (about 15 us for 2816 columns); the kernels differ in what
+// else sits on the adding wave.
 #include "mi355_internal.h"
 
 namespace mi355 {
@@ -16,7 +17,8 @@ typedef const float __attribute__((address_space(4))) *uniform_f32_ptr;
 
 __device__ __forceinline__ float bf16_bits(uint32_t half) { return __uint_as_float(half << 16); }
 
-// cols % 64 == 0 and 16-byte aligned values: groups never straddle rows.  blockIdx.y is the activation row.
+// More than 4096 columns (cols % 64 == 0, 16-byte aligned values): a lane owns a row and does all of its work;
+// activations reach it as scalar operands.  blockIdx.y is the activation row.
 __global__ __launch_bounds__(64) void q8_rows_kernel(Q8Launch L) {
     const int lane = threadIdx.x;
     const int row0 = blockIdx.x * 64;
@@ -52,6 +54,102 @@ __global__ __launch_bounds__(64) void q8_rows_kernel(Q8Launch L) {
     if (lane < rows_here) L.y[(size_t)token * L.y_stride + row] = acc;
 }
 
+// Up to 4096 columns.  A workgroup owns 16 rows and one activation row.  The chain of a row is one addition per column and
+// nothing else can be taken off it, so the work is split by kind: three waves turn bytes into rounded products
+// ((float)byte * scale + bias) * x and leave them in LDS, and the fourth wave only adds them, in column order, one
+// lane per row.  Products travel in chunks of 192 columns through two LDS buffers; all bytes of the 16 rows are held in
+// registers from the start, so the memory latency is paid once.
+constexpr int CH_ROWS = 16;
+constexpr int CH_COLS = 192;                       // 16 rows x 12 segments of 16 bytes = 192 items, one per producer lane
+constexpr int CH_PITCH = CH_COLS + 4;              // floats; lanes 0..15 of a 16-byte read then touch distinct banks
+constexpr int CH_MAX_COLS = 4096;
+constexpr int CH_MAX_CHUNKS = (CH_MAX_COLS + CH_COLS - 1) / CH_COLS;
+
+__global__ __launch_bounds__(256) void q8_chain_kernel(Q8Launch L) {
+    __shared__ float x_lds[CH_MAX_COLS];
+    __shared__ float scale_lds[CH_ROWS][CH_MAX_COLS / 64], bias_lds[CH_ROWS][CH_MAX_COLS / 64];
+    __shared__ __attribute__((aligned(16))) float ring[2][CH_ROWS][CH_PITCH];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int row0 = blockIdx.x * CH_ROWS;
+    const int rows_here = L.rows - row0 < CH_ROWS ? L.rows - row0 : CH_ROWS;
+    const int C = L.cols, groups = C / 64;
+    const int nchunk = (C + CH_COLS - 1) / CH_COLS;
+    const float *x = L.x + (size_t)blockIdx.y * L.x_stride;
+
+    // producer item: one row, 16 consecutive columns of every chunk.  All of a lane's bytes are requested before
+    // anything else happens, unconditionally (a column past the row re-reads the row's last segment), so the loads
+    // are straight-line code and each use waits only for its own load.
+    const int pid = tid >= 64 ? tid - 64 : 0;
+    const int prow = pid / 12, pseg = pid % 12;
+    const int prow_src = prow < rows_here ? prow : rows_here - 1;
+    const global_u128_ptr src = (global_u128_ptr)(uintptr_t)(L.vals + (size_t)(row0 + prow_src) * C);
+    u32x4 bytes[CH_MAX_CHUNKS];
+#pragma unroll
+    for (int k = 0; k < CH_MAX_CHUNKS; ++k) {
+        const int col = k * CH_COLS + pseg * 16;
+        bytes[k] = src[(col < C ? col : C - 16) / 16];
+    }
+    for (int c = tid; c < C; c += 256) x_lds[c] = x[c];
+    for (int i = tid; i < CH_ROWS * groups; i += 256) {
+        const int r = i / groups, g = i % groups;
+        const size_t at = (size_t)(row0 + (r < rows_here ? r : rows_here - 1)) * groups + g;
+        scale_lds[r][g] = bf16_bits(((const uint16_t *)L.scales)[at]);
+        bias_lds[r][g] = L.biases ? bf16_bits(((const uint16_t *)L.biases)[at]) : 0.0f;
+    }
+    __syncthreads();
+
+    float acc = 0.0f;
+    const int crow = lane < CH_ROWS ? lane : 0;
+    // step i: producers fill ring[i % 2] with chunk i while the adder walks chunk i - 1 in ring[(i - 1) % 2]
+#pragma unroll
+    for (int i = 0; i <= CH_MAX_CHUNKS; ++i) {
+        if (i > nchunk) continue;                 // uniform over the workgroup
+        if (wave != 0) {
+            const int col = i * CH_COLS + pseg * 16;
+            if (i < CH_MAX_CHUNKS && col < C) {
+                const u32x4 v = bytes[i < CH_MAX_CHUNKS ? i : 0];
+                const uint32_t word[4] = {v.x, v.y, v.z, v.w};
+                const float s = scale_lds[prow][col / 64], b = bias_lds[prow][col / 64];
+                float *out = &ring[i & 1][prow][pseg * 16];
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    const float4 xv = *(const float4 *)&x_lds[col + 4 * p];
+                    const float xs[4] = {xv.x, xv.y, xv.z, xv.w};
+                    float prod[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        float value = (float)((word[p] >> (8 * q)) & 0xffu) * s;
+                        value = value + b;
+                        prod[q] = value * xs[q];
+                    }
+                    *(float4 *)&out[4 * p] = make_float4(prod[0], prod[1], prod[2], prod[3]);
+                }
+            }
+        } else if (i >= 1) {
+            const int c0 = (i - 1) * CH_COLS;
+            const int units = (C - c0 < CH_COLS ? C - c0 : CH_COLS) / 64;
+            const float *in = &ring[(i - 1) & 1][crow][0];
+            auto add_units = [&](int count) {
+#pragma unroll
+                for (int j = 0; j < 16 * 3; ++j) {
+                    if (j >= 16 * count) break;
+                    const float4 p = *(const float4 *)&in[4 * j];
+                    acc = acc + p.x;
+                    acc = acc + p.y;
+                    acc = acc + p.z;
+                    acc = acc + p.w;
+                }
+            };
+            if (units == 3) add_units(3);
+            else if (units == 2) add_units(2);
+            else add_units(1);
+        }
+        __syncthreads();
+    }
+    if (wave == 0 && lane < rows_here) L.y[(size_t)blockIdx.y * L.y_stride + row0 + lane] = acc;
+}
+
 // Any column count and alignment.
 __global__ __launch_bounds__(64) void q8_generic_kernel(Q8Launch L) {
     const int row = blockIdx.x * 64 + threadIdx.x;
@@ -78,7 +176,9 @@ int q8_launch(const Q8Launch &L, hipStream_t stream) {
     const dim3 grid((L.rows + 63) / 64, L.tokens);
     const bool fast = L.cols % 64 == 0 && ((uintptr_t)L.vals & 15) == 0 && ((uintptr_t)L.scales & 1) == 0 &&
                       ((uintptr_t)L.biases & 1) == 0 && ((uintptr_t)L.x & 3) == 0;
-    if (fast) q8_rows_kernel<<<grid, dim3(64), 0, stream>>>(L);
+    if (fast && L.cols <= CH_MAX_COLS)
+        q8_chain_kernel<<<dim3((L.rows + CH_ROWS - 1) / CH_ROWS, L.tokens), dim3(256), 0, stream>>>(L);
+    else if (fast) q8_rows_kernel<<<grid, dim3(64), 0, stream>>>(L);
     else q8_generic_kernel<<<grid, dim3(64), 0, stream>>>(L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }

@@ -121,7 +121,10 @@ def bind(lib):
     sig("salt_gpu_nvfp4_mixed_batch", i32, vp, vp, vp, vp, vp, i32, i32)
     sig("salt_gpu_residency_backend_ops", C.POINTER(ResidencyOps))
     sig("salt_gpu_q8_matvec", i32, vp, vp, vp, i32, i32, vp, vp)
+    sig("salt_gpu_q8_batch", i32, vp, vp, vp, vp, vp, vp, vp, i32, i32)
+    sig("salt_gpu_bf16_resource_slot", i32, u32, u32, vp, vp, i32, i32)
     sig("salt_gpu_bf16_matvec", i32, vp, i32, i32, vp, vp)
+    sig("salt_gpu_bf16_matvec_batch", i32, vp, i32, i32, i32, vp, vp)
     sig("salt_dispatch_get", vp)
     sig("salt_gpu_tensor_program_ops", vp)
     sig("salt_gpu_resident_trunk_map", i32, vp, sz)

@@ -93,7 +93,8 @@ def q8_tensor(R, C, seed):
 
 
 @pytest.mark.parametrize("R,C,B,offset", [(128, 2816, 1, 0), (128, 2816, 5, 0), (1, 64, 1, 0), (70, 128, 2, 0),
-                                          (3, 96, 2, 0), (65, 200, 1, 0), (16, 256, 1, 4)])
+                                          (3, 96, 2, 0), (65, 200, 1, 0), (16, 256, 1, 4), (20, 384, 1, 0), (17, 576, 3, 0),
+                                          (33, 4096, 1, 0), (40, 4160, 2, 0), (130, 1728, 1, 0)])
 def test_q8_matvec(gpu, oracle, R, C, B, offset):
     print("q8", R, C, B, offset, flush=True)
     vals, scales, biases = q8_tensor(R, C, R + C)

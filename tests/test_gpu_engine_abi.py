@@ -79,7 +79,7 @@ def test_resource_lifecycle_matvec_batch_and_stats(eng, oracle, pkg):
         assert eng.salt_gpu_weight_resource_slot(TRUNK, 7, keys[k], v, s, b, 4, R, Cc) == 0          # identical re-registration
     v0, s0, b0 = trunk.pointers(0)
     assert eng.salt_gpu_weight_resource_slot(TRUNK, 7, keys[0], v0 + 16, s0, b0, 4, 704, 2816) == -1  # conflicting key
-    assert eng.salt_gpu_weight_resource_slot(TRUNK, 7, 0x2000, v0, s0, b0, 8, 704, 2816) == -1        # q8 is off-path
+    assert eng.salt_gpu_weight_resource_slot(TRUNK, 7, 0x2000, v0, s0, b0, 3, 704, 2816) == -1        # neither 4 nor 8 bits
     assert eng.salt_gpu_weight_resource_slot(TRUNK, 9, 0x2000, v0, s0, b0, 4, 704, 2816) == -1        # unknown resource
     assert eng.salt_gpu_weight_resource_slot(TRUNK, 7, 0x2000, v0, s0, b0, 4, 70400, 2816) == -1      # outside the range
 
@@ -437,10 +437,74 @@ def test_nvfp4_engine_entry_points(eng, oracle, pkg):
     assert eng.salt_gpu_nvfp4_matvec(key, R, Cc, ptr(xs[0]), ptr(y)) == -1
 
 
+def test_router_gate_and_head_through_the_engine(eng, oracle, pkg):
+    """An 8-bit router gate (one job per token of the same matrix, the way the engine batches it) and the bf16 head,
+    both inside one described trunk resource."""
+    g = synth.rng(77)
+    GR, Cc, HR = 128, 2816, 4100
+    gate_vals = g.integers(0, 256, size=GR * Cc, dtype=np.uint8)
+    gate_scales = (g.uniform(0.001, 0.01, GR * Cc // 64).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    gate_biases = (g.uniform(-1.0, 0.0, GR * Cc // 64).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    head = (g.standard_normal(HR * Cc).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    parts, offs, at = [], [], 0
+    for a in (gate_vals, gate_scales, gate_biases, head):
+        offs.append(at); parts.append(a.view(np.uint8)); at += a.nbytes
+        pad = (-at) % 16; parts.append(np.zeros(pad, np.uint8)); at += pad
+    blob = np.concatenate(parts); base = blob.ctypes.data
+    gv, gs, gb, hw = (base + o for o in offs)
+    assert eng.salt_gpu_weight_resource_describe(TRUNK, 21, base, blob.nbytes) == 0
+    assert eng.salt_gpu_weight_resource_activate(TRUNK, 21, 2) == 0, err(pkg)
+    assert eng.salt_gpu_weight_resource_slot(TRUNK, 21, gv, gv, gs, gb, 8, GR, Cc) == 0, err(pkg)
+    assert eng.salt_gpu_bf16_resource_slot(TRUNK, 21, hw, hw, HR, Cc) == 0, err(pkg)
+    assert eng.salt_gpu_bf16_resource_slot(TRUNK, 21, hw, hw, HR, Cc) == 0                 # identical re-registration
+    assert eng.salt_gpu_bf16_resource_slot(TRUNK, 21, hw, hw + 16, HR - 1, Cc) == -1       # key bound to another tensor
+    assert eng.salt_gpu_bf16_resource_slot(TRUNK, 21, 0x5000, hw, HR, Cc + 4) == -1        # columns not a multiple of 8
+    assert eng.salt_gpu_bf16_resource_slot(TRUNK, 21, 0x5000, hw, HR * 4, Cc) == -1        # outside the resource
+    eng.salt_gpu_set_mapped_only(1)
+    before = abi.BatchStats(); eng.salt_gpu_batch_stats_get(C.byref(before))
+
+    T = 5
+    xs = synth.activations(Cc, T, 31); ys = np.full((T, GR), np.nan, np.float32)
+    rc = eng.salt_gpu_q8_batch(abi.ptr_array([gv] * T), abi.ptr_array([gs] * T), abi.ptr_array([gb] * T),
+                               abi.ptr_array([xs[t] for t in range(T)]), abi.ptr_array([ys[t] for t in range(T)]),
+                               abi.ptr_array([gv] * T), (C.c_int * T)(*([GR] * T)), Cc, T)
+    assert rc == 0, err(pkg)
+    want = np.zeros(GR, np.float32)
+    for t in range(T):
+        oracle.orc_q8_matvec(ptr(gate_vals), ptr(gate_scales), ptr(gate_biases), GR, Cc, ptr(xs[t]), ptr(want))
+        assert np.array_equal(bits(ys[t]), bits(want)), t
+    y1 = np.full(GR, np.nan, np.float32)
+    assert eng.salt_gpu_q8_matvec(gv, gs, gb, GR, Cc, ptr(xs[2]), ptr(y1)) == 0, err(pkg)
+    assert np.array_equal(bits(y1), bits(ys[2]))
+    # a key registered for another geometry is refused; so are weights outside every resource in mapped-only mode
+    assert eng.salt_gpu_q8_matvec(gv, gs, gb, GR - 1, Cc, ptr(xs[2]), ptr(y1)) == -1
+    loose = gate_vals.copy()
+    assert eng.salt_gpu_q8_matvec(ptr(loose), gs, gb, GR, Cc, ptr(xs[2]), ptr(y1)) == -1
+
+    logits = np.full(HR, np.nan, np.float32)
+    assert eng.salt_gpu_bf16_matvec(hw, HR, Cc, ptr(xs[0]), ptr(logits)) == 0, err(pkg)
+    want = np.zeros(HR, np.float32)
+    oracle.orc_bf16_matvec(ptr(head), HR, Cc, ptr(xs[0]), None, ptr(want))
+    assert np.array_equal(bits(logits), bits(want))
+    assert eng.salt_gpu_bf16_matvec(hw, HR - 1, Cc, ptr(xs[0]), ptr(logits)) == -1         # geometry differs from the slot
+    assert eng.salt_gpu_bf16_matvec(0x5000, HR, Cc, ptr(xs[0]), ptr(logits)) == -1         # unknown key
+    assert eng.salt_gpu_bf16_matvec(gv, GR, Cc, ptr(xs[0]), ptr(logits)) == -1             # an 8-bit tensor's key
+    assert eng.salt_gpu_bf16_matvec_batch(hw, HR, Cc, 2, ptr(xs), ptr(logits)) == -1       # left to the CPU, like the ROCm reference
+    after = abi.BatchStats(); eng.salt_gpu_batch_stats_get(C.byref(after))
+    assert after.trunk_batches - before.trunk_batches == 3
+    eng.salt_gpu_set_mapped_only(0)
+    # deferred publication: outputs appear at salt_gpu_sync
+    assert eng.salt_gpu_set_defer(1) == 0
+    logits[:] = np.nan
+    assert eng.salt_gpu_bf16_matvec(hw, HR, Cc, ptr(xs[0]), ptr(logits)) == 0
+    assert eng.salt_gpu_sync() == 0 and np.array_equal(bits(logits), bits(want))
+    assert eng.salt_gpu_set_defer(0) == 0
+    assert eng.salt_gpu_weight_resource_unbind(TRUNK, 21) == 0
+    assert eng.salt_gpu_bf16_matvec(hw, HR, Cc, ptr(xs[0]), ptr(logits)) == -1
+
+
 def test_off_path_entry_points_answer_like_the_null_backend(eng):
     z = np.zeros(64, np.float32)
-    assert eng.salt_gpu_q8_matvec(ptr(z), ptr(z), ptr(z), 1, 64, ptr(z), ptr(z)) == -1
-    assert eng.salt_gpu_bf16_matvec(1, 1, 64, ptr(z), ptr(z)) == -1
     assert eng.salt_gpu_resident_trunk_map(ptr(z), 256) == -1 and eng.salt_gpu_resident_pool_map(ptr(z), 256) == -1
     assert eng.salt_dispatch_get() is None and eng.salt_gpu_tensor_program_ops() is None
 
