@@ -358,6 +358,36 @@ def main():
         extra["moe_prefill_useful_tflops"] = round(flops / (ms_pf * 1e-3) / 1e12, 1)
         # the activation travels as three exact bf16 planes, so the matrix cores execute three times the useful flops
         extra["moe_prefill_mfma_frac"] = round(3 * flops / (ms_pf * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
+        del prefill
+        # the bf16 head (262144 x 2816, the largest matrix a decode step streams) and the 8-bit router gate
+        # (128 x 2816, one unsplittable 2816-step chain per row), both bit-exact
+        RH, CH = 262144, 2816
+        block = (synth.rng(51).standard_normal(4096 * CH).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        head = gpu.DeviceBuffer(RH * CH * 2)
+        for k in range(RH // 4096):
+            head.upload(block, k * block.nbytes)
+        xh = gpu.DeviceBuffer.from_host(synth.activations(CH, 1, 52))
+        yh = gpu.DeviceBuffer(RH * 4)
+
+        def head_step(s):
+            if lib.salt_mi355_bf16_matvec_dev(head.ptr, RH, CH, 1, xh.ptr, None, yh.ptr, s) != 0:
+                raise RuntimeError(lib.salt_mi355_last_error().decode())
+
+        ms_h = timed(lib, stream, events, head_step, 2, 20)
+        extra["bf16_head_262144x2816_us"] = round(ms_h * 1e3, 1)
+        extra["bf16_head_gbps"] = round((RH * CH * 2 + RH * 4 + CH * 4) / (ms_h * 1e-3) / 1e9, 1)
+        extra["bf16_head_hbm_frac"] = round((RH * CH * 2 + RH * 4 + CH * 4) / (ms_h * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+        del head, yh
+        RG = 128
+        gv = gpu.DeviceBuffer.from_host(synth.rng(53).integers(0, 256, RG * CH, dtype=np.uint8))
+        gs = gpu.DeviceBuffer.from_host(np.full(RG * CH // 64, 0x3C00, np.uint16))
+        yg = gpu.DeviceBuffer(RG * 4)
+
+        def gate_step(s):
+            if lib.salt_mi355_q8_matvec_dev(gv.ptr, gs.ptr, gs.ptr, RG, CH, 1, xh.ptr, yg.ptr, s) != 0:
+                raise RuntimeError(lib.salt_mi355_last_error().decode())
+
+        extra["q8_router_gate_128x2816_us"] = round(timed(lib, stream, events, gate_step, 5, 100) * 1e3, 2)
         result["extra"] = extra
 
     if not args.no_cpu:
