@@ -216,7 +216,7 @@ __global__ __launch_bounds__((32 / S) * 64) void fp4_tile_kernel(const Fp4Launch
         for (int i = 0; i < PIECES; ++i) {
             int blk = ck * CHUNK_BLOCKS + (int)seg;
             blk = blk < nblk ? blk : nblk - 1;
-            wreg[i] = *(global_u128_ptr)(codes + (src_row[i] * row_bytes + (uint32_t)blk * 16u));
+            wreg[i] = __builtin_nontemporal_load((global_u128_ptr)(codes + (src_row[i] * row_bytes + (uint32_t)blk * 16u)));
             mreg[i] = scale_pairs[src_row[i] * row_pairs + (uint32_t)blk];
         }
     };

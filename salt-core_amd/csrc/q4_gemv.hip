@@ -268,6 +268,12 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
     // the address is a wave-uniform base plus the fixed per-thread offset; in
     // the last one group indices past the end of the row are clamped (the data
     // is staged but never consumed).
+    // With several activation rows per launch the weights are fetched with the non-temporal policy: they are read
+    // once, and keeping them out of the caches leaves the activations there (measured +17 % at four rows; at one row
+    // the default policy is 1 % faster).
+    auto load_weights = [](global_u8_ptr p) {
+        return NB > 1 ? __builtin_nontemporal_load((global_u128_ptr)p) : *(global_u128_ptr)p;
+    };
     auto issue = [&](int ck) {
         if (!has_item) return;
         const bool tail = (ck + 1) * CHUNK_GROUPS > ngrp;
@@ -277,8 +283,8 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
             const global_u16_ptr bp = biases16 ? biases16 + (size_t)ck * CHUNK_GROUPS : (global_u16_ptr)0;
 #pragma unroll
             for (int i = 0; i < ITEMS; ++i) {
-                wreg[i][0] = *(global_u128_ptr)(v + w_off[i]);
-                wreg[i][1] = *(global_u128_ptr)(v + w_off[i] + 16);
+                wreg[i][0] = load_weights(v + w_off[i]);
+                wreg[i][1] = load_weights(v + w_off[i] + 16);
                 sreg[i] = sp[m_off[i]];
                 breg[i] = bp ? (uint32_t)bp[m_off[i]] : 0u;
             }
@@ -288,8 +294,8 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
                 int g = ck * CHUNK_GROUPS + (int)it_grp;
                 const uint32_t back = g < ngrp ? 0u : (uint32_t)(g - (ngrp - 1));     // groups to step back to the last one
                 const global_u8_ptr v = vals + (size_t)ck * (CHUNK_GROUPS * 32);
-                wreg[i][0] = *(global_u128_ptr)(v + (w_off[i] - back * 32));
-                wreg[i][1] = *(global_u128_ptr)(v + (w_off[i] - back * 32) + 16);
+                wreg[i][0] = load_weights(v + (w_off[i] - back * 32));
+                wreg[i][1] = load_weights(v + (w_off[i] - back * 32) + 16);
                 const uint32_t at = m_off[i] + (uint32_t)ck * CHUNK_GROUPS - back;
                 sreg[i] = scales16[at];
                 breg[i] = biases16 ? (uint32_t)biases16[at] : 0u;
