@@ -19,6 +19,16 @@
  *   orc_expf / orc_tanhf / orc_gelu_tanh   no vectors exist in the reference
  *       tree; pinned by fixtures generated from the compiled reference and by
  *       closeness to libm (a dropped Horner term or a wrong constant fails).
+ *   orc_rsqrtf / orc_sqrtf / orc_pow_minus_half   exact powers of four, libm
+ *       within one ulp, the compiled reference on 20k points and the edges.
+ *   orc_rmsnorm / orc_router_input / orc_residual_postnorm /
+ *   orc_parallel_ffn_combine / orc_softcap   the compiled reference
+ *       (bit-equal outputs, same rejections), closed forms (constant
+ *       vectors, a 2^24 + 1 + 1 ... chain that a tree would round
+ *       differently, cancelling branches).
+ *   orc_ffn_block   the compiled reference's public constituents driven in
+ *       feed_forward's order (feed_forward is a static function of the model
+ *       file).
  *   orc_router_topk / orc_sort_selection   brute-force ordering on small E,
  *       weight identities, fixtures from the compiled reference.
  *   orc_mix64 / orc_router_fixture         splitmix64 published test values,
@@ -472,6 +482,192 @@ float orc_gelu_tanh(float x) {
     return half * (1.0f + t);
 }
 
+static double inverse_root64(float x) {
+    uint32_t bits;
+    float seed;
+    memcpy(&bits, &x, 4);
+    bits = UINT32_C(0x5f3759df) - (bits >> 1);
+    memcpy(&seed, &bits, 4);
+    double y = (double)seed, wide = (double)x;
+    for (int i = 0; i < 6; i++) {
+        double square = y * y;
+        double half = 0.5 * wide;
+        double step = 1.5 - half * square;
+        y = y * step;
+    }
+    return y;
+}
+
+float orc_rsqrtf(float x) {
+    if (x != x) return x;
+    if (x < 0.0f) return NAN;
+    if (x == 0.0f) return INFINITY;
+    if (x == 1.0f) return 1.0f;
+    if (x < 0x1p-126f) return orc_rsqrtf(x * 0x1p24f) * 0x1p12f;
+    return (float)inverse_root64(x);
+}
+
+float orc_sqrtf(float x) {
+    if (x != x) return x;
+    if (x < 0.0f) return NAN;
+    if (x == 0.0f || x == 1.0f) return x;
+    if (x < 0x1p-126f) return orc_sqrtf(x * 0x1p24f) * 0x1p-12f;
+    return (float)((double)x * inverse_root64(x));
+}
+
+float orc_pow_minus_half(float x) {
+    if (x == 1.0f) return 1.0f;
+    if (x > 0.0f) return orc_rsqrtf(x);
+    return x;
+}
+
+/* ------------------------------------------------------------------ */
+/* norms and residual combinations                                     */
+/* ------------------------------------------------------------------ */
+
+static int ranges_touch(const void *a, size_t na, const void *b, size_t nb);
+
+static int norm_inverse(const float *x, const float *weight, int n, float eps,
+                        int with_scale, float *inv_out) {
+    float ss = 0.0f;
+    if (!x || n < 1 || !(eps >= 0.0f) || !isfinite(eps) ||
+        (with_scale && !weight))
+        return -1;
+    for (int i = 0; i < n; i++) {
+        if (!isfinite(x[i]) || (with_scale && !isfinite(weight[i]))) return -1;
+        float sq = x[i] * x[i];
+        ss = ss + sq;
+    }
+    float mean = ss / (float)n;
+    float inv = orc_pow_minus_half(mean + eps);
+    if (!isfinite(inv)) return -1;
+    for (int i = 0; i < n; i++) {
+        float y = x[i] * inv;
+        if (with_scale) y = y * weight[i];
+        if (!isfinite(y)) return -1;
+    }
+    *inv_out = inv;
+    return 0;
+}
+
+int orc_rmsnorm(float *out, const float *x, const float *weight, int n,
+                float eps, int with_scale) {
+    float inv;
+    if (!out || n < 1) return -1;
+    size_t bytes = (size_t)n * 4;
+    if ((out != x && x && ranges_touch(out, bytes, x, bytes)) ||
+        (with_scale && weight && ranges_touch(out, bytes, weight, bytes)) ||
+        norm_inverse(x, weight, n, eps, with_scale, &inv) != 0)
+        return -1;
+    for (int i = 0; i < n; i++) {
+        float y = x[i] * inv;
+        if (with_scale) y = y * weight[i];
+        out[i] = y;
+    }
+    return 0;
+}
+
+int orc_router_input(float *out, const float *state, const float *scale,
+                     int hidden, float eps) {
+    float inv;
+    if (!out || !state || !scale || hidden < 1) return -1;
+    size_t bytes = (size_t)hidden * 4;
+    if ((out != state && ranges_touch(out, bytes, state, bytes)) ||
+        ranges_touch(out, bytes, scale, bytes))
+        return -1;
+    for (int i = 0; i < hidden; i++)
+        if (!isfinite(scale[i])) return -1;
+    if (norm_inverse(state, NULL, hidden, eps, 0, &inv) != 0) return -1;
+    float root = 1.0f / orc_sqrtf((float)hidden);
+    for (int pass = 0; pass < 2; pass++)
+        for (int i = 0; i < hidden; i++) {
+            float y = state[i] * inv;
+            y = y * scale[i];
+            y = y * root;
+            if (pass == 0) { if (!isfinite(y)) return -1; }
+            else out[i] = y;
+        }
+    return 0;
+}
+
+int orc_residual_postnorm(float *out, const float *residual,
+                          const float *branch, const float *weight, int n,
+                          float eps) {
+    float inv;
+    if (!out || !residual || !branch || !weight || n < 1) return -1;
+    size_t bytes = (size_t)n * 4;
+    if (ranges_touch(out, bytes, residual, bytes) ||
+        ranges_touch(out, bytes, branch, bytes) ||
+        ranges_touch(out, bytes, weight, bytes))
+        return -1;
+    for (int i = 0; i < n; i++)
+        if (!isfinite(residual[i])) return -1;
+    if (norm_inverse(branch, weight, n, eps, 1, &inv) != 0) return -1;
+    for (int pass = 0; pass < 2; pass++)
+        for (int i = 0; i < n; i++) {
+            float normalized = branch[i] * inv;
+            normalized = normalized * weight[i];
+            float y = residual[i] + normalized;
+            if (pass == 0) { if (!isfinite(y)) return -1; }
+            else out[i] = y;
+        }
+    return 0;
+}
+
+int orc_parallel_ffn_combine(float *out, const float *residual,
+                             const float *dense, const float *routed,
+                             const float *dense_post_weight,
+                             const float *routed_post_weight,
+                             const float *final_post_weight,
+                             float layer_scalar, int n, float eps) {
+    if (!out || !residual || !dense || !routed || !dense_post_weight ||
+        !routed_post_weight || !final_post_weight || n < 1 ||
+        !isfinite(layer_scalar))
+        return -1;
+    size_t bytes = (size_t)n * 4;
+    const void *inputs[6] = {residual, dense, routed, dense_post_weight,
+                             routed_post_weight, final_post_weight};
+    for (int k = 0; k < 6; k++)
+        if (ranges_touch(out, bytes, inputs[k], bytes)) return -1;
+    for (int i = 0; i < n; i++)
+        if (!isfinite(residual[i])) return -1;
+    float *sum = (float *)malloc(2 * bytes);
+    if (!sum) return -1;
+    float *final = sum + n;
+    int rc = -1;
+    if (orc_rmsnorm(sum, dense, dense_post_weight, n, eps, 1) != 0 ||
+        orc_rmsnorm(final, routed, routed_post_weight, n, eps, 1) != 0)
+        goto done;
+    for (int i = 0; i < n; i++) {
+        float combined = sum[i] + final[i];
+        if (!isfinite(combined)) goto done;
+        sum[i] = combined;
+    }
+    if (orc_rmsnorm(final, sum, final_post_weight, n, eps, 1) != 0) goto done;
+    for (int pass = 0; pass < 2; pass++)
+        for (int i = 0; i < n; i++) {
+            float y = residual[i] + final[i];
+            y = y * layer_scalar;
+            if (pass == 0) { if (!isfinite(y)) goto done; }
+            else out[i] = y;
+        }
+    rc = 0;
+done:
+    free(sum);
+    return rc;
+}
+
+int orc_softcap(float *logits, int n, float cap) {
+    if (!logits || n < 1 || !(cap > 0.0f) || !isfinite(cap)) return -1;
+    for (int i = 0; i < n; i++)
+        if (!isfinite(logits[i])) return -1;
+    for (int i = 0; i < n; i++) {
+        float t = orc_tanhf(logits[i] / cap);
+        logits[i] = cap * t;
+    }
+    return 0;
+}
+
 /* ------------------------------------------------------------------ */
 /* routers                                                             */
 /* ------------------------------------------------------------------ */
@@ -767,5 +963,53 @@ int orc_moe_group(const OrcExpertGeometry *g, const unsigned char *pool,
             }
         }
     free(calls); free(scratch); free(pick_out);
+    return rc;
+}
+
+/* ------------------------------------------------------------------ */
+/* feed-forward half of a decoder layer                                */
+/* ------------------------------------------------------------------ */
+
+int orc_ffn_block(const OrcFfnLayer *L, const float *residual, float *output,
+                  int *selected, float *weights, int threads) {
+    if (!L || !residual || !output || L->hidden < 1 || L->dense < 1 ||
+        L->topk < 1 || L->topk > L->n_experts)
+        return -1;
+    size_t H = (size_t)L->hidden, D = (size_t)L->dense;
+    size_t E = (size_t)L->n_experts, K = (size_t)L->topk;
+    float *buf = (float *)malloc((4 * H + 2 * D + E + K) * sizeof(float));
+    int *sel = (int *)malloc(K * sizeof(int));
+    int rc = -1;
+    if (!buf || !sel) goto done;
+    float *norm = buf, *dense_out = buf + H, *routed_out = buf + 2 * H;
+    float *router_in = buf + 3 * H, *gate = buf + 4 * H, *up = gate + D;
+    float *logits = up + D, *w = logits + E;
+    OrcExpertGeometry g = {L->hidden, L->routed};
+
+    if (orc_rmsnorm(norm, residual, L->pre_norm, L->hidden, L->eps, 1) != 0 ||
+        orc_q4_matvec_threads(L->dense_gate[0], L->dense_gate[1], L->dense_gate[2], L->dense, L->hidden, norm, gate,
+                              threads) != 0 ||
+        orc_q4_matvec_threads(L->dense_up[0], L->dense_up[1], L->dense_up[2], L->dense, L->hidden, norm, up,
+                              threads) != 0)
+        goto done;
+    for (size_t i = 0; i < D; i++) gate[i] = orc_gelu_tanh(gate[i]) * up[i];
+    if (orc_q4_matvec_threads(L->dense_down[0], L->dense_down[1], L->dense_down[2], L->hidden, L->dense, gate,
+                              dense_out, threads) != 0)
+        goto done;
+
+    if (orc_router_input(router_in, residual, L->router_scale, L->hidden, L->eps) != 0) goto done;
+    orc_q8_matvec(L->router[0], L->router[1], L->router[2], L->n_experts, L->hidden, router_in, logits);
+    if (orc_rmsnorm(norm, residual, L->pre_norm_2, L->hidden, L->eps, 1) != 0) goto done;
+    if (orc_moe_decode_step(&g, L->pool, L->n_experts, L->topk, logits, L->per_expert_scale, norm, sel, w, NULL,
+                            routed_out, threads) != 0)
+        goto done;
+    if (orc_parallel_ffn_combine(output, residual, dense_out, routed_out, L->post_norm_1, L->post_norm_2,
+                                 L->post_norm, L->layer_scalar, L->hidden, L->eps) != 0)
+        goto done;
+    if (selected) memcpy(selected, sel, K * sizeof(int));
+    if (weights) memcpy(weights, w, K * sizeof(float));
+    rc = 0;
+done:
+    free(buf); free(sel);
     return rc;
 }

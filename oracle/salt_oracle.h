@@ -104,6 +104,40 @@ float orc_tanhf(float x);
 /* reference models/gemma4-26b-a4b/src/gemma4.c:80-83 */
 float orc_gelu_tanh(float x);
 
+/* reference src/bitmath.c:117-142 (six double Newton steps from the
+ * 0x5f3759df seed; tiny inputs rescaled by 2^24) */
+float orc_rsqrtf(float x);
+float orc_sqrtf(float x);
+/* reference src/bitmath.c:107-112 restricted to the exponent -0.5, the only
+ * one the norms use */
+float orc_pow_minus_half(float x);
+
+/* ---- norms and residual combinations of the decoder block (all reject
+ *      non-finite inputs or results with -1 and then write nothing) */
+
+/* reference gemma4.c:46-71, 85-101: ss = serial sum of x*x; inv =
+ * pow(ss / n + eps, -0.5); out = (x * inv) * weight (weight only when
+ * with_scale) */
+int orc_rmsnorm(float *out, const float *x, const float *weight, int n,
+                float eps, int with_scale);
+/* reference gemma4.c:103-130: ((state * inv) * scale) * (1 / sqrt(hidden)) */
+int orc_router_input(float *out, const float *state, const float *scale,
+                     int hidden, float eps);
+/* reference gemma4.c:188-214: residual + (branch * inv) * weight */
+int orc_residual_postnorm(float *out, const float *residual,
+                          const float *branch, const float *weight, int n,
+                          float eps);
+/* reference gemma4.c:216-276: norm(dense) + norm(routed), norm of that sum,
+ * (residual + it) * layer_scalar */
+int orc_parallel_ffn_combine(float *out, const float *residual,
+                             const float *dense, const float *routed,
+                             const float *dense_post_weight,
+                             const float *routed_post_weight,
+                             const float *final_post_weight,
+                             float layer_scalar, int n, float eps);
+/* reference gemma4.c:278-286: cap * tanh(logit / cap), in place */
+int orc_softcap(float *logits, int n, float cap);
+
 /* ---- routers */
 
 /* reference models/gemma4-26b-a4b/src/gemma4.c:132-186 */
@@ -151,6 +185,27 @@ int orc_moe_group(const OrcExpertGeometry *g, const unsigned char *pool,
                   int n_experts, int topk, int batch, const int *selected,
                   const float *weights, const float *inputs, float *outputs,
                   int *group_rows, int threads);
+
+/* ---- the feed-forward half of one decoder layer, one token */
+
+/* Weights of one layer's feed-forward block.  Q4 tensors are [vals|scales|
+ * biases] pointer triples; the router gate is 8-bit affine. */
+typedef struct OrcFfnLayer {
+    int hidden, dense, routed, n_experts, topk;
+    float eps, layer_scalar;
+    const float *pre_norm, *pre_norm_2, *router_scale, *per_expert_scale;
+    const float *post_norm_1, *post_norm_2, *post_norm;
+    const void *dense_gate[3], *dense_up[3], *dense_down[3];
+    const void *router[3];
+    const unsigned char *pool;       /* expert 0; orc_expert_slot_bytes apart */
+} OrcFfnLayer;
+
+/* reference gemma4_text.c:8308-8390 (feed_forward): pre-norm, dense gate/up,
+ * gelu * up, dense down; router input, 8-bit gate, top-k, ascending sort;
+ * second pre-norm, routed experts, weighted sum; parallel combine.
+ * selected / weights (optional) receive the sorted routing. */
+int orc_ffn_block(const OrcFfnLayer *layer, const float *residual,
+                  float *output, int *selected, float *weights, int threads);
 
 #ifdef __cplusplus
 }

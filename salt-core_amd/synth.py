@@ -98,6 +98,35 @@ def expert_views(pool: np.ndarray, expert: int, proj_index: int, hidden: int, ro
     return vals, scales, biases
 
 
+def q8_tensor(R: int, C: int, seed: int):
+    """(vals u8 [R*C], scales u16, biases u16): 8-bit affine, one bf16 scale and bias per 64 flat elements, values
+    spread over about +-0.06."""
+    g = rng(seed)
+    vals = g.integers(0, 256, size=R * C, dtype=np.uint8)
+    groups = (R * C + GROUP - 1) // GROUP
+    scales = f32_to_bf16_bits(g.uniform(0.0003, 0.0006, groups).astype(np.float32))
+    biases = f32_to_bf16_bits(g.uniform(-0.07, -0.04, groups).astype(np.float32))
+    return vals, scales, biases
+
+
+def ffn_layer(hidden: int, dense: int, routed: int, n_experts: int, topk: int, seed: int) -> dict:
+    """Weights of the feed-forward half of one decoder layer: norm weights, dense gate/up/down (affine Q4), the 8-bit
+    router gate, router and per-expert scales, the expert pool."""
+    g = rng(seed)
+    norm = lambda: (1.0 + 0.1 * g.standard_normal(hidden)).astype(np.float32)
+    return {
+        "hidden": hidden, "dense": dense, "routed": routed, "n_experts": n_experts, "topk": topk,
+        "eps": np.float32(1e-6), "layer_scalar": np.float32(0.61),
+        "pre_norm": norm(), "pre_norm_2": norm(), "post_norm_1": norm(), "post_norm_2": norm(), "post_norm": norm(),
+        "router_scale": (1.0 + 0.3 * g.standard_normal(hidden)).astype(np.float32),
+        "per_expert_scale": g.uniform(0.5, 2.0, n_experts).astype(np.float32),
+        "dense_gate": q4_tensor(dense, hidden, seed * 7 + 1), "dense_up": q4_tensor(dense, hidden, seed * 7 + 2),
+        "dense_down": q4_tensor(hidden, dense, seed * 7 + 3),
+        "router": q8_tensor(n_experts, hidden, seed * 7 + 4),
+        "pool": expert_pool(n_experts, hidden, routed, seed * 7 + 5),
+    }
+
+
 def router_logits(n_experts: int, seed: int) -> np.ndarray:
     return rng(seed).standard_normal(size=n_experts).astype(np.float32)
 

@@ -30,6 +30,27 @@ class ExpertGeometry(C.Structure):
     _fields_ = [("hidden", C.c_int), ("routed", C.c_int)]
 
 
+class FfnLayer(C.Structure):
+    """Mirror of OrcFfnLayer; keep() holds the arrays its pointers name."""
+    _fields_ = [("hidden", C.c_int), ("dense", C.c_int), ("routed", C.c_int), ("n_experts", C.c_int), ("topk", C.c_int),
+                ("eps", C.c_float), ("layer_scalar", C.c_float),
+                ("pre_norm", vp), ("pre_norm_2", vp), ("router_scale", vp), ("per_expert_scale", vp),
+                ("post_norm_1", vp), ("post_norm_2", vp), ("post_norm", vp),
+                ("dense_gate", vp * 3), ("dense_up", vp * 3), ("dense_down", vp * 3), ("router", vp * 3), ("pool", vp)]
+
+
+def ffn_layer_struct(w: dict) -> FfnLayer:
+    """OrcFfnLayer over the arrays of a synth.ffn_layer() dictionary (which must outlive it)."""
+    at = lambda a: a.ctypes.data
+    L = FfnLayer(w["hidden"], w["dense"], w["routed"], w["n_experts"], w["topk"], float(w["eps"]), float(w["layer_scalar"]))
+    for name in ("pre_norm", "pre_norm_2", "router_scale", "per_expert_scale", "post_norm_1", "post_norm_2", "post_norm",
+                 "pool"):
+        setattr(L, name, at(w[name]))
+    for name in ("dense_gate", "dense_up", "dense_down", "router"):
+        setattr(L, name, (vp * 3)(*[at(a) for a in w[name]]))
+    return L
+
+
 def _sig(fn, restype, *argtypes):
     fn.restype = restype
     fn.argtypes = list(argtypes)
@@ -71,6 +92,15 @@ def load_oracle() -> C.CDLL:
     _sig(lib.orc_sort_selection, None, vp, vp, i)
     _sig(lib.orc_mix64, C.c_uint64, C.c_uint64)
     _sig(lib.orc_router_fixture, i, vp, vp, i, i, C.c_uint64, i, d)
+    _sig(lib.orc_rsqrtf, f, f)
+    _sig(lib.orc_sqrtf, f, f)
+    _sig(lib.orc_pow_minus_half, f, f)
+    _sig(lib.orc_rmsnorm, i, vp, vp, vp, i, f, i)
+    _sig(lib.orc_router_input, i, vp, vp, vp, i, f)
+    _sig(lib.orc_residual_postnorm, i, vp, vp, vp, vp, i, f)
+    _sig(lib.orc_parallel_ffn_combine, i, vp, vp, vp, vp, vp, vp, vp, f, i, f)
+    _sig(lib.orc_softcap, i, vp, i, f)
+    _sig(lib.orc_ffn_block, i, C.POINTER(FfnLayer), vp, vp, vp, vp, i)
     G = C.POINTER(ExpertGeometry)
     _sig(lib.orc_expert_proj_bytes, sz, G)
     _sig(lib.orc_expert_slot_bytes, sz, G)
@@ -108,6 +138,14 @@ def load_reference() -> C.CDLL | None:
     _sig(lib.salt_gemma4_gelu_tanh, f, f)
     _sig(lib.salt_gemma4_router_topk, i, vp, vp, i, i, vp, vp)
     _sig(lib.salt_mix64, C.c_uint64, C.c_uint64)
+    _sig(lib.salt_rsqrtf, f, f)
+    _sig(lib.salt_sqrtf, f, f)
+    _sig(lib.salt_powf, f, f, f)
+    _sig(lib.salt_gemma4_rmsnorm, i, vp, vp, vp, i, f, i)
+    _sig(lib.salt_gemma4_router_input, i, vp, vp, vp, i, f)
+    _sig(lib.salt_gemma4_residual_postnorm, i, vp, vp, vp, vp, i, f)
+    _sig(lib.salt_gemma4_parallel_ffn_combine, i, vp, vp, vp, vp, vp, vp, vp, f, i, f, vp)
+    _sig(lib.salt_gemma4_softcap, i, vp, i, f)
     return lib
 
 
