@@ -194,6 +194,58 @@ int salt_mi355_q8_matvec_dev(const void *vals, const void *scales,
                              const void *biases, int R, int C, int B,
                              const float *xs, float *ys, void *stream);
 
+/* ---- fp32 cells of a decoder block, device-resident --------------------- */
+
+/* One cell of salt_gpu_exact_cells (include/salt/gpu.h:211-234) over device
+ * pointers.  kind and the meaning of views, n, aux, eps and scalar are the
+ * reference's (src/gpu_hip.cpp:5299-5400):
+ *   1 RMSNORM            views: x, weight (read when aux = 1), out
+ *   2 TOPK               views: logits, per-expert scale, selected (int), weights; n experts, aux = k; ascending ids
+ *   3 RESIDUAL_POSTNORM  views: residual, branch, weight, out
+ *   4 PARALLEL_COMBINE   views: residual, dense, routed, dense / routed / final post-norm weights, scratch (2n), out
+ *   5 SOFTCAP            views: logits (in place); scalar = cap
+ *   6 ROUTER_INPUT       views: state, scale, out; scalar = 1/sqrt(n) or 0 to have it computed
+ * Arithmetic: gemma4.c:46-130, 188-286 (serial sum of squares, pow(., -0.5)
+ * by double Newton steps, separately rounded products): bit-exact. */
+typedef struct SaltMi355Cell {
+    int kind;
+    const void *views[8];
+    uint32_t n, aux;
+    float eps, scalar;
+} SaltMi355Cell;
+
+/* Enqueues the cells in order.  status_dev points at two device ints that the
+ * caller has cleared: [0] becomes -1 when a cell meets a non-finite input or
+ * result (that cell and every later one then publish nothing), [1] is scratch. */
+int salt_mi355_cells_dev(const SaltMi355Cell *cells, int count, int *status_dev,
+                         void *stream);
+
+/* The feed-forward half of one decoder layer for one token, reference
+ * feed_forward (models/gemma4-26b-a4b/src/gemma4_text.c:8308-8390): pre-norm,
+ * dense gate/up (affine Q4), gelu * up, dense down; router input, 8-bit router
+ * gate, top-k; second pre-norm, routed experts, weighted sum; parallel
+ * combine.  Every pointer is a device pointer; Q4 and 8-bit tensors are
+ * {values, scales, biases}. */
+typedef struct SaltMi355FfnLayer {
+    int hidden, dense, routed, n_experts, topk;
+    float eps, layer_scalar;
+    const float *pre_norm, *pre_norm_2, *router_scale, *per_expert_scale;
+    const float *post_norm_1, *post_norm_2, *post_norm;
+    const void *dense_gate[3], *dense_up[3], *dense_down[3];
+    const void *router[3];
+    const void *pool;          /* expert 0 */
+    size_t expert_stride;
+} SaltMi355FfnLayer;
+
+size_t salt_mi355_ffn_block_workspace_bytes(const SaltMi355FfnLayer *layer);
+/* residual and out hold `hidden` floats (distinct buffers); selected / weights
+ * receive the sorted routing (topk entries).  *status_dev (one device int,
+ * cleared by the call) becomes -1 when any step rejects its input; out is then
+ * not written.  workspace: 256-byte aligned, sized by the query above. */
+int salt_mi355_ffn_block_dev(const SaltMi355FfnLayer *layer, const float *residual,
+                             float *out, int *selected, float *weights,
+                             int *status_dev, void *workspace, void *stream);
+
 /* ---- MoE decode layer-step, device-resident ----------------------------- */
 
 /* reference salt_gemma4_router_topk (gemma4.c:132-186).  sorted_by_id = 0

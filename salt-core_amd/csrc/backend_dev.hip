@@ -263,6 +263,161 @@ int salt_mi355_q8_matvec_dev(const void *vals, const void *scales, const void *b
     return 0;
 }
 
+int salt_mi355_cells_dev(const SaltMi355Cell *cells, int count, int *status_dev, void *stream_handle) {
+    hipStream_t stream = (hipStream_t)stream_handle;
+    if (!g_state.ready) { set_error("cells: library not initialised"); return -1; }
+    if (!cells || count < 1 || !status_dev) { set_error("cells: bad arguments"); return -1; }
+    for (int c = 0; c < count; ++c) {
+        const SaltMi355Cell &cell = cells[c];
+        const void *const *v = cell.views;
+        const int n = (int)cell.n;
+        int need = 0, rc = -1;
+        switch (cell.kind) {
+        case 1: need = 3; break;
+        case 2: need = 4; break;
+        case 3: need = 4; break;
+        case 4: need = 8; break;
+        case 5: need = 1; break;
+        case 6: need = 3; break;
+        default: set_error("cells: cell %d has unknown kind %d", c, cell.kind); return -1;
+        }
+        bool ok = cell.n >= 1 && (cell.kind == 5 || cell.n <= 0x7fffffffu);
+        for (int k = 0; k < need; ++k)
+            ok = ok && (v[k] || (cell.kind == 1 && k == 1 && cell.aux == 0)) && ((uintptr_t)v[k] & 3) == 0;
+        if (!ok) { set_error("cells: cell %d has a null or misaligned view, or n = 0", c); return -1; }
+        switch (cell.kind) {
+        case 1:
+            if (cell.aux > 1) { set_error("cells: rmsnorm aux must be 0 or 1"); return -1; }
+            rc = norm_cell_launch(0, (const float *)v[0], cell.aux ? (const float *)v[1] : nullptr, nullptr, (float *)v[2], n,
+                                  cell.eps, 0.0f, status_dev, stream);
+            break;
+        case 2:
+            if (cell.aux < 1 || cell.aux > cell.n) { set_error("cells: topk aux must be in [1, n]"); return -1; }
+            rc = router_topk_launch((const float *)v[0], (const float *)v[1], n, (int)cell.aux, 1, (int *)v[2], (float *)v[3],
+                                    status_dev + 1, stream);
+            if (rc == 0) rc = merge_status_launch(status_dev, status_dev + 1, stream);
+            break;
+        case 3:
+            rc = norm_cell_launch(2, (const float *)v[1], (const float *)v[2], (const float *)v[0], (float *)v[3], n, cell.eps,
+                                  0.0f, status_dev, stream);
+            break;
+        case 4:
+            rc = combine_cell_launch((const float *)v[0], (const float *)v[1], (const float *)v[2], (const float *)v[3],
+                                     (const float *)v[4], (const float *)v[5], (float *)v[6], (float *)v[7], n, cell.eps,
+                                     cell.scalar, status_dev, nullptr, stream);
+            break;
+        case 5:
+            rc = softcap_cell_launch((float *)v[0], cell.n, cell.scalar, status_dev, stream);
+            break;
+        case 6:
+            rc = norm_cell_launch(1, (const float *)v[0], (const float *)v[1], nullptr, (float *)v[2], n, cell.eps, cell.scalar,
+                                  status_dev, stream);
+            break;
+        }
+        if (rc != 0) { set_error("cells: cell %d (kind %d) was refused or failed to launch", c, cell.kind); return -1; }
+    }
+    return 0;
+}
+
+namespace {
+
+struct FfnWorkspace {
+    int *status;               // [0] block, [1] scratch
+    float *norm_a, *norm_b, *router_in, *dense_out, *routed_out, *sum, *gate, *up, *act, *logits, *expert_out;
+    void *moe;
+};
+
+size_t pad256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+size_t ffn_carve(const SaltMi355FfnLayer &L, void *base, FfnWorkspace *ws) {
+    uint8_t *p = (uint8_t *)base;
+    const size_t H = (size_t)L.hidden * 4, D = (size_t)L.dense * 4;
+    auto take = [&](size_t bytes) { uint8_t *at = p; p += pad256(bytes); return at; };
+    FfnWorkspace w;
+    w.status = (int *)take(256);
+    w.norm_a = (float *)take(H); w.norm_b = (float *)take(H); w.router_in = (float *)take(H);
+    w.dense_out = (float *)take(H); w.routed_out = (float *)take(H); w.sum = (float *)take(2 * H);
+    w.gate = (float *)take(D); w.up = (float *)take(D); w.act = (float *)take(D);
+    w.logits = (float *)take((size_t)L.n_experts * 4);
+    w.expert_out = (float *)take((size_t)L.topk * H);
+    w.moe = take(moe_workspace_bytes(MoeGeometry{L.hidden, L.routed, L.n_experts, L.topk}));
+    if (ws) *ws = w;
+    return (size_t)(p - (uint8_t *)base);
+}
+
+bool ffn_layer_ok(const SaltMi355FfnLayer *L) {
+    if (!L || L->hidden < 64 || (L->hidden & 63) || L->routed < 64 || (L->routed & 63) || L->dense < 64 || (L->dense & 63) ||
+        L->n_experts < 1 || L->topk < 1 || L->topk > L->n_experts)
+        return false;
+    const void *need[] = {L->pre_norm, L->pre_norm_2, L->router_scale, L->per_expert_scale, L->post_norm_1, L->post_norm_2,
+                          L->post_norm, L->dense_gate[0], L->dense_gate[1], L->dense_up[0], L->dense_up[1],
+                          L->dense_down[0], L->dense_down[1], L->router[0], L->router[1], L->pool};
+    for (const void *q : need)
+        if (!q) return false;
+    const size_t n = (size_t)L->hidden * (size_t)L->routed;
+    return ((uintptr_t)L->pool & 15) == 0 && (L->expert_stride & 15) == 0 && L->expert_stride >= 3 * (n / 2 + 4 * (n / 64));
+}
+
+}  // namespace
+
+size_t salt_mi355_ffn_block_workspace_bytes(const SaltMi355FfnLayer *layer) {
+    return ffn_layer_ok(layer) ? ffn_carve(*layer, nullptr, nullptr) : 0;
+}
+
+int salt_mi355_ffn_block_dev(const SaltMi355FfnLayer *layer, const float *residual, float *out, int *selected,
+                             float *weights, int *status_dev, void *workspace, void *stream_handle) {
+    hipStream_t stream = (hipStream_t)stream_handle;
+    if (!g_state.ready) { set_error("ffn block: library not initialised"); return -1; }
+    if (!ffn_layer_ok(layer) || !residual || !out || !selected || !weights || !status_dev || !workspace ||
+        ((uintptr_t)workspace & 255) || residual == out) {
+        set_error("ffn block: bad arguments (hidden, dense, routed multiples of 64; workspace 256-byte aligned)");
+        return -1;
+    }
+    const SaltMi355FfnLayer &L = *layer;
+    FfnWorkspace ws;
+    ffn_carve(L, workspace, &ws);
+    const MoeGeometry g = {L.hidden, L.routed, L.n_experts, L.topk};
+    MoeWorkspace moe;
+    moe_workspace_carve(g, ws.moe, &moe);
+    if (clear_words_launch(ws.status, 2, stream) != 0 ||
+        ffn_pre_launch(residual, L.pre_norm, L.pre_norm_2, L.router_scale, ws.norm_a, ws.norm_b, ws.router_in, L.hidden, L.eps,
+                       ws.status, stream) != 0) {
+        set_error("ffn block: pre-norm launch failed");
+        return -1;
+    }
+    // dense branch
+    SaltMi355Q4Job gate_up[2];
+    gate_up[0].vals = L.dense_gate[0]; gate_up[0].scales = L.dense_gate[1]; gate_up[0].biases = L.dense_gate[2];
+    gate_up[1].vals = L.dense_up[0]; gate_up[1].scales = L.dense_up[1]; gate_up[1].biases = L.dense_up[2];
+    gate_up[0].xs = gate_up[1].xs = ws.norm_a;
+    gate_up[0].ys = ws.gate; gate_up[1].ys = ws.up;
+    gate_up[0].rows = gate_up[1].rows = L.dense;
+    if (salt_mi355_q4_jobs_dev(gate_up, 2, L.hidden, 1, 0, stream) != 0 ||
+        moe_activate_launch(ws.gate, ws.up, ws.act, (size_t)L.dense, stream) != 0 ||
+        salt_mi355_q4_matvec_dev(L.dense_down[0], L.dense_down[1], L.dense_down[2], L.hidden, L.dense, 1, ws.act,
+                                 ws.dense_out, 0, stream) != 0)
+        return -1;
+    // routed branch
+    if (salt_mi355_q8_matvec_dev(L.router[0], L.router[1], L.router[2], L.n_experts, L.hidden, 1, ws.router_in, ws.logits,
+                                 stream) != 0)
+        return -1;
+    if (moe_decode_step_launch(g, (const uint8_t *)L.pool, L.expert_stride, ws.logits, L.per_expert_scale, ws.norm_b,
+                               selected, weights, ws.expert_out, ws.routed_out, moe, g_state.code_scale, stream) != 0) {
+        set_error("ffn block: unsupported MoE geometry or launch failure");
+        return -1;
+    }
+    // A rejected residual leaves the branch buffers unwritten: the router then works on whatever they held, which it
+    // either rejects or routes harmlessly; the combine below publishes nothing in both cases.
+    if (merge_status_launch(ws.status, moe.status, stream) != 0 ||
+        combine_cell_launch(residual, ws.dense_out, ws.routed_out, L.post_norm_1, L.post_norm_2, L.post_norm, ws.sum, out,
+                            L.hidden, L.eps, L.layer_scalar, ws.status, nullptr, stream) != 0 ||
+        hip_ok(hipMemcpyAsync(status_dev, ws.status, sizeof(int), hipMemcpyDeviceToDevice, stream), "ffn block status") != 0) {
+        set_error("ffn block: combine launch failed");
+        return -1;
+    }
+    return 0;
+}
+
 int salt_mi355_router_topk_dev(const float *logits, const float *per_expert_scale, int n_experts, int topk,
                                int sorted_by_id, int *selected, float *weights, int *status_dev, void *stream) {
     if (!g_state.ready) { set_error("router: library not initialised"); return -1; }

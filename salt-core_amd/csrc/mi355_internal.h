@@ -184,6 +184,20 @@ struct Q8Launch {
 };
 int q8_launch(const Q8Launch &launch, hipStream_t stream);
 
+// ---------------------------------------------------------------- fp32 cells of a decoder block
+
+// Each launcher enqueues kernels that do nothing when *status != 0 and set it to -1 (publishing nothing) when an
+// input or a result is not finite.  kind: 0 rms norm (weight optional), 1 router input, 2 residual post-norm.
+int norm_cell_launch(int kind, const float *x, const float *weight, const float *residual, float *out, int n, float eps,
+                     float root, int *status, hipStream_t stream);
+int ffn_pre_launch(const float *residual, const float *w1, const float *w2, const float *router_scale, float *norm_a,
+                   float *norm_b, float *router_in, int n, float eps, int *status, hipStream_t stream);
+int combine_cell_launch(const float *residual, const float *dense, const float *routed, const float *wd, const float *wr,
+                        const float *wf, float *sum_scratch, float *out, int n, float eps, float scalar, int *status,
+                        const int *other_status, hipStream_t stream);
+int softcap_cell_launch(float *logits, size_t n, float cap, int *status, hipStream_t stream);
+int merge_status_launch(int *status, const int *other, hipStream_t stream);
+
 // ---------------------------------------------------------------- MoE
 
 struct MoeGeometry {

@@ -21,6 +21,22 @@ class Fp4Job(C.Structure):
                 ("rows", C.c_int)]
 
 
+class Cell(C.Structure):
+    _fields_ = [("kind", C.c_int), ("views", vp * 8), ("n", C.c_uint32), ("aux", C.c_uint32), ("eps", C.c_float),
+                ("scalar", C.c_float)]
+
+
+class FfnLayerDesc(C.Structure):
+    _fields_ = [("hidden", C.c_int), ("dense", C.c_int), ("routed", C.c_int), ("n_experts", C.c_int), ("topk", C.c_int),
+                ("eps", C.c_float), ("layer_scalar", C.c_float),
+                ("pre_norm", vp), ("pre_norm_2", vp), ("router_scale", vp), ("per_expert_scale", vp),
+                ("post_norm_1", vp), ("post_norm_2", vp), ("post_norm", vp),
+                ("dense_gate", vp * 3), ("dense_up", vp * 3), ("dense_down", vp * 3), ("router", vp * 3),
+                ("pool", vp), ("expert_stride", C.c_size_t)]
+
+
+CELL_RMSNORM, CELL_TOPK, CELL_RESIDUAL_POSTNORM, CELL_PARALLEL_COMBINE, CELL_SOFTCAP, CELL_ROUTER_INPUT = 1, 2, 3, 4, 5, 6
+
 _lib = None
 
 INCLUDE_DIR = Path(__file__).resolve().parent.parent / "include"
@@ -80,6 +96,9 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_nvfp4_matmul_dev, i, vp, vp, f, f, i, i, i, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_bf16_matvec_dev, i, vp, i, i, i, vp, vp, vp, vp)
     _sig(lib.salt_mi355_q8_matvec_dev, i, vp, vp, vp, i, i, i, vp, vp, vp)
+    _sig(lib.salt_mi355_cells_dev, i, C.POINTER(Cell), i, vp, vp)
+    _sig(lib.salt_mi355_ffn_block_workspace_bytes, sz, C.POINTER(FfnLayerDesc))
+    _sig(lib.salt_mi355_ffn_block_dev, i, C.POINTER(FfnLayerDesc), vp, vp, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_router_topk_dev, i, vp, vp, i, i, i, vp, vp, vp, vp)
     _sig(lib.salt_mi355_moe_workspace_bytes, sz, i, i, i, i)
     _sig(lib.salt_mi355_moe_decode_step_dev, i, vp, sz, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, vp, vp)
@@ -269,6 +288,57 @@ def router_topk(logits: np.ndarray, scale: np.ndarray, topk: int, sorted_by_id: 
           "router_topk_dev")
     check(lib.salt_mi355_stream_sync(stream), "sync")
     return int(st.to_host(np.int32)[0]), sel.to_host(np.int32), w.to_host(np.float32)
+
+
+def run_cells(cells: list[tuple], arrays: dict[str, np.ndarray]) -> tuple[int, dict[str, np.ndarray]]:
+    """Runs a sequence of cells over host arrays.  Each cell is (kind, [names of its views], n, aux, eps, scalar); a
+    name maps to one device buffer for the whole sequence (so aliasing is expressed by repeating a name).  Returns the
+    status word and every array as it is on the device afterwards."""
+    lib = init()
+    bufs = {k: DeviceBuffer.from_host(v) for k, v in arrays.items()}
+    status = DeviceBuffer(8, fill=0)
+    table = (Cell * len(cells))()
+    for c, (kind, names, n, aux, eps, scalar) in enumerate(cells):
+        views = (vp * 8)(*[bufs[name].ptr if name is not None else None for name in names] + [None] * (8 - len(names)))
+        table[c] = Cell(kind, views, n, aux, eps, scalar)
+    stream = lib.salt_mi355_stream()
+    check(lib.salt_mi355_cells_dev(table, len(cells), status.ptr, stream), "cells_dev")
+    check(lib.salt_mi355_stream_sync(stream), "sync")
+    return int(status.to_host(np.int32)[0]), {k: b.to_host(arrays[k].dtype) for k, b in bufs.items()}
+
+
+class FfnBlock:
+    """The weights of one layer's feed-forward block (a synth.ffn_layer dictionary) resident in HBM."""
+
+    def __init__(self, w: dict):
+        self.lib = init()
+        self.H, self.K = w["hidden"], w["topk"]
+        self.bufs = {}
+        up = lambda name, a: self.bufs.setdefault(name, DeviceBuffer.from_host(a)).ptr
+        d = FfnLayerDesc(w["hidden"], w["dense"], w["routed"], w["n_experts"], w["topk"], float(w["eps"]),
+                         float(w["layer_scalar"]))
+        for name in ("pre_norm", "pre_norm_2", "router_scale", "per_expert_scale", "post_norm_1", "post_norm_2",
+                     "post_norm", "pool"):
+            setattr(d, name, up(name, w[name]))
+        for name in ("dense_gate", "dense_up", "dense_down", "router"):
+            setattr(d, name, (vp * 3)(*[up(f"{name}{k}", a) for k, a in enumerate(w[name])]))
+        d.expert_stride = w["pool"].nbytes // w["n_experts"]
+        self.desc = d
+        self.ws = DeviceBuffer(self.lib.salt_mi355_ffn_block_workspace_bytes(C.byref(d)), fill=0)
+        self.residual, self.out = DeviceBuffer(self.H * 4), DeviceBuffer(self.H * 4, fill=0xFF)
+        self.sel, self.w, self.status = DeviceBuffer(self.K * 4), DeviceBuffer(self.K * 4), DeviceBuffer(4, fill=0x55)
+
+    def enqueue(self, stream):
+        return self.lib.salt_mi355_ffn_block_dev(C.byref(self.desc), self.residual.ptr, self.out.ptr, self.sel.ptr,
+                                                 self.w.ptr, self.status.ptr, self.ws.ptr, stream)
+
+    def step(self, residual: np.ndarray):
+        self.residual.upload(np.ascontiguousarray(residual, np.float32))
+        stream = self.lib.salt_mi355_stream()
+        check(self.enqueue(stream), "ffn_block_dev")
+        check(self.lib.salt_mi355_stream_sync(stream), "sync")
+        return (int(self.status.to_host(np.int32)[0]), self.sel.to_host(np.int32), self.w.to_host(np.float32),
+                self.out.to_host(np.float32))
 
 
 class MoeLayer:
