@@ -140,9 +140,16 @@ int salt_mi355_init(void) {
     }
     s.compute_units = prop.multiProcessorCount;
     if (hip_ok(hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking), "hipStreamCreate") != 0) return -1;
-    if (verify_converters() != 0) {
+    if (hip_ok(hipStreamCreateWithFlags(&s.side, hipStreamNonBlocking), "hipStreamCreate side") != 0 ||
+        hip_ok(hipEventCreateWithFlags(&s.fork, hipEventDisableTiming | hipEventDisableSystemFence), "hipEventCreate fork") != 0 ||
+        hip_ok(hipEventCreateWithFlags(&s.join, hipEventDisableTiming | hipEventDisableSystemFence), "hipEventCreate join") != 0 ||
+        verify_converters() != 0) {
         (void)hipStreamDestroy(s.stream);
-        s.stream = nullptr;
+        if (s.side) (void)hipStreamDestroy(s.side);
+        if (s.fork) (void)hipEventDestroy(s.fork);
+        if (s.join) (void)hipEventDestroy(s.join);
+        s.stream = s.side = nullptr;
+        s.fork = s.join = nullptr;
         return -1;
     }
     const char *fused = getenv("SALT_MI355_Q4_FUSED");
@@ -163,6 +170,9 @@ int salt_mi355_shutdown(void) {
         if (slot.done) (void)hipEventDestroy(slot.done);
     }
     if (s.stream) failed |= hip_ok(hipStreamDestroy(s.stream), "hipStreamDestroy");
+    if (s.side) failed |= hip_ok(hipStreamDestroy(s.side), "hipStreamDestroy side");
+    if (s.fork) (void)hipEventDestroy(s.fork);
+    if (s.join) (void)hipEventDestroy(s.join);
     char keep[sizeof s.last_error];
     memcpy(keep, s.last_error, sizeof keep);
     s = State();

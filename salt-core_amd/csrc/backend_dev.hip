@@ -304,7 +304,7 @@ int salt_mi355_cells_dev(const SaltMi355Cell *cells, int count, int *status_dev,
         case 4:
             rc = combine_cell_launch((const float *)v[0], (const float *)v[1], (const float *)v[2], (const float *)v[3],
                                      (const float *)v[4], (const float *)v[5], (float *)v[6], (float *)v[7], n, cell.eps,
-                                     cell.scalar, status_dev, nullptr, stream);
+                                     cell.scalar, status_dev, nullptr, nullptr, nullptr, 0, stream);
             break;
         case 5:
             rc = softcap_cell_launch((float *)v[0], cell.n, cell.scalar, status_dev, stream);
@@ -322,7 +322,7 @@ int salt_mi355_cells_dev(const SaltMi355Cell *cells, int count, int *status_dev,
 namespace {
 
 struct FfnWorkspace {
-    int *status;               // [0] block, [1] scratch
+    Q4Job *dense_jobs;         // two records written by the opening kernel
     float *norm_a, *norm_b, *router_in, *dense_out, *routed_out, *sum, *gate, *up, *act, *logits, *expert_out;
     void *moe;
 };
@@ -334,7 +334,7 @@ size_t ffn_carve(const SaltMi355FfnLayer &L, void *base, FfnWorkspace *ws) {
     const size_t H = (size_t)L.hidden * 4, D = (size_t)L.dense * 4;
     auto take = [&](size_t bytes) { uint8_t *at = p; p += pad256(bytes); return at; };
     FfnWorkspace w;
-    w.status = (int *)take(256);
+    w.dense_jobs = (Q4Job *)take(2 * sizeof(Q4Job));
     w.norm_a = (float *)take(H); w.norm_b = (float *)take(H); w.router_in = (float *)take(H);
     w.dense_out = (float *)take(H); w.routed_out = (float *)take(H); w.sum = (float *)take(2 * H);
     w.gate = (float *)take(D); w.up = (float *)take(D); w.act = (float *)take(D);
@@ -379,39 +379,60 @@ int salt_mi355_ffn_block_dev(const SaltMi355FfnLayer *layer, const float *residu
     const MoeGeometry g = {L.hidden, L.routed, L.n_experts, L.topk};
     MoeWorkspace moe;
     moe_workspace_carve(g, ws.moe, &moe);
-    if (clear_words_launch(ws.status, 2, stream) != 0 ||
-        ffn_pre_launch(residual, L.pre_norm, L.pre_norm_2, L.router_scale, ws.norm_a, ws.norm_b, ws.router_in, L.hidden, L.eps,
-                       ws.status, stream) != 0) {
+
+    // dense gate and up as one two-job launch; the job records reach the device inside the opening kernel's arguments
+    Q4Job dense[2];
+    memset(dense, 0, sizeof dense);
+    for (int k = 0; k < 2; ++k) {
+        const void *const *t = k == 0 ? L.dense_gate : L.dense_up;
+        dense[k].vals = (const uint8_t *)t[0]; dense[k].scales = (const uint8_t *)t[1]; dense[k].biases = (const uint8_t *)t[2];
+        dense[k].x = ws.norm_a; dense[k].y = k == 0 ? ws.gate : ws.up;
+        dense[k].rows = L.dense; dense[k].x_stride = L.hidden; dense[k].y_stride = L.dense;
+    }
+    Q4Launch gate_up;
+    memset(&gate_up, 0, sizeof gate_up);
+    gate_up.total_tiles = q4_assign_tiles(dense, 2);
+    gate_up.table = ws.dense_jobs; gate_up.njobs = 2; gate_up.cols = L.hidden; gate_up.tokens = 1;
+    gate_up.code_scale = g_state.code_scale; gate_up.fused = g_state.q4_fused;
+    const bool tileable = q4_job_is_tileable(dense[0], L.hidden) && q4_job_is_tileable(dense[1], L.hidden);
+
+    if (ffn_pre_launch(residual, L.pre_norm, L.pre_norm_2, L.router_scale, ws.norm_a, ws.norm_b, ws.router_in, L.hidden, L.eps,
+                       status_dev, dense, ws.dense_jobs, stream) != 0) {
         set_error("ffn block: pre-norm launch failed");
         return -1;
     }
-    // dense branch
-    SaltMi355Q4Job gate_up[2];
-    gate_up[0].vals = L.dense_gate[0]; gate_up[0].scales = L.dense_gate[1]; gate_up[0].biases = L.dense_gate[2];
-    gate_up[1].vals = L.dense_up[0]; gate_up[1].scales = L.dense_up[1]; gate_up[1].biases = L.dense_up[2];
-    gate_up[0].xs = gate_up[1].xs = ws.norm_a;
-    gate_up[0].ys = ws.gate; gate_up[1].ys = ws.up;
-    gate_up[0].rows = gate_up[1].rows = L.dense;
-    if (salt_mi355_q4_jobs_dev(gate_up, 2, L.hidden, 1, 0, stream) != 0 ||
-        moe_activate_launch(ws.gate, ws.up, ws.act, (size_t)L.dense, stream) != 0 ||
-        salt_mi355_q4_matvec_dev(L.dense_down[0], L.dense_down[1], L.dense_down[2], L.hidden, L.dense, 1, ws.act,
-                                 ws.dense_out, 0, stream) != 0)
+    // The dense branch runs beside the routed one on the library's second stream.
+    hipStream_t side = g_state.side;
+    if (hip_ok(hipEventRecord(g_state.fork, stream), "ffn block fork") != 0 ||
+        hip_ok(hipStreamWaitEvent(side, g_state.fork, 0), "ffn block fork wait") != 0)
         return -1;
-    // routed branch
+    int rc = tileable ? q4_launch(gate_up, 0, side) : q4_launch_generic(gate_up, side);
+    if (rc == 0) rc = moe_activate_launch(ws.gate, ws.up, ws.act, (size_t)L.dense, side);
+    if (rc == 0)
+        rc = salt_mi355_q4_matvec_dev(L.dense_down[0], L.dense_down[1], L.dense_down[2], L.hidden, L.dense, 1, ws.act,
+                                      ws.dense_out, 0, side);
+    // the join is recorded even after a failure, so that the caller's stream never outruns the side stream
+    const int recorded = hip_ok(hipEventRecord(g_state.join, side), "ffn block join");
+    if (rc != 0 || recorded != 0) {
+        (void)hipStreamWaitEvent(stream, g_state.join, 0);
+        set_error("ffn block: dense branch failed to launch");
+        return -1;
+    }
+
+    // routed branch; a rejected residual leaves its inputs unwritten: the router then works on whatever they held,
+    // which it either rejects or routes harmlessly, and the combine publishes nothing in both cases
     if (salt_mi355_q8_matvec_dev(L.router[0], L.router[1], L.router[2], L.n_experts, L.hidden, 1, ws.router_in, ws.logits,
                                  stream) != 0)
         return -1;
     if (moe_decode_step_launch(g, (const uint8_t *)L.pool, L.expert_stride, ws.logits, L.per_expert_scale, ws.norm_b,
-                               selected, weights, ws.expert_out, ws.routed_out, moe, g_state.code_scale, stream) != 0) {
+                               selected, weights, ws.expert_out, nullptr, moe, g_state.code_scale, stream) != 0) {
         set_error("ffn block: unsupported MoE geometry or launch failure");
         return -1;
     }
-    // A rejected residual leaves the branch buffers unwritten: the router then works on whatever they held, which it
-    // either rejects or routes harmlessly; the combine below publishes nothing in both cases.
-    if (merge_status_launch(ws.status, moe.status, stream) != 0 ||
-        combine_cell_launch(residual, ws.dense_out, ws.routed_out, L.post_norm_1, L.post_norm_2, L.post_norm, ws.sum, out,
-                            L.hidden, L.eps, L.layer_scalar, ws.status, nullptr, stream) != 0 ||
-        hip_ok(hipMemcpyAsync(status_dev, ws.status, sizeof(int), hipMemcpyDeviceToDevice, stream), "ffn block status") != 0) {
+    if (hip_ok(hipStreamWaitEvent(stream, g_state.join, 0), "ffn block join wait") != 0) return -1;
+    if (combine_cell_launch(residual, ws.dense_out, ws.routed_out, L.post_norm_1, L.post_norm_2, L.post_norm, ws.sum, out,
+                            L.hidden, L.eps, L.layer_scalar, status_dev, moe.status, ws.expert_out, weights, L.topk,
+                            stream) != 0) {
         set_error("ffn block: combine launch failed");
         return -1;
     }

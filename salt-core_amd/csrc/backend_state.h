@@ -13,6 +13,8 @@ struct State {
     int ready = 0;
     int compute_units = 0;
     hipStream_t stream = nullptr;
+    hipStream_t side = nullptr;         // second branch of a forked sequence (default priority, like every stream)
+    hipEvent_t fork = nullptr, join = nullptr;
     float code_scale = 0.0f;            // 1 / fp8_table[1]
     int q4_fused = 0;                   // 1: fma accumulate (tolerance class) instead of mul + add
     int fp8_is_ocp = 0;                 // the converter decodes every byte as OCP E4M3FN

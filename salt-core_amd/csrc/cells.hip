@@ -13,8 +13,9 @@
 namespace mi355 {
 namespace {
 
-constexpr int THREADS = 256;
-constexpr int SQ_CHUNK = 4096;          // squares staged per pass of the serial adder
+constexpr int THREADS = 1024;         // one workgroup per cell: sixteen waves keep enough loads in flight
+constexpr int SLOTS = 4;              // elements a thread handles per pass: i = base + tid + k * THREADS
+constexpr int SQ_CHUNK = SLOTS * THREADS;   // squares staged per pass of the serial adder
 
 __device__ __forceinline__ double inverse_root64(float x) {
     const float seed = __uint_as_float(0x5f3759dfu - (__float_as_uint(x) >> 1));
@@ -62,39 +63,73 @@ __device__ __forceinline__ float pow_minus_half(float x) {
     return x;
 }
 
-__device__ __forceinline__ bool finite(float v) { return (__float_as_uint(v) & 0x7f800000u) != 0x7f800000u; }
+// 1 for an infinity or a NaN; an unsigned, so that flags combine with | and no load hides behind a short circuit
+__device__ __forceinline__ unsigned nonfinite(float v) { return (__float_as_uint(v) & 0x7f800000u) == 0x7f800000u; }
 
-// Serial sums of squares of `vectors` (1..4) vectors of n floats: vector v is x[v].  Returns the sums in ss[] on
-// every thread.  bad is set when an element is not finite.  sq is LDS scratch of vectors * SQ_CHUNK floats.
+// Visits the elements [0, n) SLOTS at a time per thread: f(i, k) for the live slots of a pass, all loads of a pass
+// being independent of each other.
+template <typename F>
+__device__ __forceinline__ void each_element(int n, F f) {
+    for (int base = 0; base < n; base += SQ_CHUNK) {
+#pragma unroll
+        for (int k = 0; k < SLOTS; ++k) {
+            const int i = base + (int)threadIdx.x + k * THREADS;
+            if (i < n) f(i);
+        }
+    }
+}
+
+// Serial sums of squares of `vectors` (1 or 2) vectors of n floats: lane v of wave 0 adds vector v's squares left to
+// right.  Returns the sums in ss_out[] on every thread; `bad` collects non-finite elements.  sq is LDS scratch of
+// vectors * SQ_CHUNK floats, shared of at least `vectors` floats.
 __device__ void serial_square_sums(const float *const *x, int vectors, int n, float *sq, float *ss_out, float *shared,
-                                   bool &bad) {
+                                   unsigned &bad) {
     const int tid = threadIdx.x;
-    float acc = 0.0f;                                   // lane v of wave 0 owns vector v
+    float acc = 0.0f;
     for (int base = 0; base < n; base += SQ_CHUNK) {
         const int count = n - base < SQ_CHUNK ? n - base : SQ_CHUNK;
-        for (int v = 0; v < vectors; ++v)
-            for (int i = tid; i < count; i += THREADS) {
-                const float value = x[v][base + i];
-                bad = bad || !finite(value);
-                sq[v * SQ_CHUNK + i] = value * value;
-            }
-        __syncthreads();
-        if (tid < vectors) {
-            const float *mine = sq + tid * SQ_CHUNK;
-            int i = 0;
-            for (; i + 16 <= count; i += 16) {
-                float4 p[4];
+        for (int v = 0; v < vectors; ++v) {
+            const float *src = x[v] + base;
 #pragma unroll
-                for (int k = 0; k < 4; ++k) p[k] = *(const float4 *)&mine[i + 4 * k];
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    acc = acc + p[k].x;
-                    acc = acc + p[k].y;
-                    acc = acc + p[k].z;
-                    acc = acc + p[k].w;
+            for (int k = 0; k < SLOTS; ++k) {
+                const int i = tid + k * THREADS;
+                if (i < count) {
+                    const float value = src[i];
+                    bad |= nonfinite(value);
+                    sq[v * SQ_CHUNK + i] = value * value;
                 }
             }
-            for (; i < count; ++i) acc = acc + mine[i];
+        }
+        __syncthreads();
+        if (tid < vectors) {
+            // 32 squares per batch; the next batch is read from LDS while the current one is added
+            const float *mine = sq + tid * SQ_CHUNK;
+            const int full = count & ~31;
+            float4 a[8], b[8];
+            auto fetch = [&](float4 (&dst)[8], int at) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) dst[k] = *(const float4 *)&mine[at + 4 * k];
+            };
+            auto add = [&](const float4 (&src)[8]) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    acc = acc + src[k].x;
+                    acc = acc + src[k].y;
+                    acc = acc + src[k].z;
+                    acc = acc + src[k].w;
+                }
+            };
+            if (full) fetch(a, 0);
+            for (int i = 0; i < full; i += 64) {
+                const bool second = i + 32 < full;
+                if (second) fetch(b, i + 32);
+                add(a);
+                if (second) {
+                    if (i + 64 < full) fetch(a, i + 64);
+                    add(b);
+                }
+            }
+            for (int i = full; i < count; ++i) acc = acc + mine[i];
         }
         __syncthreads();
     }
@@ -124,35 +159,33 @@ __global__ __launch_bounds__(THREADS) void norm_cell_kernel(NormArgs a) {
     __shared__ __attribute__((aligned(16))) float sq[SQ_CHUNK];
     __shared__ float shared[4];
     if (*a.status != 0) return;
-    bool bad = !(a.eps >= 0.0f) || !finite(a.eps);
+    unsigned bad = !(a.eps >= 0.0f) || nonfinite(a.eps);
     const float *vec[1] = {a.x};
     float ss;
     serial_square_sums(vec, 1, a.n, sq, &ss, shared, bad);
     const float inv = inverse_from_sum(ss, a.n, a.eps);
-    bad = bad || !finite(inv);
+    bad |= nonfinite(inv);
     float root = a.root;
     if (a.kind == 1 && !(root > 0.0f)) root = 1.0f / det_sqrtf((float)a.n);
-    for (int i = threadIdx.x; i < a.n; i += THREADS) {
+    auto value = [&](int i, unsigned &flag) {
         float y = a.x[i] * inv;
-        if (a.weight) { bad = bad || !finite(a.weight[i]); y = y * a.weight[i]; }
+        if (a.weight) { const float w = a.weight[i]; flag |= nonfinite(w); y = y * w; }
         if (a.kind == 1) y = y * root;
-        bad = bad || !finite(y);
+        flag |= nonfinite(y);
         if (a.kind == 2) {
-            bad = bad || !finite(a.residual[i]);
-            bad = bad || !finite(a.residual[i] + y);
+            const float r = a.residual[i];
+            y = r + y;
+            flag |= nonfinite(r) | nonfinite(y);
         }
-    }
-    if (__syncthreads_or(bad)) {
+        return y;
+    };
+    each_element(a.n, [&](int i) { (void)value(i, bad); });
+    if (__syncthreads_or((int)bad)) {
         if (threadIdx.x == 0) *a.status = -1;
         return;
     }
-    for (int i = threadIdx.x; i < a.n; i += THREADS) {
-        float y = a.x[i] * inv;
-        if (a.weight) y = y * a.weight[i];
-        if (a.kind == 1) y = y * root;
-        if (a.kind == 2) y = a.residual[i] + y;
-        a.out[i] = y;
-    }
+    unsigned ignored = 0;
+    each_element(a.n, [&](int i) { a.out[i] = value(i, ignored); });
 }
 
 // One pass over the residual for the three vectors a feed-forward block derives from it:
@@ -162,35 +195,36 @@ struct PreArgs {
     float *norm_a, *norm_b, *router_in;
     int n;
     float eps;
-    int *status;
+    int *status;               // written, not only set: this kernel opens the block
+    Q4Job jobs[2];             // copied to jobs_out for the launch that follows
+    Q4Job *jobs_out;
 };
 
 __global__ __launch_bounds__(THREADS) void ffn_pre_kernel(PreArgs a) {
     __shared__ __attribute__((aligned(16))) float sq[SQ_CHUNK];
     __shared__ float shared[4];
-    if (*a.status != 0) return;
-    bool bad = !(a.eps >= 0.0f) || !finite(a.eps);
+    if (a.jobs_out && threadIdx.x < 2) a.jobs_out[threadIdx.x] = a.jobs[threadIdx.x];
+    unsigned bad = !(a.eps >= 0.0f) || nonfinite(a.eps);
     const float *vec[1] = {a.residual};
     float ss;
     serial_square_sums(vec, 1, a.n, sq, &ss, shared, bad);
     const float inv = inverse_from_sum(ss, a.n, a.eps);
-    bad = bad || !finite(inv);
+    bad |= nonfinite(inv);
     const float root = 1.0f / det_sqrtf((float)a.n);
-    for (int i = threadIdx.x; i < a.n; i += THREADS) {
-        const float y = a.residual[i] * inv;
-        bad = bad || !finite(a.w1[i]) || !finite(a.w2[i]) || !finite(a.router_scale[i]);
-        bad = bad || !finite(y) || !finite(y * a.w1[i]) || !finite(y * a.w2[i]) || !finite((y * a.router_scale[i]) * root);
-    }
-    if (__syncthreads_or(bad)) {
-        if (threadIdx.x == 0) *a.status = -1;
-        return;
-    }
-    for (int i = threadIdx.x; i < a.n; i += THREADS) {
+    each_element(a.n, [&](int i) {
+        const float y = a.residual[i] * inv, w1 = a.w1[i], w2 = a.w2[i], rs = a.router_scale[i];
+        bad |= nonfinite(w1) | nonfinite(w2) | nonfinite(rs) | nonfinite(y) | nonfinite(y * w1) | nonfinite(y * w2) |
+               nonfinite((y * rs) * root);
+    });
+    const bool failed = __syncthreads_or((int)bad);
+    if (threadIdx.x == 0) *a.status = failed ? -1 : 0;
+    if (failed) return;
+    each_element(a.n, [&](int i) {
         const float y = a.residual[i] * inv;
         a.norm_a[i] = y * a.w1[i];
         a.norm_b[i] = y * a.w2[i];
         a.router_in[i] = (y * a.router_scale[i]) * root;
-    }
+    });
 }
 
 // out = (residual + norm(norm(dense) * wd + norm(routed) * wr) * wf) * scalar.  `other` is a second status word
@@ -202,6 +236,9 @@ struct CombineArgs {
     float eps, scalar;
     int *status;
     const int *other;
+    // when expert_out is given, routed (writable then) is first filled with sum_k expert_out[k] * weights[k], k ascending
+    const float *expert_out, *weights;
+    int topk;
 };
 
 __global__ __launch_bounds__(THREADS) void combine_cell_kernel(CombineArgs a) {
@@ -212,50 +249,77 @@ __global__ __launch_bounds__(THREADS) void combine_cell_kernel(CombineArgs a) {
         if (threadIdx.x == 0) *a.status = -1;
         return;
     }
-    bool bad = !(a.eps >= 0.0f) || !finite(a.eps) || !finite(a.scalar);
+    unsigned bad = !(a.eps >= 0.0f) || nonfinite(a.eps) || nonfinite(a.scalar);
+    if (a.expert_out) {                                 // each thread later reads back only what it wrote here
+        float *routed = const_cast<float *>(a.routed);
+        for (int base = 0; base < a.n; base += SQ_CHUNK) {
+            float sum[SLOTS];
+#pragma unroll
+            for (int k = 0; k < SLOTS; ++k) sum[k] = 0.0f;
+            for (int e = 0; e < a.topk; ++e) {
+                const float w = a.weights[e];
+#pragma unroll
+                for (int k = 0; k < SLOTS; ++k) {
+                    const int i = base + (int)threadIdx.x + k * THREADS;
+                    if (i < a.n) {
+                        const float term = a.expert_out[(size_t)e * a.n + i] * w;
+                        sum[k] = sum[k] + term;
+                    }
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < SLOTS; ++k) {
+                const int i = base + (int)threadIdx.x + k * THREADS;
+                if (i < a.n) routed[i] = sum[k];
+            }
+        }
+    }
     const float *vec[2] = {a.dense, a.routed};
     float ss[2];
     serial_square_sums(vec, 2, a.n, sq, ss, shared, bad);
     const float inv_d = inverse_from_sum(ss[0], a.n, a.eps), inv_r = inverse_from_sum(ss[1], a.n, a.eps);
-    bad = bad || !finite(inv_d) || !finite(inv_r);
-    for (int i = threadIdx.x; i < a.n; i += THREADS) {
-        const float d = (a.dense[i] * inv_d) * a.wd[i], r = (a.routed[i] * inv_r) * a.wr[i];
+    bad |= nonfinite(inv_d) | nonfinite(inv_r);
+    each_element(a.n, [&](int i) {
+        const float wd = a.wd[i], wr = a.wr[i], res = a.residual[i], wf = a.wf[i];
+        const float d0 = a.dense[i] * inv_d, r0 = a.routed[i] * inv_r;
+        const float d = d0 * wd, r = r0 * wr;
         const float s = d + r;
-        bad = bad || !finite(a.residual[i]) || !finite(a.wd[i]) || !finite(a.wr[i]) || !finite(a.wf[i]);
-        bad = bad || !finite(a.dense[i] * inv_d) || !finite(a.routed[i] * inv_r) || !finite(d) || !finite(r) || !finite(s);
+        bad |= nonfinite(res) | nonfinite(wd) | nonfinite(wr) | nonfinite(wf) | nonfinite(d0) | nonfinite(r0) | nonfinite(d) | nonfinite(r) |
+               nonfinite(s);
         a.sum[i] = s;
-    }
-    __syncthreads();                                    // a.sum is read back by other threads below
-    const float *vec2[1] = {a.sum};
+    });
+    const float *vec2[1] = {a.sum};                     // a thread reads back the elements it wrote itself
     float ss_sum;
     serial_square_sums(vec2, 1, a.n, sq, &ss_sum, shared, bad);
     const float inv_f = inverse_from_sum(ss_sum, a.n, a.eps);
-    bad = bad || !finite(inv_f);
-    for (int i = threadIdx.x; i < a.n; i += THREADS) {
-        const float f = (a.sum[i] * inv_f) * a.wf[i];
+    bad |= nonfinite(inv_f);
+    each_element(a.n, [&](int i) {
+        const float f0 = a.sum[i] * inv_f;
+        const float f = f0 * a.wf[i];
         const float y = (a.residual[i] + f) * a.scalar;
-        bad = bad || !finite(a.sum[i] * inv_f) || !finite(f) || !finite(y);
-    }
-    if (__syncthreads_or(bad)) {
+        bad |= nonfinite(f0) | nonfinite(f) | nonfinite(y);
+    });
+    if (__syncthreads_or((int)bad)) {
         if (threadIdx.x == 0) *a.status = -1;
         return;
     }
-    for (int i = threadIdx.x; i < a.n; i += THREADS) {
+    each_element(a.n, [&](int i) {
         const float f = (a.sum[i] * inv_f) * a.wf[i];
         a.out[i] = (a.residual[i] + f) * a.scalar;
-    }
+    });
 }
 
-__global__ __launch_bounds__(THREADS) void finite_check_kernel(const float *x, size_t n, int *status) {
-    bool bad = false;
-    for (size_t i = (size_t)blockIdx.x * THREADS + threadIdx.x; i < n; i += (size_t)gridDim.x * THREADS)
-        bad = bad || !finite(x[i]);
-    if (__syncthreads_or(bad) && threadIdx.x == 0) *status = -1;      // every writer stores the same value
+constexpr int WIDE = 256;             // threads per workgroup of the grid-wide elementwise kernels
+
+__global__ __launch_bounds__(WIDE) void finite_check_kernel(const float *x, size_t n, int *status) {
+    unsigned bad = 0;
+    for (size_t i = (size_t)blockIdx.x * WIDE + threadIdx.x; i < n; i += (size_t)gridDim.x * WIDE) bad |= nonfinite(x[i]);
+    if (__syncthreads_or((int)bad) && threadIdx.x == 0) *status = -1;      // every writer stores the same value
 }
 
-__global__ __launch_bounds__(THREADS) void softcap_kernel(float *logits, size_t n, float cap, const int *status) {
+__global__ __launch_bounds__(WIDE) void softcap_kernel(float *logits, size_t n, float cap, const int *status) {
     if (*status != 0) return;
-    const size_t i = (size_t)blockIdx.x * THREADS + threadIdx.x;
+    const size_t i = (size_t)blockIdx.x * WIDE + threadIdx.x;
     if (i < n) logits[i] = cap * det_tanhf(logits[i] / cap);
 }
 
@@ -277,28 +341,34 @@ int norm_cell_launch(int kind, const float *x, const float *weight, const float 
 }
 
 int ffn_pre_launch(const float *residual, const float *w1, const float *w2, const float *router_scale, float *norm_a,
-                   float *norm_b, float *router_in, int n, float eps, int *status, hipStream_t stream) {
+                   float *norm_b, float *router_in, int n, float eps, int *status, const Q4Job *jobs, Q4Job *jobs_out,
+                   hipStream_t stream) {
     if (!residual || !w1 || !w2 || !router_scale || !norm_a || !norm_b || !router_in || !status || n < 1) return -1;
-    PreArgs a = {residual, w1, w2, router_scale, norm_a, norm_b, router_in, n, eps, status};
+    PreArgs a = {residual, w1, w2, router_scale, norm_a, norm_b, router_in, n, eps, status, {}, jobs_out};
+    if (jobs_out) { a.jobs[0] = jobs[0]; a.jobs[1] = jobs[1]; }
     ffn_pre_kernel<<<dim3(1), dim3(THREADS), 0, stream>>>(a);
     return launched() ? 0 : -1;
 }
 
 int combine_cell_launch(const float *residual, const float *dense, const float *routed, const float *wd, const float *wr,
                         const float *wf, float *sum_scratch, float *out, int n, float eps, float scalar, int *status,
-                        const int *other_status, hipStream_t stream) {
-    if (!residual || !dense || !routed || !wd || !wr || !wf || !sum_scratch || !out || !status || n < 1) return -1;
-    CombineArgs a = {residual, dense, routed, wd, wr, wf, sum_scratch, out, n, eps, scalar, status, other_status};
+                        const int *other_status, const float *expert_out, const float *weights, int topk,
+                        hipStream_t stream) {
+    if (!residual || !dense || !routed || !wd || !wr || !wf || !sum_scratch || !out || !status || n < 1 ||
+        (expert_out && (!weights || topk < 1)))
+        return -1;
+    CombineArgs a = {residual, dense, routed, wd, wr, wf, sum_scratch, out, n, eps, scalar, status, other_status,
+                     expert_out, weights, topk};
     combine_cell_kernel<<<dim3(1), dim3(THREADS), 0, stream>>>(a);
     return launched() ? 0 : -1;
 }
 
 int softcap_cell_launch(float *logits, size_t n, float cap, int *status, hipStream_t stream) {
     if (!logits || !status || n < 1 || !(cap > 0.0f) || !(cap < __builtin_inff())) return -1;
-    const size_t blocks = (n + THREADS - 1) / THREADS;
-    finite_check_kernel<<<dim3((unsigned)(blocks < 1024 ? blocks : 1024)), dim3(THREADS), 0, stream>>>(logits, n, status);
+    const size_t blocks = (n + WIDE - 1) / WIDE;
+    finite_check_kernel<<<dim3((unsigned)(blocks < 1024 ? blocks : 1024)), dim3(WIDE), 0, stream>>>(logits, n, status);
     if (!launched()) return -1;
-    softcap_kernel<<<dim3((unsigned)blocks), dim3(THREADS), 0, stream>>>(logits, n, cap, status);
+    softcap_kernel<<<dim3((unsigned)blocks), dim3(WIDE), 0, stream>>>(logits, n, cap, status);
     return launched() ? 0 : -1;
 }
 

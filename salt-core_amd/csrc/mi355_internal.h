@@ -190,11 +190,15 @@ int q8_launch(const Q8Launch &launch, hipStream_t stream);
 // input or a result is not finite.  kind: 0 rms norm (weight optional), 1 router input, 2 residual post-norm.
 int norm_cell_launch(int kind, const float *x, const float *weight, const float *residual, float *out, int n, float eps,
                      float root, int *status, hipStream_t stream);
+// Opens a feed-forward block: *status is written (0 or -1); two job records (optional) are copied to jobs_out for the
+// dense gate/up launch that follows.
 int ffn_pre_launch(const float *residual, const float *w1, const float *w2, const float *router_scale, float *norm_a,
-                   float *norm_b, float *router_in, int n, float eps, int *status, hipStream_t stream);
+                   float *norm_b, float *router_in, int n, float eps, int *status, const Q4Job *jobs, Q4Job *jobs_out,
+                   hipStream_t stream);
 int combine_cell_launch(const float *residual, const float *dense, const float *routed, const float *wd, const float *wr,
                         const float *wf, float *sum_scratch, float *out, int n, float eps, float scalar, int *status,
-                        const int *other_status, hipStream_t stream);
+                        const int *other_status, const float *expert_out, const float *weights, int topk,
+                        hipStream_t stream);
 int softcap_cell_launch(float *logits, size_t n, float cap, int *status, hipStream_t stream);
 int merge_status_launch(int *status, const int *other, hipStream_t stream);
 
@@ -226,6 +230,7 @@ void moe_workspace_carve(const MoeGeometry &g, void *base, MoeWorkspace *ws);
 int router_topk_launch(const float *logits, const float *per_expert_scale, int n_experts, int topk,
                        int sorted_by_id, int *selected, float *weights, int *status, hipStream_t stream);
 
+// out == nullptr leaves the ordered weighted reduction of expert_out to the caller
 int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_stride,
                            const float *logits, const float *per_expert_scale, const float *x,
                            int *selected, float *weights, float *expert_out, float *out,

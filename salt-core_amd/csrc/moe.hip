@@ -167,7 +167,7 @@ int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t exp
         m.status = ws.status; m.n_experts = g.n_experts; m.topk = g.topk; m.hidden = g.hidden; m.routed = g.routed;
         if (q4_moe_gate_up_launch(fused, stream) != 0) return -1;
         if (q4_moe_down_launch(fused, stream) != 0) return -1;
-        return moe_reduce_launch(eo, weights, g.topk, g.hidden, out, ws.status, stream);
+        return out ? moe_reduce_launch(eo, weights, g.topk, g.hidden, out, ws.status, stream) : 0;
     }
     JobEmit emit;
     emit.gate_up_jobs = ws.gate_up_jobs;
@@ -204,7 +204,7 @@ int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t exp
     down.code_scale = code_scale;
     if (q4_launch(down, 0, stream) != 0) return -1;
 
-    return moe_reduce_launch(eo, weights, g.topk, g.hidden, out, nullptr, stream);
+    return out ? moe_reduce_launch(eo, weights, g.topk, g.hidden, out, nullptr, stream) : 0;
 }
 
 }  // namespace mi355
