@@ -16,6 +16,7 @@ namespace {
 constexpr int THREADS = 1024;         // one workgroup per cell: sixteen waves keep enough loads in flight
 constexpr int SLOTS = 4;              // elements a thread handles per pass: i = base + tid + k * THREADS
 constexpr int SQ_CHUNK = SLOTS * THREADS;   // squares staged per pass of the serial adder
+constexpr int SQ_TAIL = 64;           // floats the adder may read (and drop) past the staged squares
 
 __device__ __forceinline__ double inverse_root64(float x) {
     const float seed = __uint_as_float(0x5f3759dfu - (__float_as_uint(x) >> 1));
@@ -79,9 +80,61 @@ __device__ __forceinline__ void each_element(int n, F f) {
     }
 }
 
+// acc + mine[0] + mine[1] + ... + mine[count - 1], left to right.  32 values per batch; the next batch is read from
+// LDS while the current one is added, unconditionally one batch ahead (what is read past the end is dropped, the
+// staging buffers have a tail for it).
+__device__ __forceinline__ float add_staged(const float *mine, int count, float acc) {
+    const int full = count & ~31, pairs = full & ~63;
+    float4 a[8], b[8];
+    auto fetch = [&](float4 (&dst)[8], int at) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) dst[k] = *(const float4 *)&mine[at + 4 * k];
+    };
+    auto add = [&](const float4 (&src)[8]) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            acc = acc + src[k].x;
+            acc = acc + src[k].y;
+            acc = acc + src[k].z;
+            acc = acc + src[k].w;
+        }
+    };
+    fetch(a, 0);
+    for (int i = 0; i < pairs; i += 64) {
+        fetch(b, i + 32);
+        add(a);
+        fetch(a, i + 64);
+        add(b);
+    }
+    if (full != pairs) add(a);
+    for (int i = full; i < count; ++i) acc = acc + mine[i];
+    return acc;
+}
+
+// The same sums for at most SQ_CHUNK elements that the threads already hold: val[v][k] is element tid + k * THREADS of
+// vector v.
+template <int V>
+__device__ __forceinline__ void chains_from_registers(const float (&val)[V][SLOTS], int n, float *sq, float *shared,
+                                                      float (&ss)[V]) {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int v = 0; v < V; ++v)
+#pragma unroll
+        for (int k = 0; k < SLOTS; ++k) {
+            const int i = tid + k * THREADS;
+            if (i < n) sq[v * SQ_CHUNK + i] = val[v][k] * val[v][k];
+        }
+    __syncthreads();
+    if (tid < V) shared[tid] = add_staged(sq + tid * SQ_CHUNK, n, 0.0f);
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < V; ++v) ss[v] = shared[v];
+    __syncthreads();
+}
+
 // Serial sums of squares of `vectors` (1 or 2) vectors of n floats: lane v of wave 0 adds vector v's squares left to
 // right.  Returns the sums in ss_out[] on every thread; `bad` collects non-finite elements.  sq is LDS scratch of
-// vectors * SQ_CHUNK floats, shared of at least `vectors` floats.
+// vectors * SQ_CHUNK + SQ_TAIL floats, shared of at least `vectors` floats.
 __device__ void serial_square_sums(const float *const *x, int vectors, int n, float *sq, float *ss_out, float *shared,
                                    unsigned &bad) {
     const int tid = threadIdx.x;
@@ -101,36 +154,7 @@ __device__ void serial_square_sums(const float *const *x, int vectors, int n, fl
             }
         }
         __syncthreads();
-        if (tid < vectors) {
-            // 32 squares per batch; the next batch is read from LDS while the current one is added
-            const float *mine = sq + tid * SQ_CHUNK;
-            const int full = count & ~31;
-            float4 a[8], b[8];
-            auto fetch = [&](float4 (&dst)[8], int at) {
-#pragma unroll
-                for (int k = 0; k < 8; ++k) dst[k] = *(const float4 *)&mine[at + 4 * k];
-            };
-            auto add = [&](const float4 (&src)[8]) {
-#pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    acc = acc + src[k].x;
-                    acc = acc + src[k].y;
-                    acc = acc + src[k].z;
-                    acc = acc + src[k].w;
-                }
-            };
-            if (full) fetch(a, 0);
-            for (int i = 0; i < full; i += 64) {
-                const bool second = i + 32 < full;
-                if (second) fetch(b, i + 32);
-                add(a);
-                if (second) {
-                    if (i + 64 < full) fetch(a, i + 64);
-                    add(b);
-                }
-            }
-            for (int i = full; i < count; ++i) acc = acc + mine[i];
-        }
+        if (tid < vectors) acc = add_staged(sq + tid * SQ_CHUNK, count, acc);
         __syncthreads();
     }
     if (tid < vectors) shared[tid] = acc;
@@ -156,7 +180,7 @@ struct NormArgs {
 };
 
 __global__ __launch_bounds__(THREADS) void norm_cell_kernel(NormArgs a) {
-    __shared__ __attribute__((aligned(16))) float sq[SQ_CHUNK];
+    __shared__ __attribute__((aligned(16))) float sq[SQ_CHUNK + SQ_TAIL];
     __shared__ float shared[4];
     if (*a.status != 0) return;
     unsigned bad = !(a.eps >= 0.0f) || nonfinite(a.eps);
@@ -200,8 +224,49 @@ struct PreArgs {
     Q4Job *jobs_out;
 };
 
+// n <= SQ_CHUNK: every input is requested once, up front, and lives in registers from then on
+__global__ __launch_bounds__(THREADS) void ffn_pre_small_kernel(PreArgs a) {
+    __shared__ __attribute__((aligned(16))) float sq[SQ_CHUNK + SQ_TAIL];
+    __shared__ float shared[4];
+    if (a.jobs_out && threadIdx.x < 2) a.jobs_out[threadIdx.x] = a.jobs[threadIdx.x];
+    unsigned bad = !(a.eps >= 0.0f) || nonfinite(a.eps);
+    float r[1][SLOTS], w1[SLOTS], w2[SLOTS], rs[SLOTS];
+#pragma unroll
+    for (int k = 0; k < SLOTS; ++k) {
+        const int i = (int)threadIdx.x + k * THREADS;
+        const bool live = i < a.n;
+        r[0][k] = live ? a.residual[i] : 0.0f;
+        w1[k] = live ? a.w1[i] : 0.0f;
+        w2[k] = live ? a.w2[i] : 0.0f;
+        rs[k] = live ? a.router_scale[i] : 0.0f;
+        bad |= nonfinite(r[0][k]) | nonfinite(w1[k]) | nonfinite(w2[k]) | nonfinite(rs[k]);
+    }
+    float ss[1];
+    chains_from_registers<1>(r, a.n, sq, shared, ss);
+    const float inv = inverse_from_sum(ss[0], a.n, a.eps);
+    bad |= nonfinite(inv);
+    const float root = 1.0f / det_sqrtf((float)a.n);
+    float na[SLOTS], nb[SLOTS], ri[SLOTS];
+#pragma unroll
+    for (int k = 0; k < SLOTS; ++k) {
+        const float y = r[0][k] * inv;
+        na[k] = y * w1[k];
+        nb[k] = y * w2[k];
+        ri[k] = (y * rs[k]) * root;
+        bad |= nonfinite(y) | nonfinite(na[k]) | nonfinite(nb[k]) | nonfinite(ri[k]);
+    }
+    const bool failed = __syncthreads_or((int)bad);
+    if (threadIdx.x == 0) *a.status = failed ? -1 : 0;
+    if (failed) return;
+#pragma unroll
+    for (int k = 0; k < SLOTS; ++k) {
+        const int i = (int)threadIdx.x + k * THREADS;
+        if (i < a.n) { a.norm_a[i] = na[k]; a.norm_b[i] = nb[k]; a.router_in[i] = ri[k]; }
+    }
+}
+
 __global__ __launch_bounds__(THREADS) void ffn_pre_kernel(PreArgs a) {
-    __shared__ __attribute__((aligned(16))) float sq[SQ_CHUNK];
+    __shared__ __attribute__((aligned(16))) float sq[SQ_CHUNK + SQ_TAIL];
     __shared__ float shared[4];
     if (a.jobs_out && threadIdx.x < 2) a.jobs_out[threadIdx.x] = a.jobs[threadIdx.x];
     unsigned bad = !(a.eps >= 0.0f) || nonfinite(a.eps);
@@ -241,8 +306,81 @@ struct CombineArgs {
     int topk;
 };
 
+// n <= SQ_CHUNK: one load phase, everything else in registers and LDS
+__global__ __launch_bounds__(THREADS) void combine_small_kernel(CombineArgs a) {
+    __shared__ __attribute__((aligned(16))) float sq[2 * SQ_CHUNK + SQ_TAIL];
+    __shared__ float shared[4];
+    if (*a.status != 0) return;
+    if (a.other && *a.other != 0) {
+        if (threadIdx.x == 0) *a.status = -1;
+        return;
+    }
+    unsigned bad = !(a.eps >= 0.0f) || nonfinite(a.eps) || nonfinite(a.scalar);
+    float dr[2][SLOTS], res[SLOTS], wd[SLOTS], wr[SLOTS], wf[SLOTS];
+#pragma unroll
+    for (int k = 0; k < SLOTS; ++k) {
+        const int i = (int)threadIdx.x + k * THREADS;
+        const bool live = i < a.n;
+        res[k] = live ? a.residual[i] : 0.0f;
+        wd[k] = live ? a.wd[i] : 0.0f;
+        wr[k] = live ? a.wr[i] : 0.0f;
+        wf[k] = live ? a.wf[i] : 0.0f;
+        dr[0][k] = live ? a.dense[i] : 0.0f;
+        dr[1][k] = live && !a.expert_out ? a.routed[i] : 0.0f;
+    }
+    if (a.expert_out)
+        for (int e = 0; e < a.topk; ++e) {
+            const float w = a.weights[e];
+#pragma unroll
+            for (int k = 0; k < SLOTS; ++k) {
+                const int i = (int)threadIdx.x + k * THREADS;
+                if (i < a.n) {
+                    const float term = a.expert_out[(size_t)e * a.n + i] * w;
+                    dr[1][k] = dr[1][k] + term;
+                }
+            }
+        }
+#pragma unroll
+    for (int k = 0; k < SLOTS; ++k)
+        bad |= nonfinite(res[k]) | nonfinite(wd[k]) | nonfinite(wr[k]) | nonfinite(wf[k]) | nonfinite(dr[0][k]) |
+               nonfinite(dr[1][k]);
+    float ss[2];
+    chains_from_registers<2>(dr, a.n, sq, shared, ss);
+    const float inv_d = inverse_from_sum(ss[0], a.n, a.eps), inv_r = inverse_from_sum(ss[1], a.n, a.eps);
+    bad |= nonfinite(inv_d) | nonfinite(inv_r);
+    float sum[1][SLOTS];
+#pragma unroll
+    for (int k = 0; k < SLOTS; ++k) {
+        const float d0 = dr[0][k] * inv_d, r0 = dr[1][k] * inv_r;
+        const float d = d0 * wd[k], r = r0 * wr[k];
+        sum[0][k] = d + r;
+        bad |= nonfinite(d0) | nonfinite(r0) | nonfinite(d) | nonfinite(r) | nonfinite(sum[0][k]);
+    }
+    float ss_sum[1];
+    chains_from_registers<1>(sum, a.n, sq, shared, ss_sum);
+    const float inv_f = inverse_from_sum(ss_sum[0], a.n, a.eps);
+    bad |= nonfinite(inv_f);
+    float y[SLOTS];
+#pragma unroll
+    for (int k = 0; k < SLOTS; ++k) {
+        const float f0 = sum[0][k] * inv_f;
+        const float f = f0 * wf[k];
+        y[k] = (res[k] + f) * a.scalar;
+        bad |= nonfinite(f0) | nonfinite(f) | nonfinite(y[k]);
+    }
+    if (__syncthreads_or((int)bad)) {
+        if (threadIdx.x == 0) *a.status = -1;
+        return;
+    }
+#pragma unroll
+    for (int k = 0; k < SLOTS; ++k) {
+        const int i = (int)threadIdx.x + k * THREADS;
+        if (i < a.n) a.out[i] = y[k];
+    }
+}
+
 __global__ __launch_bounds__(THREADS) void combine_cell_kernel(CombineArgs a) {
-    __shared__ __attribute__((aligned(16))) float sq[2 * SQ_CHUNK];
+    __shared__ __attribute__((aligned(16))) float sq[2 * SQ_CHUNK + SQ_TAIL];
     __shared__ float shared[4];
     if (*a.status != 0) return;
     if (a.other && *a.other != 0) {
@@ -346,7 +484,8 @@ int ffn_pre_launch(const float *residual, const float *w1, const float *w2, cons
     if (!residual || !w1 || !w2 || !router_scale || !norm_a || !norm_b || !router_in || !status || n < 1) return -1;
     PreArgs a = {residual, w1, w2, router_scale, norm_a, norm_b, router_in, n, eps, status, {}, jobs_out};
     if (jobs_out) { a.jobs[0] = jobs[0]; a.jobs[1] = jobs[1]; }
-    ffn_pre_kernel<<<dim3(1), dim3(THREADS), 0, stream>>>(a);
+    if (n <= SQ_CHUNK) ffn_pre_small_kernel<<<dim3(1), dim3(THREADS), 0, stream>>>(a);
+    else ffn_pre_kernel<<<dim3(1), dim3(THREADS), 0, stream>>>(a);
     return launched() ? 0 : -1;
 }
 
@@ -359,7 +498,8 @@ int combine_cell_launch(const float *residual, const float *dense, const float *
         return -1;
     CombineArgs a = {residual, dense, routed, wd, wr, wf, sum_scratch, out, n, eps, scalar, status, other_status,
                      expert_out, weights, topk};
-    combine_cell_kernel<<<dim3(1), dim3(THREADS), 0, stream>>>(a);
+    if (n <= SQ_CHUNK) combine_small_kernel<<<dim3(1), dim3(THREADS), 0, stream>>>(a);
+    else combine_cell_kernel<<<dim3(1), dim3(THREADS), 0, stream>>>(a);
     return launched() ? 0 : -1;
 }
 

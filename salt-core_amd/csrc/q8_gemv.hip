@@ -54,21 +54,26 @@ __global__ __launch_bounds__(64) void q8_rows_kernel(Q8Launch L) {
     if (lane < rows_here) L.y[(size_t)token * L.y_stride + row] = acc;
 }
 
-// Up to 4096 columns.  A workgroup owns 16 rows and one activation row.  The chain of a row is one addition per column and
-// nothing else can be taken off it, so the work is split by kind: three waves turn bytes into rounded products
+// Up to 4096 columns.  A workgroup owns 8 rows and one activation row.  The chain of a row is one addition per column
+// and nothing else can be taken off it, so the work is split by kind: three waves turn bytes into rounded products
 // ((float)byte * scale + bias) * x and leave them in LDS, and the fourth wave only adds them, in column order, one
-// lane per row.  Products travel in chunks of 192 columns through two LDS buffers; all bytes of the 16 rows are held in
-// registers from the start, so the memory latency is paid once.
-constexpr int CH_ROWS = 16;
-constexpr int CH_COLS = 192;                       // 16 rows x 12 segments of 16 bytes = 192 items, one per producer lane
-constexpr int CH_PITCH = CH_COLS + 4;              // floats; lanes 0..15 of a 16-byte read then touch distinct banks
+// lane per row, reading the next 32 products while it adds the current 32.  Products travel in chunks of 704 columns
+// through two LDS buffers (few chunks, so few barriers); all bytes of the 8 rows are held in registers from the
+// start, so the memory latency is paid once.
+constexpr int CH_ROWS = 8;
+constexpr int CH_COLS = 704;                       // 44 segments of 16 bytes per row
+constexpr int CH_SEGS = CH_COLS / 16;
+constexpr int CH_ITEMS = CH_ROWS * CH_SEGS;        // 352 (row, segment) items per chunk over 192 producer lanes
+constexpr int CH_PER_LANE = (CH_ITEMS + 191) / 192;
+constexpr int CH_PITCH = CH_COLS + 4;              // floats; the eight adding lanes then touch distinct banks
 constexpr int CH_MAX_COLS = 4096;
 constexpr int CH_MAX_CHUNKS = (CH_MAX_COLS + CH_COLS - 1) / CH_COLS;
 
 __global__ __launch_bounds__(256) void q8_chain_kernel(Q8Launch L) {
     __shared__ float x_lds[CH_MAX_COLS];
-    __shared__ float scale_lds[CH_ROWS][CH_MAX_COLS / 64], bias_lds[CH_ROWS][CH_MAX_COLS / 64];
-    __shared__ __attribute__((aligned(16))) float ring[2][CH_ROWS][CH_PITCH];
+    __shared__ uint16_t scale_lds[CH_ROWS][CH_MAX_COLS / 64], bias_lds[CH_ROWS][CH_MAX_COLS / 64];     // bf16 bits
+    // the adder reads up to 64 floats past the end of a chunk (and discards them): hence the tail
+    __shared__ __attribute__((aligned(16))) float ring[2 * CH_ROWS * CH_PITCH + 64];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int row0 = blockIdx.x * CH_ROWS;
@@ -77,25 +82,32 @@ __global__ __launch_bounds__(256) void q8_chain_kernel(Q8Launch L) {
     const int nchunk = (C + CH_COLS - 1) / CH_COLS;
     const float *x = L.x + (size_t)blockIdx.y * L.x_stride;
 
-    // producer item: one row, 16 consecutive columns of every chunk.  All of a lane's bytes are requested before
-    // anything else happens, unconditionally (a column past the row re-reads the row's last segment), so the loads
-    // are straight-line code and each use waits only for its own load.
+    // producer items: item = row * 44 + segment.  All of a lane's bytes are requested before anything else happens,
+    // unconditionally (a column past the row re-reads the row's last segment), so the loads are straight-line code
+    // and each use waits only for its own load.
     const int pid = tid >= 64 ? tid - 64 : 0;
-    const int prow = pid / 12, pseg = pid % 12;
-    const int prow_src = prow < rows_here ? prow : rows_here - 1;
-    const global_u128_ptr src = (global_u128_ptr)(uintptr_t)(L.vals + (size_t)(row0 + prow_src) * C);
-    u32x4 bytes[CH_MAX_CHUNKS];
+    int prow[CH_PER_LANE], pseg[CH_PER_LANE];
+    u32x4 bytes[CH_MAX_CHUNKS][CH_PER_LANE];
 #pragma unroll
-    for (int k = 0; k < CH_MAX_CHUNKS; ++k) {
-        const int col = k * CH_COLS + pseg * 16;
-        bytes[k] = src[(col < C ? col : C - 16) / 16];
+    for (int j = 0; j < CH_PER_LANE; ++j) {
+        const int item = pid + 192 * j < CH_ITEMS ? pid + 192 * j : CH_ITEMS - 1;
+        prow[j] = item / CH_SEGS;
+        pseg[j] = item % CH_SEGS;
     }
+#pragma unroll
+    for (int k = 0; k < CH_MAX_CHUNKS; ++k)
+#pragma unroll
+        for (int j = 0; j < CH_PER_LANE; ++j) {
+            const int row = prow[j] < rows_here ? prow[j] : rows_here - 1;
+            const int col = k * CH_COLS + pseg[j] * 16;
+            bytes[k][j] = *(global_u128_ptr)(uintptr_t)(L.vals + (size_t)(row0 + row) * C + (col < C ? col : C - 16));
+        }
     for (int c = tid; c < C; c += 256) x_lds[c] = x[c];
     for (int i = tid; i < CH_ROWS * groups; i += 256) {
         const int r = i / groups, g = i % groups;
         const size_t at = (size_t)(row0 + (r < rows_here ? r : rows_here - 1)) * groups + g;
-        scale_lds[r][g] = bf16_bits(((const uint16_t *)L.scales)[at]);
-        bias_lds[r][g] = L.biases ? bf16_bits(((const uint16_t *)L.biases)[at]) : 0.0f;
+        scale_lds[r][g] = ((const uint16_t *)L.scales)[at];
+        bias_lds[r][g] = L.biases ? ((const uint16_t *)L.biases)[at] : (uint16_t)0;
     }
     __syncthreads();
 
@@ -106,44 +118,54 @@ __global__ __launch_bounds__(256) void q8_chain_kernel(Q8Launch L) {
     for (int i = 0; i <= CH_MAX_CHUNKS; ++i) {
         if (i > nchunk) continue;                 // uniform over the workgroup
         if (wave != 0) {
-            const int col = i * CH_COLS + pseg * 16;
-            if (i < CH_MAX_CHUNKS && col < C) {
-                const u32x4 v = bytes[i < CH_MAX_CHUNKS ? i : 0];
-                const uint32_t word[4] = {v.x, v.y, v.z, v.w};
-                const float s = scale_lds[prow][col / 64], b = bias_lds[prow][col / 64];
-                float *out = &ring[i & 1][prow][pseg * 16];
 #pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    const float4 xv = *(const float4 *)&x_lds[col + 4 * p];
-                    const float xs[4] = {xv.x, xv.y, xv.z, xv.w};
-                    float prod[4];
+            for (int j = 0; j < CH_PER_LANE; ++j) {
+                const int col = i * CH_COLS + pseg[j] * 16;
+                if (i < CH_MAX_CHUNKS && pid + 192 * j < CH_ITEMS && col < C) {
+                    const u32x4 v = bytes[i < CH_MAX_CHUNKS ? i : 0][j];
+                    const uint32_t word[4] = {v.x, v.y, v.z, v.w};
+                    const float s = bf16_bits(scale_lds[prow[j]][col / 64]), b = bf16_bits(bias_lds[prow[j]][col / 64]);
+                    float *out = &ring[((i & 1) * CH_ROWS + prow[j]) * CH_PITCH + pseg[j] * 16];
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        float value = (float)((word[p] >> (8 * q)) & 0xffu) * s;
-                        value = value + b;
-                        prod[q] = value * xs[q];
+                    for (int p = 0; p < 4; ++p) {
+                        const float4 xv = *(const float4 *)&x_lds[col + 4 * p];
+                        const float xs[4] = {xv.x, xv.y, xv.z, xv.w};
+                        float prod[4];
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            float value = (float)((word[p] >> (8 * q)) & 0xffu) * s;
+                            value = value + b;
+                            prod[q] = value * xs[q];
+                        }
+                        *(float4 *)&out[4 * p] = make_float4(prod[0], prod[1], prod[2], prod[3]);
                     }
-                    *(float4 *)&out[4 * p] = make_float4(prod[0], prod[1], prod[2], prod[3]);
                 }
             }
-        } else if (i >= 1) {
+        } else if (i >= 1 && lane < CH_ROWS) {
             const int c0 = (i - 1) * CH_COLS;
-            const int units = (C - c0 < CH_COLS ? C - c0 : CH_COLS) / 64;
-            const float *in = &ring[(i - 1) & 1][crow][0];
-            auto add_units = [&](int count) {
+            const int count = C - c0 < CH_COLS ? C - c0 : CH_COLS;          // a multiple of 64
+            const float *in = &ring[(((i - 1) & 1) * CH_ROWS + crow) * CH_PITCH];
+            float4 a[8], b[8];
+            auto fetch = [&](float4 (&dst)[8], int at) {
 #pragma unroll
-                for (int j = 0; j < 16 * 3; ++j) {
-                    if (j >= 16 * count) break;
-                    const float4 p = *(const float4 *)&in[4 * j];
-                    acc = acc + p.x;
-                    acc = acc + p.y;
-                    acc = acc + p.z;
-                    acc = acc + p.w;
+                for (int k = 0; k < 8; ++k) dst[k] = *(const float4 *)&in[at + 4 * k];
+            };
+            auto add = [&](const float4 (&src)[8]) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    acc = acc + src[k].x;
+                    acc = acc + src[k].y;
+                    acc = acc + src[k].z;
+                    acc = acc + src[k].w;
                 }
             };
-            if (units == 3) add_units(3);
-            else if (units == 2) add_units(2);
-            else add_units(1);
+            fetch(a, 0);
+            for (int at = 0; at < count; at += 64) {        // the last fetch of a reads past the chunk and is dropped
+                fetch(b, at + 32);
+                add(a);
+                fetch(a, at + 64);
+                add(b);
+            }
         }
         __syncthreads();
     }
