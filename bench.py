@@ -176,6 +176,15 @@ def cpu_other_configs(synth, pool, cores: int, budget_s: float = 3.0):
                                                         None, cores), T, budget_s)
     out["moe_prefill_tokens_per_s"] = {"value": round(tok_per_s, 1), "kind": "port", "cores": cores,
                                        "sample": f"{reps} passes over {T} tokens"}
+    # the whole feed-forward block of a layer (port of feed_forward; matvecs and experts on `cores` threads)
+    from oracle_lib import ffn_layer_struct
+    weights = synth.ffn_layer(H, 2112, F, E, K, 70, pool=pool)
+    layer = ffn_layer_struct(weights)
+    residual = (synth.activations(H, 1, 71)[0] * 3).astype(np.float32)
+    blocks_per_s, reps = rate(lambda: oracle.orc_ffn_block(C.byref(layer), ptr(residual), ptr(y), None, None, cores), 1,
+                              budget_s)
+    out["ffn_block_us"] = {"value": round(1e6 / blocks_per_s, 1), "kind": "port", "cores": cores,
+                           "sample": f"{reps} blocks"}
     # NVFP4 8192 x 8192, batch 1: the reference's own function (single thread)
     R = Cc = 8192
     packed, fscales = synth.nvfp4_tensor(R, Cc, 40)
@@ -263,6 +272,21 @@ def main():
         extra["moe_decode_step_gbps"] = round(step_bytes / (ms_moe * 1e-3) / 1e9, 1)
         extra["moe_decode_step_hbm_frac"] = round(step_bytes / (ms_moe * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
         del layers
+        # the whole feed-forward block of a decoder layer for one token: pre-norms, dense FFN (2112 wide), router input,
+        # 8-bit gate, top-8 of 128, routed experts, parallel combine -- bit-exact, device-resident
+        block = gpu.FfnBlock(synth.ffn_layer(H, 2112, F, E, K, 70, pool=pool))
+        block.residual.upload((synth.activations(H, 1, 71)[0] * 3).astype(np.float32))
+
+        def ffn_step(st):
+            if block.enqueue(st) != 0:
+                raise RuntimeError(lib.salt_mi355_last_error().decode())
+
+        ms_ffn = timed(lib, stream, events, ffn_step, 5, 100)
+        if int(block.status.to_host(np.int32)[0]) != 0:
+            raise RuntimeError("the feed-forward block rejected its input")
+        extra["ffn_block_us"] = round(ms_ffn * 1e3, 2)
+        extra["ffn_block_layer_tokens_per_s"] = round(1e3 / ms_ffn, 1)
+        del block
         # NVFP4 8192 x 8192, batch 1, reference semantics (activation Q/DQ inside the rows' launch), 16 instances
         R = Cc = 8192
         packed, fscales = synth.nvfp4_tensor(R, Cc, 40)

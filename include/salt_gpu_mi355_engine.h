@@ -305,21 +305,52 @@ typedef struct SaltGpuResidencyBackendOps {
 } SaltGpuResidencyBackendOps;
 const SaltGpuResidencyBackendOps *salt_gpu_residency_backend_ops(void);   /* reference gpu_residency.h:149 */
 
-/* ---- outside the quantized decode path: answered like the null backend ---- */
+/* ---- 8-bit affine router gates and the bf16 head --------------------------- */
 
-struct SaltGpuExactCell;
-struct SaltGpuDispatch;
-struct SaltTextGpuProgramOps;
+/* 8-bit tensors are registered with salt_gpu_weight_resource_slot(bits = 8).  One left-to-right chain per row
+ * (reference src/kernels.c:343-370): bit-exact. */
 int salt_gpu_q8_matvec(const uint32_t *vals, const uint16_t *scales, const uint16_t *biases, int R, int C,
                        const float *x, float *y);                               /* reference gpu.h:37 */
 int salt_gpu_q8_batch(const uint32_t *const *vals, const uint16_t *const *scales, const uint16_t *const *biases,
                       const float *const *xs, float *const *ys, const void *const *ids, const int *Rj, int C,
                       int njobs);                                                /* reference gpu.h:89 */
+/* C must be a multiple of 8 and the key registered (reference gpu_hip.cpp:4414-4443, 4591-4622); eight chains per row
+ * in the order of src/kernels.c:139-174: bit-exact. */
 int salt_gpu_bf16_resource_slot(uint32_t kind, uint32_t resource_id, const void *key, const uint16_t *weights,
                                 int R, int C);                                   /* reference gpu.h:60 */
-int salt_gpu_bf16_matvec(const void *key, int R, int C, const float *input, float *output);
+int salt_gpu_bf16_matvec(const void *key, int R, int C, const float *input, float *output);   /* reference gpu.h:63 */
+
+/* ---- fp32 cells over shared buffers ----------------------------------------- */
+
+typedef enum SaltGpuExactCellKind {               /* reference gpu.h:211-218 */
+    SALT_GPU_EXACT_RMSNORM = 1,
+    SALT_GPU_EXACT_TOPK = 2,
+    SALT_GPU_EXACT_RESIDUAL_POSTNORM = 3,
+    SALT_GPU_EXACT_PARALLEL_COMBINE = 4,
+    SALT_GPU_EXACT_SOFTCAP = 5,
+    SALT_GPU_EXACT_ROUTER_INPUT = 6
+} SaltGpuExactCellKind;
+
+typedef struct SaltGpuExactCell {                 /* reference gpu.h:224-232 */
+    SaltGpuExactCellKind kind;
+    SaltGpuSharedBuffer *views[8];   /* per kind as in reference gpu_hip.cpp:5299-5400 */
+    size_t offsets[8];               /* element offsets (floats; ints for the selection of TOPK) */
+    uint32_t n;
+    uint32_t aux;
+    float eps;
+    float scalar;
+} SaltGpuExactCell;
+
+/* The cells run in order on the device; one completion for the sequence.  -1 when a cell meets a non-finite input or
+ * result (that cell and every later one then publish nothing) or a view lies outside its buffer. */
+int salt_gpu_exact_cells(const SaltGpuExactCell *cells, int count);              /* reference gpu.h:234 */
+
+/* ---- outside the quantized decode path: answered like the null backend ---- */
+
+struct SaltGpuDispatch;
+struct SaltTextGpuProgramOps;
+/* left to the CPU, as in the reference's ROCm backend (gpu_hip.cpp:4624-4628) */
 int salt_gpu_bf16_matvec_batch(const void *key, int R, int C, int B, const float *inputs, float *outputs);
-int salt_gpu_exact_cells(const struct SaltGpuExactCell *cells, int count);       /* reference gpu.h:234 */
 const struct SaltGpuDispatch *salt_dispatch_get(void);                           /* reference gpu.h:163 */
 const struct SaltTextGpuProgramOps *salt_gpu_tensor_program_ops(void);           /* reference gpu.h:209 */
 int salt_gpu_resident_trunk_map(const void *base, size_t nbytes);                /* reference gpu.h:180 */

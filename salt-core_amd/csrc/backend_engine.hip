@@ -1331,6 +1331,74 @@ int salt_gpu_bf16_matvec(const void *key, int R, int C, const float *input, floa
     return finish_call(copies);
 }
 
+// ================================================================ fp32 cells over shared buffers
+
+int salt_gpu_exact_cells(const SaltGpuExactCell *cells, int count) {
+    if (ready_or_fail("exact_cells") != 0) return -1;
+    if (!cells || count < 1 || count > 4096) { set_error("exact_cells: bad arguments"); return -1; }
+    std::vector<SaltMi355Cell> table((size_t)count);
+    for (int c = 0; c < count; ++c) {
+        const SaltGpuExactCell &cell = cells[c];
+        size_t elements[8] = {0};
+        int views = 0;
+        if (cell.n == 0) { set_error("exact_cells: cell %d is empty", c); return -1; }
+        switch (cell.kind) {
+        case SALT_GPU_EXACT_RMSNORM:
+            if (cell.aux > 1u) { set_error("exact_cells: rmsnorm aux must be 0 or 1"); return -1; }
+            views = 3; elements[0] = cell.n; elements[1] = cell.aux ? cell.n : 1u; elements[2] = cell.n;
+            break;
+        case SALT_GPU_EXACT_TOPK:
+            if (cell.aux == 0 || cell.aux > cell.n) { set_error("exact_cells: topk aux must be in [1, n]"); return -1; }
+            views = 4; elements[0] = elements[1] = cell.n; elements[2] = elements[3] = cell.aux;
+            break;
+        case SALT_GPU_EXACT_RESIDUAL_POSTNORM:
+            views = 4; for (int k = 0; k < 4; ++k) elements[k] = cell.n;
+            break;
+        case SALT_GPU_EXACT_PARALLEL_COMBINE:
+            views = 8; for (int k = 0; k < 8; ++k) elements[k] = k == 6 ? (size_t)cell.n * 2u : cell.n;
+            break;
+        case SALT_GPU_EXACT_SOFTCAP:
+            if (!(cell.scalar > 0.0f) || !isfinite(cell.scalar)) { set_error("exact_cells: softcap needs a positive cap"); return -1; }
+            views = 1; elements[0] = cell.n;
+            break;
+        case SALT_GPU_EXACT_ROUTER_INPUT:
+            views = 3; for (int k = 0; k < 3; ++k) elements[k] = cell.n;
+            break;
+        default:
+            set_error("exact_cells: cell %d has unknown kind %d", c, (int)cell.kind);
+            return -1;
+        }
+        SaltMi355Cell &out = table[(size_t)c];
+        memset(&out, 0, sizeof out);
+        out.kind = (int)cell.kind; out.n = cell.n; out.aux = cell.aux; out.eps = cell.eps; out.scalar = cell.scalar;
+        for (int k = 0; k < views; ++k) {
+            const SaltGpuSharedBuffer *b = cell.views[k];
+            // element offsets and capacities count floats (ints for the selection of TOPK have the same size)
+            const size_t capacity = b && b->contents ? b->nbytes / sizeof(float) : 0;
+            if (!b || !b->contents || cell.offsets[k] > capacity || elements[k] > capacity - cell.offsets[k]) {
+                set_error("exact_cells: cell %d view %d lies outside its buffer", c, k);
+                return -1;
+            }
+            uint8_t *dev = (uint8_t *)shared_device_view(b->contents, b->nbytes);
+            if (!dev) { set_error("exact_cells: cell %d view %d is not a shared buffer of this backend", c, k); return -1; }
+            out.views[k] = dev + cell.offsets[k] * sizeof(float);
+        }
+    }
+    if (staging_reserve(256, 256) != 0) return -1;
+    int *status_dev = (int *)device_take(256), *status_pin = (int *)pinned_take(256);
+    *status_pin = -1;
+    if (clear_words_launch(status_dev, 2, g_state.stream) != 0 ||
+        salt_mi355_cells_dev(table.data(), count, status_dev, g_state.stream) != 0 ||
+        hip_ok(hipMemcpyAsync(status_pin, status_dev, sizeof(int), hipMemcpyDeviceToHost, g_state.stream),
+               "exact_cells status") != 0) {
+        (void)salt_gpu_sync();
+        return -1;
+    }
+    if (salt_gpu_sync() != 0) return -1;          // one status-bearing completion for the whole sequence
+    if (*status_pin != 0) { set_error("exact_cells: a cell met a non-finite input or result"); return -1; }
+    return 0;
+}
+
 // ================================================================ residency operations
 
 static int res_create(void *, const SaltGpuResidencyPlan *plan) {
@@ -1473,7 +1541,6 @@ const SaltGpuResidencyBackendOps *salt_gpu_residency_backend_ops(void) { return 
 // The ROCm backend of the reference leaves the batched bf16 matvec to the CPU (src/gpu_hip.cpp:4624-4628); its CUDA
 // counterpart computes a different, single-chain order for the vision tower.
 int salt_gpu_bf16_matvec_batch(const void *, int, int, int, const float *, float *) { return -1; }
-int salt_gpu_exact_cells(const struct SaltGpuExactCell *, int) { return -1; }
 const struct SaltGpuDispatch *salt_dispatch_get(void) { return nullptr; }
 const struct SaltTextGpuProgramOps *salt_gpu_tensor_program_ops(void) { return nullptr; }
 int salt_gpu_resident_trunk_map(const void *, size_t) { return -1; }

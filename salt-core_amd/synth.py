@@ -109,9 +109,9 @@ def q8_tensor(R: int, C: int, seed: int):
     return vals, scales, biases
 
 
-def ffn_layer(hidden: int, dense: int, routed: int, n_experts: int, topk: int, seed: int) -> dict:
+def ffn_layer(hidden: int, dense: int, routed: int, n_experts: int, topk: int, seed: int, pool=None) -> dict:
     """Weights of the feed-forward half of one decoder layer: norm weights, dense gate/up/down (affine Q4), the 8-bit
-    router gate, router and per-expert scales, the expert pool."""
+    router gate, router and per-expert scales, the expert pool (generated unless one is passed in)."""
     g = rng(seed)
     norm = lambda: (1.0 + 0.1 * g.standard_normal(hidden)).astype(np.float32)
     return {
@@ -123,7 +123,7 @@ def ffn_layer(hidden: int, dense: int, routed: int, n_experts: int, topk: int, s
         "dense_gate": q4_tensor(dense, hidden, seed * 7 + 1), "dense_up": q4_tensor(dense, hidden, seed * 7 + 2),
         "dense_down": q4_tensor(hidden, dense, seed * 7 + 3),
         "router": q8_tensor(n_experts, hidden, seed * 7 + 4),
-        "pool": expert_pool(n_experts, hidden, routed, seed * 7 + 5),
+        "pool": pool if pool is not None else expert_pool(n_experts, hidden, routed, seed * 7 + 5),
     }
 
 

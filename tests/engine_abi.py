@@ -72,6 +72,11 @@ class ResidencyOps(C.Structure):
                 ("permanent_publish", C.CFUNCTYPE(i32, vp))]
 
 
+class ExactCell(C.Structure):
+    _fields_ = [("kind", C.c_int), ("views", C.POINTER(SharedBuffer) * 8), ("offsets", C.c_size_t * 8), ("n", u32),
+                ("aux", u32), ("eps", C.c_float), ("scalar", C.c_float)]
+
+
 def bind(lib):
     """Sets argument and result types of the engine entry points used by tests."""
     def sig(name, res, *args):
@@ -125,6 +130,7 @@ def bind(lib):
     sig("salt_gpu_bf16_resource_slot", i32, u32, u32, vp, vp, i32, i32)
     sig("salt_gpu_bf16_matvec", i32, vp, i32, i32, vp, vp)
     sig("salt_gpu_bf16_matvec_batch", i32, vp, i32, i32, i32, vp, vp)
+    sig("salt_gpu_exact_cells", i32, C.POINTER(ExactCell), i32)
     sig("salt_dispatch_get", vp)
     sig("salt_gpu_tensor_program_ops", vp)
     sig("salt_gpu_resident_trunk_map", i32, vp, sz)

@@ -503,6 +503,75 @@ def test_router_gate_and_head_through_the_engine(eng, oracle, pkg):
     assert eng.salt_gpu_bf16_matvec(hw, HR, Cc, ptr(xs[0]), ptr(logits)) == -1
 
 
+def test_exact_cells_over_a_shared_buffer(eng, oracle, pkg):
+    """The block's fp32 cells the way the engine submits them: views into one startup-owned shared buffer, element
+    offsets, one completion for the sequence (reference gemma4_text.c:6704-6822)."""
+    n, E, K = 2816, 128, 8
+    f32 = np.float32
+    buf = abi.SharedBuffer()
+    total = 16 * n
+    assert eng.salt_gpu_shared_buffer_alloc(C.byref(buf), total * 4) == 0
+    arr = np.ctypeslib.as_array(C.cast(buf.contents, C.POINTER(C.c_float)), shape=(total,))
+    g = synth.rng(91)
+    names = ["x", "w", "w2", "w3", "res", "dense", "routed", "out", "out2", "out3", "scratch", "scratch_hi", "logits",
+             "scale", "sel", "wt"]
+    off = {name: k * n for k, name in enumerate(names)}
+    view = lambda name, count=n: arr[off[name]:off[name] + count]
+    for name, spread in [("x", 3), ("w", 1), ("w2", 1), ("w3", 1), ("res", 2), ("dense", 5), ("routed", 0.01)]:
+        view(name)[:] = (g.standard_normal(n) * spread).astype(f32)
+    view("logits", E)[:] = synth.router_logits(E, 5)
+    view("scale", E)[:] = g.uniform(0.5, 2.0, E).astype(f32)
+    eps = f32(1e-6)
+
+    def cell(kind, views, count, aux=0, scalar=0.0):
+        c = abi.ExactCell()
+        c.kind, c.n, c.aux, c.eps, c.scalar = kind, count, aux, eps, scalar
+        for k, name in enumerate(views):
+            c.views[k] = C.pointer(buf)
+            c.offsets[k] = off[name]
+        return c
+
+    root = float(f32(1.0) / f32(oracle.orc_sqrtf(f32(n))))
+    cells = (abi.ExactCell * 5)(
+        cell(1, ["x", "w", "out"], n, aux=1),
+        cell(6, ["x", "w2", "out2"], n, scalar=root),
+        cell(2, ["logits", "scale", "sel", "wt"], E, aux=K),
+        cell(4, ["res", "dense", "routed", "w", "w2", "w3", "scratch", "out3"], n, scalar=0.37),
+        cell(5, ["logits"], E, scalar=30.0))
+    logits = view("logits", E).copy()
+    assert eng.salt_gpu_exact_cells(cells, 5) == 0, err(pkg)
+    want = np.zeros(n, f32)
+    assert oracle.orc_rmsnorm(ptr(want), ptr(view("x").copy()), ptr(view("w").copy()), n, eps, 1) == 0
+    assert np.array_equal(bits(view("out")), bits(want))
+    assert oracle.orc_router_input(ptr(want), ptr(view("x").copy()), ptr(view("w2").copy()), n, eps) == 0
+    assert np.array_equal(bits(view("out2")), bits(want))
+    sel = np.zeros(K, np.int32); wt = np.zeros(K, f32)
+    assert oracle.orc_router_topk(ptr(logits), ptr(view("scale", E).copy()), E, K, ptr(sel), ptr(wt)) == 0
+    oracle.orc_sort_selection(ptr(sel), ptr(wt), K)
+    assert np.array_equal(view("sel", K).view(np.int32), sel) and np.array_equal(bits(view("wt", K)), bits(wt))
+    assert oracle.orc_parallel_ffn_combine(ptr(want), ptr(view("res").copy()), ptr(view("dense").copy()),
+                                           ptr(view("routed").copy()), ptr(view("w").copy()), ptr(view("w2").copy()),
+                                           ptr(view("w3").copy()), f32(0.37), n, eps) == 0
+    assert np.array_equal(bits(view("out3")), bits(want))
+    capped = logits.copy()
+    assert oracle.orc_softcap(ptr(capped), E, f32(30.0)) == 0 and np.array_equal(bits(view("logits", E)), bits(capped))
+    # a non-finite element fails the call; a view past the buffer, an unknown kind and a foreign buffer are refused
+    view("dense")[17] = np.inf
+    before = view("out3").copy()
+    assert eng.salt_gpu_exact_cells(cells, 4) == -1 and np.array_equal(bits(view("out3")), bits(before))
+    view("dense")[17] = 1.0
+    bad = cell(1, ["x", "w", "out"], n, aux=1); bad.offsets[2] = total - n + 1
+    assert eng.salt_gpu_exact_cells(C.byref(bad), 1) == -1
+    bad = cell(9, ["x", "w", "out"], n)
+    assert eng.salt_gpu_exact_cells(C.byref(bad), 1) == -1
+    host = np.zeros(n, f32)
+    foreign = abi.SharedBuffer(host.ctypes.data, host.nbytes, host.ctypes.data)
+    bad = cell(1, ["x", "w", "out"], n, aux=1); bad.views[0] = C.pointer(foreign); bad.offsets[0] = 0
+    assert eng.salt_gpu_exact_cells(C.byref(bad), 1) == -1
+    assert eng.salt_gpu_exact_cells(cells, 0) == -1
+    assert eng.salt_gpu_shared_buffer_free(C.byref(buf)) == 0
+
+
 def test_off_path_entry_points_answer_like_the_null_backend(eng):
     z = np.zeros(64, np.float32)
     assert eng.salt_gpu_resident_trunk_map(ptr(z), 256) == -1 and eng.salt_gpu_resident_pool_map(ptr(z), 256) == -1
