@@ -59,7 +59,8 @@ class Events:
 class Q4Sweep:
     """The three decode shapes, G instances each, one multi-job launch per shape."""
 
-    def __init__(self, gpu, synth, tokens: int):
+    def __init__(self, gpu, synth, tokens: int, distinct: int = 0):
+        """distinct > 0: the same number of jobs, but only that many weight instances in memory (cache-warm)."""
         self.gpu, self.lib, self.tokens = gpu, gpu.load(), tokens
         self.launches, self.keep = [], []
         self.bytes_per_step = 0
@@ -67,8 +68,9 @@ class Q4Sweep:
             vals, scales, biases = synth.q4_tensor(R, Cc, 100 + seed)
             per = vals.nbytes + scales.nbytes + biases.nbytes
             G = max(2, int(INSTANCE_BYTES // per))
-            weights = gpu.DeviceBuffer(per * G)
-            for g in range(G):
+            copies = min(G, distinct) if distinct > 0 else G
+            weights = gpu.DeviceBuffer(per * copies)
+            for g in range(copies):
                 weights.upload(vals, g * per)
                 weights.upload(scales, g * per + vals.nbytes)
                 weights.upload(biases, g * per + vals.nbytes + scales.nbytes)
@@ -76,8 +78,9 @@ class Q4Sweep:
             ys = gpu.DeviceBuffer(G * tokens * R * 4)
             jobs = (gpu.Q4Job * G)()
             for g in range(G):
-                jobs[g] = gpu.Q4Job(weights.at(g * per), weights.at(g * per + vals.nbytes),
-                                    weights.at(g * per + vals.nbytes + scales.nbytes), xs.ptr,
+                at = (g % copies) * per
+                jobs[g] = gpu.Q4Job(weights.at(at), weights.at(at + vals.nbytes),
+                                    weights.at(at + vals.nbytes + scales.nbytes), xs.ptr,
                                     ys.at(g * tokens * R * 4), R)
             self.keep += [weights, xs, ys]
             self.launches.append((jobs, G, Cc))
@@ -133,7 +136,25 @@ def cpu_baseline(synth, budget_s: float = 12.0):
     elapsed = time.perf_counter() - t0
     nbytes = sum(synth.q4_bytes(R, Cc, 1) for R, Cc in SWEEP)
     threads = int(os.environ["SALT_ATTN_THREADS"]) if ref is not None else cores
+    # one thread: the reference's SIMD kernel without its row split (its expert-scope switch), else the scalar port
+    if ref is not None:
+        ref.salt_kernels_set_in_expert(1)
+    t0 = time.perf_counter()
+    single_reps = 0
+    while time.perf_counter() - t0 < 2.0:
+        for R, Cc, vals, scales, biases, x, y in cases:
+            if ref is not None:
+                ref.salt_q4_matvec(ptr(vals), ptr(scales), ptr(biases), R, Cc, ptr(x), ptr(y))
+            else:
+                oracle.orc_q4_matvec_threads(ptr(vals), ptr(scales), ptr(biases), R, Cc, ptr(x), ptr(y), 1)
+        single_reps += 1
+    single = nbytes * single_reps / (time.perf_counter() - t0) / 1e9
+    if ref is not None:
+        ref.salt_kernels_set_in_expert(0)
     return {
+        "single_thread": {"value": round(single, 3), "unit": "GB/s", "cores": 1,
+                          "kind": "reference" if ref is not None else "port",
+                          "sample": f"{single_reps} passes of the same sweep"},
         "value": round(nbytes * reps / elapsed / 1e9, 3), "unit": "GB/s", "cores": threads,
         "kind": "reference" if ref is not None else "port",
         "sample": f"{reps} passes of the 3-shape sweep, one weight instance per shape, batch 1, "
@@ -251,6 +272,12 @@ def main():
         ms4 = timed(lib, stream, events, s4.step, 2, max(5, args.steps // 5))
         extra["q4_sweep_batch4_gbps"] = round(s4.bytes_per_step / (ms4 * 1e-3) / 1e9, 1)
         del s4
+        # the same batch-1 launches with every job reading one of two weight instances per shape (87 MB in all):
+        # served by the 256 MB last-level cache instead of HBM
+        warm = Q4Sweep(gpu, synth, tokens=1, distinct=2)
+        ms_w = timed(lib, stream, events, warm.step, 5, max(20, args.steps))
+        extra["q4_sweep_cache_warm_gbps"] = round(warm.bytes_per_step / (ms_w * 1e-3) / 1e9, 1)
+        del warm
         # MoE decode layer-step, E = 128 top-8, d_model 2816, d_ff 704; fresh logits per layer instance
         E, K, H, F = 128, 8, 2816, 704
         pool = synth.expert_pool(E, H, F, 7)
