@@ -262,6 +262,7 @@ int salt_mi355_q4_jobs_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tok
         Q4Launch launch;
         memset(&launch, 0, sizeof launch);
         launch.total_tiles = q4_assign_tiles(table.data(), njobs);
+        launch.tiles_per_job = q4_uniform_tiles(table.data(), njobs);
         launch.njobs = njobs;
         launch.cols = C;
         launch.tokens = group;

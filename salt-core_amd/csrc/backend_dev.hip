@@ -392,6 +392,7 @@ int salt_mi355_ffn_block_dev(const SaltMi355FfnLayer *layer, const float *residu
     Q4Launch gate_up;
     memset(&gate_up, 0, sizeof gate_up);
     gate_up.total_tiles = q4_assign_tiles(dense, 2);
+    gate_up.tiles_per_job = q4_uniform_tiles(dense, 2);
     gate_up.table = ws.dense_jobs; gate_up.njobs = 2; gate_up.cols = L.hidden; gate_up.tokens = 1;
     gate_up.code_scale = g_state.code_scale; gate_up.fused = g_state.q4_fused;
     const bool tileable = q4_job_is_tileable(dense[0], L.hidden) && q4_job_is_tileable(dense[1], L.hidden);

@@ -50,6 +50,7 @@ struct Q4Launch {
     int tokens;               // 1..4 activation rows per job
     int total_tiles;
     float code_scale;         // 1 / (value the fp8 converter gives byte 1)
+    int tiles_per_job;        // > 0 when every job of the table has this many tiles (tile -> job by division), else 0
     int fused;                // 0: separately rounded multiply and add (bit-exact); 1: fma accumulate
     MoeFuse moe;              // only read by q4_moe_gate_up_launch / q4_moe_down_launch
 };
@@ -65,6 +66,8 @@ bool q4_job_is_tileable(const Q4Job &job, int cols);
 
 // fills table[i].tile0 and returns the launch's tile count
 int q4_assign_tiles(Q4Job *table, int njobs);
+// the common tile count of the jobs, or 0 when they differ
+int q4_uniform_tiles(const Q4Job *table, int njobs);
 
 // ---------------------------------------------------------------- affine Q4 on MFMA (tolerance class)
 

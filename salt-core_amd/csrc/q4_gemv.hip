@@ -68,9 +68,13 @@ __device__ __forceinline__ Q4Job find_job(const Q4Launch &L, int tile) {
     if (L.table == nullptr) return L.one;
     const uniform_u64_ptr words = (uniform_u64_ptr)(uintptr_t)L.table;     // 7 words per record
     int lo = 0, hi = L.njobs - 1;
-    while (lo < hi) {                      // last job whose tile0 <= tile
-        const int mid = (lo + hi + 1) >> 1;
-        if ((int)(words[7 * mid + 5] >> 32) <= tile) lo = mid; else hi = mid - 1;
+    if (L.tiles_per_job > 0) {             // every job has the same number of tiles: no search
+        lo = tile / L.tiles_per_job;
+    } else {
+        while (lo < hi) {                  // last job whose tile0 <= tile
+            const int mid = (lo + hi + 1) >> 1;
+            if ((int)(words[7 * mid + 5] >> 32) <= tile) lo = mid; else hi = mid - 1;
+        }
     }
     const uniform_u64_ptr rec = words + 7 * lo;
     Q4Job job;
@@ -591,6 +595,13 @@ int q4_assign_tiles(Q4Job *table, int njobs) {
         tiles += (table[i].rows + TILE_ROWS - 1) / TILE_ROWS;
     }
     return tiles;
+}
+
+int q4_uniform_tiles(const Q4Job *table, int njobs) {
+    const int first = (table[0].rows + TILE_ROWS - 1) / TILE_ROWS;
+    for (int i = 1; i < njobs; ++i)
+        if ((table[i].rows + TILE_ROWS - 1) / TILE_ROWS != first) return 0;
+    return first;
 }
 
 int q4_moe_gate_up_launch(const Q4Launch &launch, hipStream_t stream) {
