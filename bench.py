@@ -313,6 +313,14 @@ def main():
             raise RuntimeError("the feed-forward block rejected its input")
         extra["ffn_block_us"] = round(ms_ffn * 1e3, 2)
         extra["ffn_block_layer_tokens_per_s"] = round(1e3 / ms_ffn, 1)
+        # the same block captured once and replayed as a HIP graph
+        if lib.salt_mi355_graph_begin(stream) == 0:
+            ffn_step(stream)
+            graph = lib.salt_mi355_graph_end(stream)
+            if graph:
+                ms_g = timed(lib, stream, events, lambda st: lib.salt_mi355_graph_launch(graph, st), 5, 100)
+                extra["ffn_block_graph_us"] = round(ms_g * 1e3, 2)
+                lib.salt_mi355_graph_destroy(graph)
         del block
         # NVFP4 8192 x 8192, batch 1, reference semantics (activation Q/DQ inside the rows' launch), 16 instances
         R = Cc = 8192

@@ -65,6 +65,16 @@ int salt_mi355_event_destroy(void *event);
 int salt_mi355_event_record(void *event, void *stream);
 /* Waits for `stop`, then returns the milliseconds between the two events. */
 int salt_mi355_event_elapsed_ms(void *start, void *stop, float *ms);
+/* Stream capture for callers that replay a fixed sequence of the device-resident
+ * entry points as one HIP graph.  Capturable: every *_dev entry point that takes
+ * a status word and neither uploads a job table nor waits (the MoE decode step,
+ * the feed-forward block, the cells, single-matrix matvecs).  begin starts a
+ * capture on `stream`; end finishes it and returns an executable graph (NULL on
+ * failure); launch replays it on `stream`. */
+int salt_mi355_graph_begin(void *stream);
+void *salt_mi355_graph_end(void *stream);
+int salt_mi355_graph_launch(void *graph_exec, void *stream);
+int salt_mi355_graph_destroy(void *graph_exec);
 
 /* ---- affine Q4 ("mlx4") matvec, device-resident ------------------------
  * Layout as the reference's salt_q4_matvec (kernels.h:117-130): u32 words of

@@ -228,6 +228,24 @@ int salt_mi355_event_elapsed_ms(void *start, void *stop, float *ms) {
     return hip_ok(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop), "hipEventElapsedTime");
 }
 
+int salt_mi355_graph_begin(void *stream) {
+    return hip_ok(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+}
+void *salt_mi355_graph_end(void *stream) {
+    hipGraph_t graph = nullptr;
+    if (hip_ok(hipStreamEndCapture((hipStream_t)stream, &graph), "hipStreamEndCapture") != 0 || !graph) return nullptr;
+    hipGraphExec_t exec = nullptr;
+    const int rc = hip_ok(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate");
+    (void)hipGraphDestroy(graph);
+    return rc == 0 ? (void *)exec : nullptr;
+}
+int salt_mi355_graph_launch(void *graph_exec, void *stream) {
+    return hip_ok(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream), "hipGraphLaunch");
+}
+int salt_mi355_graph_destroy(void *graph_exec) {
+    return hip_ok(hipGraphExecDestroy((hipGraphExec_t)graph_exec), "hipGraphExecDestroy");
+}
+
 // ---------------------------------------------------------------- Q4, device-resident
 
 int salt_mi355_q4_jobs_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tokens, int chains,

@@ -79,6 +79,10 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_dev_fill, i, vp, i, sz)
     _sig(lib.salt_mi355_stream, vp)
     _sig(lib.salt_mi355_stream_sync, i, vp)
+    _sig(lib.salt_mi355_graph_begin, i, vp)
+    _sig(lib.salt_mi355_graph_end, vp, vp)
+    _sig(lib.salt_mi355_graph_launch, i, vp, vp)
+    _sig(lib.salt_mi355_graph_destroy, i, vp)
     _sig(lib.salt_mi355_event_create, vp)
     _sig(lib.salt_mi355_event_destroy, i, vp)
     _sig(lib.salt_mi355_event_record, i, vp, vp)

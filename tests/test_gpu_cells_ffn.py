@@ -157,3 +157,43 @@ def test_ffn_block_argument_errors(gpu):
     assert args(bad, block.residual.ptr, block.out.ptr, block.ws.ptr) == -1 and lib.salt_mi355_ffn_block_workspace_bytes(C.byref(bad)) == 0
     bad = type(d).from_buffer_copy(d); bad.topk = 5
     assert args(bad, block.residual.ptr, block.out.ptr, block.ws.ptr) == -1
+
+
+def test_block_replayed_as_a_graph(gpu, oracle):
+    """The feed-forward block (two streams forked and joined by events, kernels only: no memset node; the MoE decode
+    step is part of it) captured once and replayed with fresh inputs; every replay is compared with the checker, with
+    eager calls and synchronisations in between."""
+    print("graph replay", flush=True)
+    H, D, F, E, K = 2816, 2112, 704, 16, 8
+    w = synth.ffn_layer(H, D, F, E, K, 5)
+    block = gpu.FfnBlock(w)
+    L = ffn_layer_struct(w)
+    lib = gpu.load()
+    stream = lib.salt_mi355_stream()
+    block.residual.upload((synth.activations(H, 1, 300)[0] * 3).astype(f32))
+    gpu.check(block.enqueue(stream), "eager warm-up")              # first use outside the capture
+    gpu.check(lib.salt_mi355_stream_sync(stream), "sync")
+    gpu.check(lib.salt_mi355_graph_begin(stream), "graph_begin")
+    gpu.check(block.enqueue(stream), "captured block")
+    graph = lib.salt_mi355_graph_end(stream)
+    assert graph, lib.salt_mi355_last_error().decode()
+    want = np.zeros(H, f32); osel = np.zeros(K, np.int32); owt = np.zeros(K, f32)
+    for it in range(4):
+        residual = (synth.activations(H, 1, 301 + it)[0] * 3).astype(f32)
+        if it == 2:
+            residual[9] = np.nan                                      # a rejected input inside a replay
+        block.residual.upload(residual)
+        block.out.upload(np.full(H, 7.0, f32))
+        gpu.check(lib.salt_mi355_graph_launch(graph, stream), "graph_launch")
+        gpu.check(lib.salt_mi355_stream_sync(stream), "sync")
+        status, out = int(block.status.to_host(np.int32)[0]), block.out.to_host(f32)
+        if it == 2:
+            assert status == -1 and (out == 7.0).all()
+        else:
+            assert oracle.orc_ffn_block(C.byref(L), ptr(residual), ptr(want), ptr(osel), ptr(owt), host_threads()) == 0
+            assert status == 0 and np.array_equal(bits(out), bits(want)), it
+            assert np.array_equal(block.sel.to_host(np.int32), osel)
+        # an eager call between replays
+        st, _, _, eager = block.step((synth.activations(H, 1, 400 + it)[0] * 3).astype(f32))
+        assert st == 0
+    assert lib.salt_mi355_graph_destroy(graph) == 0
