@@ -77,3 +77,19 @@ def test_gpu_free_queries(lib):
     ops = lib.salt_gpu_residency_backend_ops()
     assert ops.contents.abi_version == 1 and ops.contents.ops_size == C.sizeof(abi.ResidencyOps)
     assert lib.salt_dispatch_get() is None and lib.salt_gpu_tensor_program_ops() is None
+
+
+def test_a_c99_translation_unit_consumes_both_headers(tmp_path):
+    """The engine is C99: its compiler must accept the public headers as they are, and a C99 program linked against the
+    library must get the documented answers to the GPU-free queries."""
+    exe = tmp_path / "c99_consumer"
+    libdir = ROOT / "salt-core_amd"
+    # taking a function's address as a data pointer is the one thing -pedantic would flag in the consumer itself
+    subprocess.check_call(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-Wno-pedantic",
+                           "-I", str(ROOT / "include"), str(ROOT / "tests" / "c99_consumer.c"), "-o", str(exe),
+                           "-L", str(libdir), "-lsalt_gpu_mi355", f"-Wl,-rpath,{libdir}"])
+    for header in ("salt_gpu_mi355.h", "salt_gpu_mi355_engine.h"):
+        subprocess.check_call(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-x", "c",
+                               "-I", str(ROOT / "include"), str(ROOT / "include" / header)])
+    out = subprocess.check_output([str(exe)], text=True)
+    assert "c99 consumer ok" in out
