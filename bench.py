@@ -278,19 +278,25 @@ def main():
         ms_w = timed(lib, stream, events, warm.step, 5, max(20, args.steps))
         extra["q4_sweep_cache_warm_gbps"] = round(warm.bytes_per_step / (ms_w * 1e-3) / 1e9, 1)
         del warm
-        # MoE decode layer-step, E = 128 top-8, d_model 2816, d_ff 704; fresh logits per layer instance
+        # MoE decode layer-step, E = 128 top-8, d_model 2816, d_ff 704.  Two layer instances (857 MB of experts) and 32
+        # logit vectors per layer taken in turn, so that the selection changes from step to step and the 256 MB
+        # last-level cache cannot hold the experts a step reads.
         E, K, H, F = 128, 8, 2816, 704
         pool = synth.expert_pool(E, H, F, 7)
         layers = [gpu.MoeLayer(pool, E, H, F, K) for _ in range(2)]
+        logit_sets = []
         for i, layer in enumerate(layers):
-            layer.logits.upload(synth.router_logits(E, 900 + i))
+            logit_sets.append([gpu.DeviceBuffer.from_host(synth.router_logits(E, 900 + 100 * i + k)) for k in range(32)])
             layer.scale.upload(np.ones(E, np.float32))
             layer.x.upload(synth.activations(H, 1, 950 + i)[0])
+        turn = [0]
 
         def moe_step(st):
-            for layer in layers:
+            for layer, sets in zip(layers, logit_sets):
+                layer.logits = sets[turn[0] % len(sets)]
                 if layer.enqueue(st) != 0:
                     raise RuntimeError(lib.salt_mi355_last_error().decode())
+            turn[0] += 1
 
         ms_moe = timed(lib, stream, events, moe_step, 5, 100) / len(layers)
         step_bytes = synth.moe_step_bytes(H, F, E, K)
@@ -298,13 +304,18 @@ def main():
         extra["moe_layer_tokens_per_s"] = round(1e3 / ms_moe, 1)
         extra["moe_decode_step_gbps"] = round(step_bytes / (ms_moe * 1e-3) / 1e9, 1)
         extra["moe_decode_step_hbm_frac"] = round(step_bytes / (ms_moe * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
-        del layers
+        del layers, logit_sets
         # the whole feed-forward block of a decoder layer for one token: pre-norms, dense FFN (2112 wide), router input,
-        # 8-bit gate, top-8 of 128, routed experts, parallel combine -- bit-exact, device-resident
+        # 8-bit gate, top-8 of 128, routed experts, parallel combine -- bit-exact, device-resident.  32 residuals taken
+        # in turn: the routing, hence the experts read, changes from block to block.
         block = gpu.FfnBlock(synth.ffn_layer(H, 2112, F, E, K, 70, pool=pool))
-        block.residual.upload((synth.activations(H, 1, 71)[0] * 3).astype(np.float32))
+        residuals = [gpu.DeviceBuffer.from_host((synth.activations(H, 1, 71 + k)[0] * 3).astype(np.float32))
+                     for k in range(32)]
+        ffn_turn = [0]
 
         def ffn_step(st):
+            block.residual = residuals[ffn_turn[0] % len(residuals)]
+            ffn_turn[0] += 1
             if block.enqueue(st) != 0:
                 raise RuntimeError(lib.salt_mi355_last_error().decode())
 
@@ -314,14 +325,14 @@ def main():
         extra["ffn_block_us"] = round(ms_ffn * 1e3, 2)
         extra["ffn_block_layer_tokens_per_s"] = round(1e3 / ms_ffn, 1)
         # the same block captured once and replayed as a HIP graph
-        if lib.salt_mi355_graph_begin(stream) == 0:
+        if lib.salt_mi355_graph_begin(stream) == 0:              # one residual: a graph replays fixed pointers
             ffn_step(stream)
             graph = lib.salt_mi355_graph_end(stream)
             if graph:
                 ms_g = timed(lib, stream, events, lambda st: lib.salt_mi355_graph_launch(graph, st), 5, 100)
                 extra["ffn_block_graph_us"] = round(ms_g * 1e3, 2)
                 lib.salt_mi355_graph_destroy(graph)
-        del block
+        del block, residuals
         # NVFP4 8192 x 8192, batch 1, reference semantics (activation Q/DQ inside the rows' launch), 16 instances
         R = Cc = 8192
         packed, fscales = synth.nvfp4_tensor(R, Cc, 40)
