@@ -66,9 +66,9 @@ int salt_mi355_nvfp4_matvec_dev(const void *packed, const void *scales, float st
     if (!g_state.ready) { set_error("nvfp4 matvec: library not initialised"); return -1; }
     if (!g_state.fp8_is_ocp) { set_error("nvfp4: this device's fp8 converter is not OCP E4M3FN"); return -1; }
     if (!packed || !scales || !xs || !ys || R < 1 || C < 32 || (C & 31) || B < 1 || !isfinite(stored_divisor) ||
-        stored_divisor == 0.0f || ((uintptr_t)packed & 15) || ((uintptr_t)scales & 1) || ((uintptr_t)xs & 3) ||
+        stored_divisor == 0.0f || ((uintptr_t)packed & 3) || ((uintptr_t)scales & 1) || ((uintptr_t)xs & 3) ||
         ((uintptr_t)ys & 3) || (chains != 0 && chains != 8 && chains != 4 && chains != 2)) {
-        set_error("nvfp4 matvec: bad arguments (C must be a multiple of 32, packed 16-byte aligned)");
+        set_error("nvfp4 matvec: bad arguments (C must be a multiple of 32, packed 4-byte aligned)");
         return -1;
     }
     for (int first = 0; first < B; first += 4) {
@@ -161,9 +161,9 @@ int salt_mi355_nvfp4_jobs_dev(const SaltMi355Fp4Job *jobs, int njobs, int C, int
     }
     for (int j = 0; j < njobs; ++j)
         if (!jobs[j].packed || !jobs[j].scales || !jobs[j].xs || !jobs[j].ys || jobs[j].rows < 1 ||
-            !isfinite(jobs[j].stored_divisor) || jobs[j].stored_divisor == 0.0f || ((uintptr_t)jobs[j].packed & 15) ||
+            !isfinite(jobs[j].stored_divisor) || jobs[j].stored_divisor == 0.0f || ((uintptr_t)jobs[j].packed & 3) ||
             ((uintptr_t)jobs[j].scales & 1) || ((uintptr_t)jobs[j].xs & 3) || ((uintptr_t)jobs[j].ys & 3)) {
-            set_error("nvfp4 jobs: job %d is malformed (packed 16-byte aligned, non-zero finite divisor)", j);
+            set_error("nvfp4 jobs: job %d is malformed (packed 4-byte aligned, non-zero finite divisor)", j);
             return -1;
         }
     std::vector<Fp4Job> table((size_t)njobs);
@@ -207,9 +207,9 @@ int salt_mi355_nvfp4_matvec_qdq_dev(const void *packed, const void *scales, floa
     if (!g_state.fp8_is_ocp) { set_error("nvfp4: this device's fp8 converter is not OCP E4M3FN"); return -1; }
     if (!packed || !scales || !x || !y || !status_dev || R < 1 || C < 32 || (C & 31) || C > FP4_FUSED_MAX_COLS ||
         !isfinite(stored_divisor) || stored_divisor == 0.0f || !isfinite(input_global_scale) ||
-        input_global_scale <= 0.0f || ((uintptr_t)packed & 15) || ((uintptr_t)scales & 1) || ((uintptr_t)x & 15) ||
+        input_global_scale <= 0.0f || ((uintptr_t)packed & 3) || ((uintptr_t)scales & 1) || ((uintptr_t)x & 15) ||
         ((uintptr_t)y & 3) || (chains != 0 && chains != 8 && chains != 4 && chains != 2)) {
-        set_error("nvfp4 matvec: bad arguments (C a multiple of 32 up to %d, packed and x 16-byte aligned)",
+        set_error("nvfp4 matvec: bad arguments (C a multiple of 32 up to %d, packed 4-byte and x 16-byte aligned)",
                   FP4_FUSED_MAX_COLS);
         return -1;
     }
@@ -355,7 +355,7 @@ bool ffn_layer_ok(const SaltMi355FfnLayer *L) {
     for (const void *q : need)
         if (!q) return false;
     const size_t n = (size_t)L->hidden * (size_t)L->routed;
-    return ((uintptr_t)L->pool & 15) == 0 && (L->expert_stride & 15) == 0 && L->expert_stride >= 3 * (n / 2 + 4 * (n / 64));
+    return ((uintptr_t)L->pool & 3) == 0 && (L->expert_stride & 15) == 0 && L->expert_stride >= 3 * (n / 2 + 4 * (n / 64));
 }
 
 }  // namespace
@@ -503,8 +503,8 @@ int salt_mi355_moe_decode_step_dev(const void *pool, size_t expert_stride, int h
                                    void *stream) {
     if (!g_state.ready) { set_error("moe step: library not initialised"); return -1; }
     if (!pool || !logits || !per_expert_scale || !x || !selected || !weights || !out || !workspace ||
-        ((uintptr_t)pool & 15) || (expert_stride & 15) || ((uintptr_t)workspace & 255)) {
-        set_error("moe step: bad arguments (pool and expert stride 16-byte aligned, workspace 256-byte aligned)");
+        ((uintptr_t)pool & 3) || (expert_stride & 15) || ((uintptr_t)workspace & 255)) {
+        set_error("moe step: bad arguments (pool 4-byte aligned, expert stride a multiple of 16, workspace 256-byte aligned)");
         return -1;
     }
     const MoeGeometry g = {hidden, routed, n_experts, topk};

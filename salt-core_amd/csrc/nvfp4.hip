@@ -31,7 +31,8 @@ typedef const float __attribute__((address_space(4))) *uniform_f32_ptr;
 typedef const uint64_t __attribute__((address_space(4))) *uniform_u64_ptr;
 typedef const uint8_t __attribute__((address_space(1))) *global_u8_ptr;
 typedef const uint16_t __attribute__((address_space(1))) *global_u16_ptr;
-typedef const u32x4 __attribute__((address_space(1))) *global_u128_ptr;
+typedef u32x4 __attribute__((aligned(4))) u32x4_dword_aligned;       // 128-bit global loads need dword alignment only
+typedef const u32x4_dword_aligned __attribute__((address_space(1))) *global_u128_ptr;
 typedef float __attribute__((address_space(1))) *global_f32_out_ptr;
 
 constexpr int TILE_ROWS = 64;

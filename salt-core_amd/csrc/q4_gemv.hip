@@ -56,7 +56,10 @@ __device__ __forceinline__ float bf16_to_f32(uint32_t half) { return __uint_as_f
 typedef const uint8_t __attribute__((address_space(1))) *global_u8_ptr;
 typedef const uint16_t __attribute__((address_space(1))) *global_u16_ptr;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef const u32x4 __attribute__((address_space(1))) *global_u128_ptr;
+// 128-bit global loads need dword alignment only; the engine's expert pool file puts every tensor 8 bytes past a
+// multiple of 16 (24-byte header), and those must still take the tiled path.
+typedef u32x4 __attribute__((aligned(4))) u32x4_dword_aligned;
+typedef const u32x4_dword_aligned __attribute__((address_space(1))) *global_u128_ptr;
 typedef float __attribute__((address_space(1))) *global_f32_out_ptr;
 typedef const uint64_t __attribute__((address_space(4))) *uniform_u64_ptr;
 
@@ -584,7 +587,7 @@ int env_chains() {
 }  // namespace
 
 bool q4_job_is_tileable(const Q4Job &job, int cols) {
-    return cols >= 64 && (cols & 63) == 0 && ((uintptr_t)job.vals & 15) == 0 && ((uintptr_t)job.scales & 1) == 0 &&
+    return cols >= 64 && (cols & 63) == 0 && ((uintptr_t)job.vals & 3) == 0 && ((uintptr_t)job.scales & 1) == 0 &&
            ((uintptr_t)job.biases & 1) == 0 && ((uintptr_t)job.x & 3) == 0 && ((uintptr_t)job.y & 3) == 0;
 }
 

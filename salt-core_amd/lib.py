@@ -175,18 +175,20 @@ class DeviceBuffer:
 
 
 def q4_matvec(vals: np.ndarray, scales: np.ndarray, biases: np.ndarray | None, R: int, C_: int,
-              xs: np.ndarray, chains: int = 0) -> np.ndarray:
+              xs: np.ndarray, chains: int = 0, value_offset: int = 0) -> np.ndarray:
     """Host-array convenience around salt_mi355_q4_matvec_dev: uploads, runs on
-    the library stream, downloads ys[B, R]."""
+    the library stream, downloads ys[B, R].  value_offset shifts the packed values by that many bytes inside their
+    device allocation (alignment cases)."""
     lib = init()
     xs = np.ascontiguousarray(xs, np.float32).reshape(-1, C_)
     B = xs.shape[0]
-    dv, ds = DeviceBuffer.from_host(vals), DeviceBuffer.from_host(scales)
+    dv, ds = DeviceBuffer(vals.nbytes + value_offset + 16, fill=0), DeviceBuffer.from_host(scales)
+    dv.upload(vals, value_offset)
     db = DeviceBuffer.from_host(biases) if biases is not None else None
     dx = DeviceBuffer.from_host(xs)
     dy = DeviceBuffer(B * R * 4, fill=0xFF)
     stream = lib.salt_mi355_stream()
-    check(lib.salt_mi355_q4_matvec_dev(dv.ptr, ds.ptr, db.ptr if db else None, R, C_, B, dx.ptr, dy.ptr,
+    check(lib.salt_mi355_q4_matvec_dev(dv.at(value_offset), ds.ptr, db.ptr if db else None, R, C_, B, dx.ptr, dy.ptr,
                                        chains, stream), "q4_matvec_dev")
     check(lib.salt_mi355_stream_sync(stream), "sync")
     return dy.to_host(np.float32).reshape(B, R)
@@ -348,11 +350,14 @@ class FfnBlock:
 class MoeLayer:
     """One layer's expert pool resident in HBM plus the step workspace."""
 
-    def __init__(self, pool: np.ndarray, n_experts: int, hidden: int, routed: int, topk: int):
+    def __init__(self, pool: np.ndarray, n_experts: int, hidden: int, routed: int, topk: int, header_bytes: int = 0):
+        """header_bytes: bytes in front of expert 0 inside the device allocation (the engine's pool file has 24)."""
         self.lib = init()
         self.E, self.H, self.F, self.K = n_experts, hidden, routed, topk
         self.stride = pool.nbytes // n_experts
-        self.pool = DeviceBuffer.from_host(pool)
+        self.header = header_bytes
+        self.pool = DeviceBuffer(pool.nbytes + header_bytes, fill=0)
+        self.pool.upload(pool, header_bytes)
         self.ws = DeviceBuffer(self.lib.salt_mi355_moe_workspace_bytes(hidden, routed, n_experts, topk), fill=0)
         self.logits, self.scale = DeviceBuffer(n_experts * 4), DeviceBuffer(n_experts * 4)
         self.x, self.out = DeviceBuffer(hidden * 4), DeviceBuffer(hidden * 4)
@@ -361,7 +366,7 @@ class MoeLayer:
 
     def enqueue(self, stream):
         return self.lib.salt_mi355_moe_decode_step_dev(
-            self.pool.ptr, self.stride, self.H, self.F, self.E, self.K, self.logits.ptr, self.scale.ptr, self.x.ptr,
+            self.pool.at(self.header), self.stride, self.H, self.F, self.E, self.K, self.logits.ptr, self.scale.ptr, self.x.ptr,
             self.sel.ptr, self.w.ptr, self.eo.ptr, self.out.ptr, self.ws.ptr, stream)
 
     def step(self, logits, scale, x):

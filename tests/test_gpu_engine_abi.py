@@ -237,6 +237,40 @@ def test_moe_chain_from_a_layer_resource(eng, oracle, pkg):
     eng.salt_gpu_set_mapped_only(0)
 
 
+def test_moe_chain_from_a_pool_file_image(eng, oracle, pkg):
+    """The engine's expert pool file: three 64-bit header words {slot bytes, layers, experts}, then the slots
+    (reference gemma4_text.c:73-79, 1618-1623).  The whole image is one resource; every tensor in it sits 8 bytes past a
+    multiple of 16 and must still be served by the tiled kernels, bit for bit."""
+    import time
+    E, H, F = 8, 2816, 704
+    slots = synth.expert_pool(E, H, F, 43)
+    slot_bytes = synth.expert_slot_bytes(H, F)
+    image = np.zeros(24 + slots.nbytes, np.uint8)
+    image[:24] = np.array([slot_bytes, 1, E], np.uint64).view(np.uint8)
+    image[24:] = slots
+    pool = image[24:]                                   # expert 0; a view, so the addresses lie inside the image
+    assert pool.ctypes.data % 16 == 8 or image.ctypes.data % 16 != 0
+    assert eng.salt_gpu_expert_resource_bind(10, image.ctypes.data, image.nbytes) == 0, err(pkg)
+    experts, groups = [0, 2, 5, 7], [1, 1, 1, 1]
+    recs = (abi.MoeExpert * 4)(*[expert_record(pool, e, H, F, n) for e, n in zip(experts, groups)])
+    rows = sum(groups)
+    inputs = synth.activations(H, rows, 44); outputs = np.zeros((rows, H), np.float32)
+    scratch = np.zeros((2, rows * F), np.float32)
+    eng.salt_gpu_set_mapped_only(1)
+    call = lambda: eng.salt_gpu_q4_moe_chain(recs, 4, H, F, ptr(inputs), ptr(outputs), ptr(scratch[0]), ptr(scratch[1]),
+                                             rows * F)
+    assert call() == 0, err(pkg)
+    assert np.array_equal(bits(outputs), bits(chain_want(oracle, slots, H, F, experts, groups, inputs)))
+    t0 = time.perf_counter()
+    for _ in range(20):
+        assert call() == 0
+    per_call_us = (time.perf_counter() - t0) / 20 * 1e6
+    print(f"moe chain from a pool-file image: {per_call_us:.0f} us per call", flush=True)
+    assert per_call_us < 2000                           # the per-row kernel for unaligned tensors needs several ms here
+    eng.salt_gpu_set_mapped_only(0)
+    assert eng.salt_gpu_expert_resource_unbind(10) == 0
+
+
 def shared_array(eng, nfloats):
     buf = abi.SharedBuffer()
     assert eng.salt_gpu_shared_buffer_alloc(C.byref(buf), nfloats * 4) == 0

@@ -244,6 +244,25 @@ def test_moe_decode_step_fresh_logits_and_rejection(gpu, oracle):
     assert layer.step(logits, scale, x)[0] == -1
 
 
+def test_moe_decode_step_behind_a_pool_file_header(gpu, oracle):
+    """Expert 0 starts 24 bytes into the allocation, as in the engine's pool file (three 64-bit header words): every
+    tensor of every expert is then 8 bytes past a multiple of 16."""
+    print("moe step, pool behind a 24-byte header", flush=True)
+    E, K, H, F = 16, 8, 2816, 704
+    pool = synth.expert_pool(E, H, F, 33)
+    layer = gpu.MoeLayer(pool, E, H, F, K, header_bytes=24)
+    g = ExpertGeometry(H, F)
+    scale = synth.rng(3).uniform(0.5, 2.0, E).astype(np.float32)
+    logits = synth.router_logits(E, 71); x = synth.activations(H, 1, 72)[0]
+    st, sel, w, eo, y = layer.step(logits, scale, x)
+    osel = np.zeros(K, np.int32); ow = np.zeros(K, np.float32)
+    oeo = np.zeros((K, H), np.float32); oy = np.zeros(H, np.float32)
+    assert oracle.orc_moe_decode_step(C.byref(g), ptr(pool), E, K, ptr(logits), ptr(scale), ptr(x), ptr(osel), ptr(ow),
+                                      ptr(oeo), ptr(oy), host_threads()) == 0
+    assert st == 0 and np.array_equal(sel, osel) and np.array_equal(bits(w), bits(ow))
+    assert np.array_equal(bits(eo), bits(oeo)) and np.array_equal(bits(y), bits(oy))
+
+
 @pytest.mark.parametrize("E,K,H,F,why", [
     (520, 4, 128, 64, "more experts than the fused prologue holds: router, gate/up, activate, down, reduce as five launches"),
     (16, 16, 2816, 2048, "more than two tiles per compute unit: eight waves per tile in both fused launches"),

@@ -60,6 +60,18 @@ def test_reference_fixtures(gpu, case):
     assert np.array_equal(bits(got)[:, fx[name + ".rows"]], fx[name + ".y_bits"])
 
 
+@pytest.mark.parametrize("offset", [4, 8, 12, 24])
+def test_tiled_kernel_with_dword_aligned_values(gpu, oracle, offset):
+    """Packed values that start 4, 8 or 12 bytes past a multiple of 16 (the engine's expert pool file puts every tensor
+    24 bytes past a page boundary): same bits, still the tiled kernel."""
+    print("q4 value offset", offset, flush=True)
+    for R, C, B in [(2816, 704, 1), (130, 2816, 2)]:
+        vals, scales, biases = synth.q4_tensor(R, C, offset + R)
+        xs = synth.activations(C, B, 9)
+        got = gpu.q4_matvec(vals, scales, biases, R, C, xs, value_offset=offset)
+        assert np.array_equal(bits(got), bits(oracle_batch(oracle, vals, scales, biases, R, C, xs)))
+
+
 def test_generic_kernel_odd_columns_and_null_bias(gpu, oracle):
     for R, C, B in [(8, 200, 1), (9, 96, 2), (70, 40, 1)]:
         print(f"generic R={R} C={C} B={B}", flush=True)
