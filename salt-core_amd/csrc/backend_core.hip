@@ -131,6 +131,9 @@ int salt_mi355_init(void) {
         return -1;
     }
     hipDeviceProp_t prop;
+    // The owner thread waits for every call's completion: spinning on it answers microseconds sooner than blocking.
+    (void)hipSetDeviceFlags(hipDeviceScheduleSpin);
+    (void)hipGetLastError();                     // refused when the process has already touched the device: harmless
     if (hip_ok(hipSetDevice(0), "hipSetDevice") != 0 ||
         hip_ok(hipGetDeviceProperties(&prop, 0), "hipGetDeviceProperties") != 0)
         return -1;
@@ -289,6 +292,8 @@ int salt_mi355_q4_jobs_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tok
         State::TableSlot *slot = nullptr;
         if (njobs == 1) {
             launch.one = table[0];
+        } else if (njobs <= Q4_INLINE_JOBS) {
+            memcpy(launch.inline_jobs, table.data(), (size_t)njobs * sizeof(Q4Job));
         } else {
             slot = table_acquire(table.data(), table.size() * sizeof(Q4Job), stream);
             if (!slot) return -1;

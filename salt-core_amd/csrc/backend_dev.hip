@@ -322,7 +322,6 @@ int salt_mi355_cells_dev(const SaltMi355Cell *cells, int count, int *status_dev,
 namespace {
 
 struct FfnWorkspace {
-    Q4Job *dense_jobs;         // two records written by the opening kernel
     float *norm_a, *norm_b, *router_in, *dense_out, *routed_out, *sum, *gate, *up, *act, *logits, *expert_out;
     void *moe;
 };
@@ -334,7 +333,6 @@ size_t ffn_carve(const SaltMi355FfnLayer &L, void *base, FfnWorkspace *ws) {
     const size_t H = (size_t)L.hidden * 4, D = (size_t)L.dense * 4;
     auto take = [&](size_t bytes) { uint8_t *at = p; p += pad256(bytes); return at; };
     FfnWorkspace w;
-    w.dense_jobs = (Q4Job *)take(2 * sizeof(Q4Job));
     w.norm_a = (float *)take(H); w.norm_b = (float *)take(H); w.router_in = (float *)take(H);
     w.dense_out = (float *)take(H); w.routed_out = (float *)take(H); w.sum = (float *)take(2 * H);
     w.gate = (float *)take(D); w.up = (float *)take(D); w.act = (float *)take(D);
@@ -380,7 +378,7 @@ int salt_mi355_ffn_block_dev(const SaltMi355FfnLayer *layer, const float *residu
     MoeWorkspace moe;
     moe_workspace_carve(g, ws.moe, &moe);
 
-    // dense gate and up as one two-job launch; the job records reach the device inside the opening kernel's arguments
+    // dense gate and up as one two-job launch; the job records travel inside that launch's arguments
     Q4Job dense[2];
     memset(dense, 0, sizeof dense);
     for (int k = 0; k < 2; ++k) {
@@ -393,12 +391,13 @@ int salt_mi355_ffn_block_dev(const SaltMi355FfnLayer *layer, const float *residu
     memset(&gate_up, 0, sizeof gate_up);
     gate_up.total_tiles = q4_assign_tiles(dense, 2);
     gate_up.tiles_per_job = q4_uniform_tiles(dense, 2);
-    gate_up.table = ws.dense_jobs; gate_up.njobs = 2; gate_up.cols = L.hidden; gate_up.tokens = 1;
+    memcpy(gate_up.inline_jobs, dense, sizeof dense);
+    gate_up.table = nullptr; gate_up.njobs = 2; gate_up.cols = L.hidden; gate_up.tokens = 1;
     gate_up.code_scale = g_state.code_scale; gate_up.fused = g_state.q4_fused;
     const bool tileable = q4_job_is_tileable(dense[0], L.hidden) && q4_job_is_tileable(dense[1], L.hidden);
 
     if (ffn_pre_launch(residual, L.pre_norm, L.pre_norm_2, L.router_scale, ws.norm_a, ws.norm_b, ws.router_in, L.hidden, L.eps,
-                       status_dev, dense, ws.dense_jobs, stream) != 0) {
+                       status_dev, stream) != 0) {
         set_error("ffn block: pre-norm launch failed");
         return -1;
     }

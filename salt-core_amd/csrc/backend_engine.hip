@@ -86,6 +86,7 @@ struct Engine {
     uint64_t device_copied_bytes = 0, peak_window_bytes = 0;
     // activation staging: bump regions of one pinned and one device buffer
     uint8_t *pinned = nullptr, *device = nullptr;
+    uint8_t *pinned_dev = nullptr;    // the pinned region as kernels address it (zero-copy for small calls)
     size_t staging_capacity = 0, pinned_used = 0, device_used = 0;
     // scratch for weights that arrive without a resident resource
     uint8_t *legacy = nullptr;
@@ -112,9 +113,12 @@ int staging_reserve(size_t pinned_bytes, size_t device_bytes) {
     e.staging_capacity = 0;
     size_t capacity = 64u << 20;
     while (capacity < need) capacity *= 2;
-    if (hip_ok(hipHostMalloc((void **)&e.pinned, capacity, hipHostMallocDefault), "hipHostMalloc staging") != 0 ||
+    if (hip_ok(hipHostMalloc((void **)&e.pinned, capacity, hipHostMallocMapped), "hipHostMalloc staging") != 0 ||
         hip_ok(hipMalloc((void **)&e.device, capacity), "hipMalloc staging") != 0)
         return -1;
+    void *view = nullptr;
+    e.pinned_dev = hipHostGetDevicePointer(&view, e.pinned, 0) == hipSuccess ? (uint8_t *)view : nullptr;
+    (void)hipGetLastError();
     e.staging_capacity = capacity;
     return 0;
 }
@@ -131,6 +135,13 @@ uint8_t *device_take(size_t nbytes) {
     e.device_used += align_up(nbytes, 256);
     return p;
 }
+
+// Calls that return this little write their results straight into the pinned staging memory: one copy command fewer
+// per call.  (Reading the activations from there as well was measured: every tile re-reads them across the bus and
+// a 4096 x 4096 call went from 33 to 51 us.)
+constexpr size_t ZERO_COPY_BYTES = 128 * 1024;
+bool zero_copy(size_t nbytes) { return g_engine.pinned_dev != nullptr && nbytes <= ZERO_COPY_BYTES; }
+uint8_t *pinned_device_view(const uint8_t *pin) { return g_engine.pinned_dev + (pin - g_engine.pinned); }
 
 // Copies host floats to the device through pinned memory on the library stream.
 float *upload_activations(const float *host, size_t count) {
@@ -341,9 +352,13 @@ int run_q4_jobs(std::vector<HostJob> &jobs, int C, std::vector<OutputCopy> *copi
         if (!j.y_dev) {
             const size_t count = (size_t)j.tokens * j.rows;
             uint8_t *dev = device_take(count * 4), *pin = pinned_take(count * 4);
-            j.y_dev = (float *)dev;
             e.pending.push_back({pin, j.y_host, count * 4});
-            copies->push_back({dev, pin, count * 4});
+            if (zero_copy(count * 4)) {
+                j.y_dev = (float *)pinned_device_view(pin);          // written in place, nothing to copy back
+            } else {
+                j.y_dev = (float *)dev;
+                copies->push_back({dev, pin, count * 4});
+            }
         }
     }
     int max_tokens = 0;
@@ -852,6 +867,8 @@ int moe_chain(const SaltGpuMoeExpert *experts, int count, int hidden, int routed
     float *gate_dev = (float *)device_take(mid_floats * 4), *up_dev = (float *)device_take(mid_floats * 4);
     float *act_dev = (float *)device_take(mid_floats * 4);
     uint8_t *out_dev = device_take(in_floats * 4), *out_pin = pinned_take(in_floats * 4);
+    const bool out_in_place = zero_copy(in_floats * 4);
+    if (out_in_place) out_dev = pinned_device_view(out_pin);
     std::vector<HostJob> jobs;
     size_t row = 0;
     for (int i = 0; i < count; ++i) {
@@ -876,7 +893,8 @@ int moe_chain(const SaltGpuMoeExpert *experts, int count, int hidden, int routed
     }
     if (run_q4_jobs(jobs, routed, &none) != 0) { (void)salt_gpu_sync(); return -1; }
     e.pending.push_back({out_pin, outputs, in_floats * 4});
-    std::vector<OutputCopy> copies(1, OutputCopy{out_dev, out_pin, in_floats * 4});
+    std::vector<OutputCopy> copies;
+    if (!out_in_place) copies.push_back(OutputCopy{out_dev, out_pin, in_floats * 4});
     count_batch(experts[0].gate_vals, any_legacy);
     return finish_call(copies);
 }

@@ -220,15 +220,12 @@ struct PreArgs {
     int n;
     float eps;
     int *status;               // written, not only set: this kernel opens the block
-    Q4Job jobs[2];             // copied to jobs_out for the launch that follows
-    Q4Job *jobs_out;
 };
 
 // n <= SQ_CHUNK: every input is requested once, up front, and lives in registers from then on
 __global__ __launch_bounds__(THREADS) void ffn_pre_small_kernel(PreArgs a) {
     __shared__ __attribute__((aligned(16))) float sq[SQ_CHUNK + SQ_TAIL];
     __shared__ float shared[4];
-    if (a.jobs_out && threadIdx.x < 2) a.jobs_out[threadIdx.x] = a.jobs[threadIdx.x];
     unsigned bad = !(a.eps >= 0.0f) || nonfinite(a.eps);
     float r[1][SLOTS], w1[SLOTS], w2[SLOTS], rs[SLOTS];
 #pragma unroll
@@ -268,7 +265,6 @@ __global__ __launch_bounds__(THREADS) void ffn_pre_small_kernel(PreArgs a) {
 __global__ __launch_bounds__(THREADS) void ffn_pre_kernel(PreArgs a) {
     __shared__ __attribute__((aligned(16))) float sq[SQ_CHUNK + SQ_TAIL];
     __shared__ float shared[4];
-    if (a.jobs_out && threadIdx.x < 2) a.jobs_out[threadIdx.x] = a.jobs[threadIdx.x];
     unsigned bad = !(a.eps >= 0.0f) || nonfinite(a.eps);
     const float *vec[1] = {a.residual};
     float ss;
@@ -479,11 +475,9 @@ int norm_cell_launch(int kind, const float *x, const float *weight, const float 
 }
 
 int ffn_pre_launch(const float *residual, const float *w1, const float *w2, const float *router_scale, float *norm_a,
-                   float *norm_b, float *router_in, int n, float eps, int *status, const Q4Job *jobs, Q4Job *jobs_out,
-                   hipStream_t stream) {
+                   float *norm_b, float *router_in, int n, float eps, int *status, hipStream_t stream) {
     if (!residual || !w1 || !w2 || !router_scale || !norm_a || !norm_b || !router_in || !status || n < 1) return -1;
-    PreArgs a = {residual, w1, w2, router_scale, norm_a, norm_b, router_in, n, eps, status, {}, jobs_out};
-    if (jobs_out) { a.jobs[0] = jobs[0]; a.jobs[1] = jobs[1]; }
+    PreArgs a = {residual, w1, w2, router_scale, norm_a, norm_b, router_in, n, eps, status};
     if (n <= SQ_CHUNK) ffn_pre_small_kernel<<<dim3(1), dim3(THREADS), 0, stream>>>(a);
     else ffn_pre_kernel<<<dim3(1), dim3(THREADS), 0, stream>>>(a);
     return launched() ? 0 : -1;

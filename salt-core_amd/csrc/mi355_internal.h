@@ -42,9 +42,11 @@ struct MoeFuse {
 constexpr int MOE_FUSE_MAX_ROUTED = 4096;      // activations of one expert held in LDS by the down launch
 constexpr int MOE_FUSE_MAX_EXPERTS = 512;      // one thread per expert in the gate/up prologue
 
+constexpr int Q4_INLINE_JOBS = 16;
+
 struct Q4Launch {
-    Q4Job one;                // used when table == nullptr
-    const Q4Job *table;       // device array of njobs jobs sorted by tile0
+    Q4Job one;                // used when njobs == 1
+    const Q4Job *table;       // device array of njobs jobs sorted by tile0; nullptr: the jobs travel in `inline_jobs`
     int njobs;
     int cols;                 // C, shared by every job of the launch
     int tokens;               // 1..4 activation rows per job
@@ -53,6 +55,9 @@ struct Q4Launch {
     int tiles_per_job;        // > 0 when every job of the table has this many tiles (tile -> job by division), else 0
     int fused;                // 0: separately rounded multiply and add (bit-exact); 1: fma accumulate
     MoeFuse moe;              // only read by q4_moe_gate_up_launch / q4_moe_down_launch
+    // Up to Q4_INLINE_JOBS job records inside the kernel arguments: a decode-sized batch (the gate and up projections
+    // of eight experts) then needs no table upload.  Must stay the last member.
+    Q4Job inline_jobs[Q4_INLINE_JOBS];
 };
 int q4_moe_gate_up_launch(const Q4Launch &launch, hipStream_t stream);   // fills tiles and jobs from launch.moe
 int q4_moe_down_launch(const Q4Launch &launch, hipStream_t stream);
@@ -193,11 +198,9 @@ int q8_launch(const Q8Launch &launch, hipStream_t stream);
 // input or a result is not finite.  kind: 0 rms norm (weight optional), 1 router input, 2 residual post-norm.
 int norm_cell_launch(int kind, const float *x, const float *weight, const float *residual, float *out, int n, float eps,
                      float root, int *status, hipStream_t stream);
-// Opens a feed-forward block: *status is written (0 or -1); two job records (optional) are copied to jobs_out for the
-// dense gate/up launch that follows.
+// Opens a feed-forward block: *status is written (0 or -1), not only set.
 int ffn_pre_launch(const float *residual, const float *w1, const float *w2, const float *router_scale, float *norm_a,
-                   float *norm_b, float *router_in, int n, float eps, int *status, const Q4Job *jobs, Q4Job *jobs_out,
-                   hipStream_t stream);
+                   float *norm_b, float *router_in, int n, float eps, int *status, hipStream_t stream);
 int combine_cell_launch(const float *residual, const float *dense, const float *routed, const float *wd, const float *wr,
                         const float *wf, float *sum_scratch, float *out, int n, float eps, float scalar, int *status,
                         const int *other_status, const float *expert_out, const float *weights, int topk,

@@ -68,8 +68,13 @@ static_assert(sizeof(Q4Job) == 56 && offsetof(Q4Job, rows) == 40 && offsetof(Q4J
               "find_job reads a job record as seven 64-bit words");
 
 __device__ __forceinline__ Q4Job find_job(const Q4Launch &L, int tile) {
-    if (L.table == nullptr) return L.one;
-    const uniform_u64_ptr words = (uniform_u64_ptr)(uintptr_t)L.table;     // 7 words per record
+    if (L.njobs <= 1) return L.one;
+    // 7 words per record, in a device table or inside the kernel arguments (the launch record is the kernel's only
+    // argument, so the inline records sit at their offset in the kernarg segment)
+    const uniform_u64_ptr words =
+        L.table ? (uniform_u64_ptr)(uintptr_t)L.table
+                : (uniform_u64_ptr)((const char __attribute__((address_space(4))) *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                    offsetof(Q4Launch, inline_jobs));
     int lo = 0, hi = L.njobs - 1;
     if (L.tiles_per_job > 0) {             // every job has the same number of tiles: no search
         lo = tile / L.tiles_per_job;
