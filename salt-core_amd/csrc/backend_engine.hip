@@ -1349,6 +1349,22 @@ int salt_gpu_bf16_matvec(const void *key, int R, int C, const float *input, floa
     return finish_call(copies);
 }
 
+// ================================================================ whole-mapping conveniences of the reference ABI
+
+// One mapped trunk range at a time (reference src/gpu_metal.m:1533-1536): trunk resource 0, copied to HBM.
+int salt_gpu_resident_trunk_map(const void *base, size_t nbytes) {
+    if (ready_or_fail("resident_trunk_map") != 0) return -1;
+    const int ri = find_resource(1, 0);
+    if (!base || nbytes < 1 || (ri >= 0 && g_engine.resources[(size_t)ri].active)) {
+        set_error("resident_trunk_map: bad arguments, or a trunk range is already mapped");
+        return -1;
+    }
+    return salt_gpu_weight_resource_bind(1, 0, base, nbytes);
+}
+int salt_gpu_resident_trunk_unmap(void) { return salt_gpu_weight_resource_unbind(1, 0); }   // reference gpu_hip.cpp:5180
+// reference src/gpu_metal.m:1633-1642: the expert pool mapping is expert-layer resource 0
+int salt_gpu_resident_pool_map(const void *base, size_t nbytes) { return salt_gpu_expert_resource_bind(0, base, nbytes); }
+
 // ================================================================ fp32 cells over shared buffers
 
 int salt_gpu_exact_cells(const SaltGpuExactCell *cells, int count) {
@@ -1561,9 +1577,6 @@ const SaltGpuResidencyBackendOps *salt_gpu_residency_backend_ops(void) { return 
 int salt_gpu_bf16_matvec_batch(const void *, int, int, int, const float *, float *) { return -1; }
 const struct SaltGpuDispatch *salt_dispatch_get(void) { return nullptr; }
 const struct SaltTextGpuProgramOps *salt_gpu_tensor_program_ops(void) { return nullptr; }
-int salt_gpu_resident_trunk_map(const void *, size_t) { return -1; }
-int salt_gpu_resident_trunk_unmap(void) { return -1; }
-int salt_gpu_resident_pool_map(const void *, size_t) { return -1; }
 int salt_gpu_attention_batch(int, int, int, int, int, const SaltGpuSharedBuffer *, size_t, const SaltGpuSharedBuffer *,
                              size_t, size_t, int, int, int, int, SaltGpuSharedBuffer *, size_t, SaltGpuSharedBuffer *,
                              size_t, size_t, int) { return -1; }

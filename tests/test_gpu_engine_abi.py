@@ -608,8 +608,28 @@ def test_exact_cells_over_a_shared_buffer(eng, oracle, pkg):
 
 def test_off_path_entry_points_answer_like_the_null_backend(eng):
     z = np.zeros(64, np.float32)
-    assert eng.salt_gpu_resident_trunk_map(ptr(z), 256) == -1 and eng.salt_gpu_resident_pool_map(ptr(z), 256) == -1
     assert eng.salt_dispatch_get() is None and eng.salt_gpu_tensor_program_ops() is None
+
+
+def test_whole_mapping_conveniences(eng, oracle, pkg):
+    """salt_gpu_resident_trunk_map / _unmap / _pool_map: one trunk range at a time, weights served from it."""
+    R, Cc = 130, 2816
+    vals, scales, biases = synth.q4_tensor(R, Cc, 61)
+    blob = np.concatenate([np.zeros(100, np.uint8), vals.view(np.uint8), scales.view(np.uint8), biases.view(np.uint8)])
+    base = blob.ctypes.data
+    v, s, b = base + 100, base + 100 + vals.nbytes, base + 100 + vals.nbytes + scales.nbytes
+    assert eng.salt_gpu_resident_trunk_map(base, blob.nbytes) == 0, err(pkg)
+    assert eng.salt_gpu_resident_trunk_map(base, blob.nbytes) == -1                 # one mapping at a time
+    eng.salt_gpu_set_mapped_only(1)
+    x = synth.activations(Cc, 1, 62)[0]; y = np.zeros(R, np.float32)
+    assert eng.salt_gpu_q4_matvec(v, s, b, R, Cc, ptr(x), ptr(y)) == 0, err(pkg)
+    assert np.array_equal(bits(y), bits(q4_want(oracle, vals, scales, biases, R, Cc, x)[0]))
+    assert eng.salt_gpu_resident_trunk_unmap() == 0
+    assert eng.salt_gpu_q4_matvec(v, s, b, R, Cc, ptr(x), ptr(y)) == -1             # gone, and copying is forbidden
+    assert eng.salt_gpu_resident_pool_map(base, blob.nbytes) == 0, err(pkg)         # expert-layer resource 0
+    assert eng.salt_gpu_q4_matvec(v, s, b, R, Cc, ptr(x), ptr(y)) == 0
+    assert eng.salt_gpu_expert_resource_unbind(0) == 0
+    eng.salt_gpu_set_mapped_only(0)
 
 
 def test_zz_free_and_reinit(eng, pkg):
