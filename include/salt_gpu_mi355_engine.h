@@ -345,6 +345,14 @@ typedef struct SaltGpuExactCell {                 /* reference gpu.h:224-232 */
  * result (that cell and every later one then publish nothing) or a view lies outside its buffer. */
 int salt_gpu_exact_cells(const SaltGpuExactCell *cells, int count);              /* reference gpu.h:234 */
 
+/* ---- whole-mapping conveniences ------------------------------------------- */
+
+/* One mapped trunk range at a time, copied to HBM as trunk resource 0 (reference gpu_metal.m:1533-1536); unmap
+ * releases it (reference gpu_hip.cpp:5180).  pool_map is expert-layer resource 0 (reference gpu_metal.m:1633-1642). */
+int salt_gpu_resident_trunk_map(const void *base, size_t nbytes);                /* reference gpu.h:180 */
+int salt_gpu_resident_trunk_unmap(void);                                         /* reference gpu.h:183 */
+int salt_gpu_resident_pool_map(const void *base, size_t nbytes);                 /* reference gpu.h:484 */
+
 /* ---- outside the quantized decode path: answered like the null backend ---- */
 
 struct SaltGpuDispatch;
@@ -353,9 +361,6 @@ struct SaltTextGpuProgramOps;
 int salt_gpu_bf16_matvec_batch(const void *key, int R, int C, int B, const float *inputs, float *outputs);
 const struct SaltGpuDispatch *salt_dispatch_get(void);                           /* reference gpu.h:163 */
 const struct SaltTextGpuProgramOps *salt_gpu_tensor_program_ops(void);           /* reference gpu.h:209 */
-int salt_gpu_resident_trunk_map(const void *base, size_t nbytes);                /* reference gpu.h:180 */
-int salt_gpu_resident_trunk_unmap(void);                                         /* reference gpu.h:183 */
-int salt_gpu_resident_pool_map(const void *base, size_t nbytes);                 /* reference gpu.h:484 */
 /* reference gpu.h:239-274: prefill attention, KV mirror and Q/K/V transform */
 int salt_gpu_attention_batch(int full_attention, int n_heads, int n_kv_heads, int head_dim, int window,
                              const SaltGpuSharedBuffer *queries, size_t query_float_offset,
