@@ -139,25 +139,40 @@ __global__ __launch_bounds__(MAX_EXPERTS) void group_scan_kernel(const ScanArgs 
     }
 }
 
-// one wave per expert: its (token, rank) pairs in token-major order.  The wave
-// walks the selection 64 pairs at a time (one coalesced load); a match's place
-// is the matches before the chunk plus the matching lanes below it, so no
-// workgroup barrier is needed.
-__global__ __launch_bounds__(256) void group_fill_kernel(const int *__restrict__ selected, int pairs, int topk,
-                                                         const int *__restrict__ offsets, int n_experts,
-                                                         const PrefillPlan *__restrict__ plan,
-                                                         int *__restrict__ row_pairs, int *__restrict__ pair_rows) {
+// One workgroup of sixteen waves per expert: its (token, rank) pairs in token-major order.  Each wave owns a
+// contiguous run of the selection and walks it 64 pairs at a time (one coalesced load), twice: first to count its
+// matches, then, knowing how many matches the waves before it hold, to place them.  A match's place inside a chunk
+// is the number of matching lanes below it, so the order is the selection's own.
+constexpr int FILL_WAVES = 16;
+
+__global__ __launch_bounds__(FILL_WAVES * 64) void group_fill_kernel(const int *__restrict__ selected, int pairs, int topk,
+                                                                     const int *__restrict__ offsets, int n_experts,
+                                                                     const PrefillPlan *__restrict__ plan,
+                                                                     int *__restrict__ row_pairs,
+                                                                     int *__restrict__ pair_rows) {
+    __shared__ int wave_count[FILL_WAVES];
     if (plan->status != 0) {            // keep the gather in range: every grouped row reads token 0
-        for (int p = blockIdx.x * 256 + threadIdx.x; p < pairs; p += gridDim.x * 256) row_pairs[p] = 0;
+        for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < pairs; p += gridDim.x * blockDim.x) row_pairs[p] = 0;
         return;
     }
-    const int lane = threadIdx.x & 63;
-    const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (e >= n_experts) return;         // uniform per wave
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int e = blockIdx.x;
+    if (e >= n_experts || offsets[e + 1] == offsets[e]) return;           // uniform over the workgroup
+    const int chunks = (pairs + 63) / 64;
+    const int per_wave = (chunks + FILL_WAVES - 1) / FILL_WAVES;
+    const int first_chunk = wave * per_wave;
+    const int last_chunk = first_chunk + per_wave < chunks ? first_chunk + per_wave : chunks;
+    int mine = 0;
+    for (int c = first_chunk; c < last_chunk; ++c) {
+        const int p = c * 64 + lane;
+        mine += __popcll(__ballot(p < pairs && selected[p] == e));
+    }
+    if (lane == 0) wave_count[wave] = mine;
+    __syncthreads();
     int at = offsets[e];
-    if (offsets[e + 1] == at) return;
-    for (int first = 0; first < pairs; first += 64) {
-        const int p = first + lane;
+    for (int w = 0; w < wave; ++w) at += wave_count[w];
+    for (int c = first_chunk; c < last_chunk; ++c) {
+        const int p = c * 64 + lane;
         const bool hit = p < pairs && selected[p] == e;
         const unsigned long long mask = __ballot(hit);
         if (hit) {
@@ -260,7 +275,7 @@ int moe_prefill_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_
     a.gate = w.gate; a.up = w.up; a.down = w.down;
     hipLaunchKernelGGL(group_scan_kernel, dim3(1), dim3(MAX_EXPERTS), 0, stream, a);
     int *rp = row_pairs ? row_pairs : w.row_pairs;
-    hipLaunchKernelGGL(group_fill_kernel, dim3((g.n_experts + 3) / 4), dim3(256), 0, stream, selected, rows, g.topk,
+    hipLaunchKernelGGL(group_fill_kernel, dim3(g.n_experts), dim3(FILL_WAVES * 64), 0, stream, selected, rows, g.topk,
                        w.offsets, g.n_experts, w.plan, rp, w.pair_rows);
     if (hipGetLastError() != hipSuccess) return -1;
 
