@@ -113,7 +113,13 @@ typedef struct SaltGpuWeightResourceUsage {       /* reference gpu.h:418-429 */
 
 /* reference gpu.h:450-460, 465-469, 480.  describe records a host range;
  * activate (AUTO or REGISTERED_PERSISTENT) copies it to HBM once;
- * BOUNDED_WINDOW copies only the windows later bound; PAGEABLE is refused. */
+ * BOUNDED_WINDOW copies only the windows later bound; PAGEABLE is refused.
+ * pool_bind (reference gpu_hip.cpp:4208-4217) turns an active, window-addressed
+ * resource with nothing bound into a component pool: only the byte ranges its
+ * registered tensors occupy become resident (merged, 4096-byte granules of the
+ * resource offset), either as the permanent spans of the residency arena or,
+ * when the engine runs no arena, in HBM allocations made at the next
+ * salt_gpu_sync.  A pool that is laid out or resident no longer grows. */
 int salt_gpu_weight_resource_describe(uint32_t kind, uint32_t resource_id, const void *base, size_t nbytes);
 int salt_gpu_weight_resource_activate(uint32_t kind, uint32_t resource_id, SaltGpuWeightAddressability policy);
 int salt_gpu_weight_resource_pool_bind(uint32_t kind, uint32_t resource_id);
@@ -283,8 +289,12 @@ typedef struct SaltGpuResidencyPermanentSpan {
  * read callback, copy staging -> seat asynchronously (populate), report
  * completion (poll), translate offsets to device addresses (resolve), drain a
  * seat before reuse (retire), and tear down (destroy).  The permanent_* ops
- * enumerate and copy backend-chosen process-lifetime spans; this backend keeps
- * whole resources resident through activate(), so it reports no spans. */
+ * (reference gpu_hip.cpp:3429-3571) enumerate the regions of the component pool
+ * as spans at 256-byte aligned offsets in front of the seats, give the engine a
+ * read callback for each, copy its staged chunks in order (permanent_copy is
+ * complete on return) and, once every span is full, make the tensors inside
+ * resolvable (permanent_publish).  Without a pool-bound resource that holds
+ * tensors permanent_layout returns -1; destroy takes the spans with the arena. */
 typedef struct SaltGpuResidencyBackendOps {
     uint32_t abi_version;
     size_t ops_size;

@@ -17,6 +17,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <unordered_map>
 #include <vector>
 
@@ -42,6 +43,21 @@ struct Resource {
     uint64_t window_offset = 0;       // bounded-window policy: the one bound window
     size_t window_bytes = 0;
     uint8_t *window_device = nullptr;
+    int pool = 0;                     // pool-bound: only the bytes its tensors occupy become resident
+};
+
+// One merged byte range of a pool-bound resource that registered tensors occupy
+// (reference gpu_hip.cpp:3212-3340).  It is resident either inside the residency
+// arena (a permanent span) or in an allocation of its own.
+struct Region {
+    int resource = -1;
+    const uint8_t *host = nullptr;
+    size_t nbytes = 0;
+    uint64_t source_offset = 0;       // of `host` inside the resource
+    uint64_t arena_offset = 0;        // inside the residency arena, once laid out
+    size_t populated = 0;             // bytes of the span copied so far
+    uint8_t *device = nullptr;        // set when the range is readable by kernels
+    uint8_t *owned = nullptr;         // allocation of its own (no residency arena)
 };
 
 struct Tensor {
@@ -73,6 +89,7 @@ struct Residency {
     std::vector<hipEvent_t> events;
     std::vector<uint64_t> slot_ticket, staging_ticket;
     std::vector<uint32_t> slot_staging;
+    int published = 0;                // the permanent spans are populated and resolvable
 };
 
 struct Engine {
@@ -93,6 +110,12 @@ struct Engine {
     size_t legacy_capacity = 0, legacy_used = 0;
     std::vector<Pending> pending;
     Residency residency;
+    // component pool
+    std::vector<Region> regions;      // sorted by (resource, source offset) once built
+    int pool_final = 0;               // regions are resident; the set no longer grows
+    uint64_t pool_bytes = 0, pool_peak_bytes = 0;
+    uint64_t pool_layout_bytes = 0, pool_layout_max_span = 0;     // permanent-span layout handed to the engine
+    uint32_t pool_span_count = 0;
 };
 
 Engine g_engine;
@@ -187,6 +210,8 @@ const uint8_t *resident_address(const void *host, size_t nbytes) {
         if (r.window_device && inside(r.host + r.window_offset, r.window_bytes, host, nbytes))
             return r.window_device + ((const uint8_t *)host - (r.host + r.window_offset));
     }
+    for (const Region &g : g_engine.regions)
+        if (g.device && inside(g.host, g.nbytes, host, nbytes)) return g.device + ((const uint8_t *)host - g.host);
     for (const Seat &s : g_engine.seats)
         if (s.active && inside(s.payload, s.nbytes - (size_t)(s.payload - s.host_base), host, nbytes))
             return s.device + ((const uint8_t *)host - s.payload);
@@ -200,9 +225,13 @@ void forget_tensors_of(int resource_index) {
         it = it->second.resource == resource_index ? g_engine.tensors.erase(it) : ++it;
 }
 
+int pool_release_resource(int resource_index);
+int pool_finalize();
+
 int release_resource_memory(Resource &r) {
     int failed = 0;
-    if (r.device || r.window_device) failed |= drain_device();      // no reader may outlive the range
+    if (r.device || r.window_device || r.pool) failed |= drain_device();      // no reader may outlive the range
+    if (r.pool) failed |= pool_release_resource((int)(&r - g_engine.resources.data()));
     if (r.device) { failed |= hip_ok(hipFree(r.device), "hipFree resource"); g_engine.device_copied_bytes -= r.nbytes; }
     if (r.window_device) failed |= hip_ok(hipFree(r.window_device), "hipFree window");
     r.device = r.window_device = nullptr;
@@ -218,6 +247,126 @@ struct Q4Weights { const uint8_t *vals, *scales, *biases; };
 size_t q4_vals_bytes(int R, int C) { return ((size_t)R * C + 7) / 8 * 4; }
 size_t q8_vals_bytes(int R, int C) { return ((size_t)R * C + 3) / 4 * 4; }
 size_t q4_meta_bytes(int R, int C) { return ((size_t)R * C + 63) / 64 * 2; }
+
+// ---- component pool -----------------------------------------------------------
+//
+// A resource that is pool-bound (reference gpu_hip.cpp:4208-4217) is not copied whole: only the byte ranges its
+// registered tensors occupy become resident, merged into few regions.  The reference pins those host ranges; here
+// they are copied to HBM, either into the residency arena as permanent spans (when the engine runs one) or into
+// allocations of their own at the first salt_gpu_sync.
+
+constexpr uint64_t POOL_GRANULE = 4096;     // a region starts on this multiple of the resource offset, so a tensor
+                                            // keeps its alignment below the granule when it moves to the device
+constexpr uint64_t POOL_ALIGN = 256;        // of a region inside the residency arena
+
+void tensor_bytes(const Tensor &t, size_t *value_bytes, size_t *scale_bytes) {
+    const size_t elements = (size_t)t.R * (size_t)t.C;
+    if (t.bits == 4) { *value_bytes = q4_vals_bytes(t.R, t.C); *scale_bytes = q4_meta_bytes(t.R, t.C); }
+    else if (t.bits == 8) { *value_bytes = q8_vals_bytes(t.R, t.C); *scale_bytes = q4_meta_bytes(t.R, t.C); }
+    else if (t.bits == 16) { *value_bytes = elements * 2; *scale_bytes = 0; }
+    else { *value_bytes = elements / 2; *scale_bytes = elements / 16; }
+}
+
+int pool_add_range(int ri, const uint8_t *p, size_t nbytes) {
+    Engine &e = g_engine;
+    const Resource &r = e.resources[(size_t)ri];
+    if (!p || nbytes < 1 || !inside(r.host, r.nbytes, p, nbytes)) return -1;
+    uint64_t first = (uint64_t)(p - r.host), last = first + nbytes;
+    first -= first % POOL_GRANULE;
+    last = (last + POOL_GRANULE - 1) / POOL_GRANULE * POOL_GRANULE;
+    if (last > r.nbytes) last = r.nbytes;
+    for (size_t i = 0; i < e.regions.size();) {              // merge with every range it overlaps or touches
+        const Region &g = e.regions[i];
+        const uint64_t g0 = g.source_offset, g1 = g0 + g.nbytes;
+        if (g.resource != ri || last < g0 || g1 < first) { ++i; continue; }
+        if (g0 < first) first = g0;
+        if (g1 > last) last = g1;
+        e.regions.erase(e.regions.begin() + (long)i);
+        i = 0;
+    }
+    Region g;
+    g.resource = ri; g.host = r.host + first; g.nbytes = (size_t)(last - first); g.source_offset = first;
+    e.regions.push_back(g);
+    return 0;
+}
+
+bool pool_resources_present() {
+    for (const Resource &r : g_engine.resources)
+        if (r.kind <= KIND_MAX && r.active && r.pool) return true;
+    return false;
+}
+
+// Builds the regions from the tensors registered so far.  -1 when the pool is already resident or holds no tensor.
+int pool_build_regions() {
+    Engine &e = g_engine;
+    if (e.pool_final) return -1;
+    if (!e.regions.empty()) return 0;
+    for (const auto &entry : e.tensors) {
+        const Tensor &t = entry.second;
+        if (t.resource < 0 || !e.resources[(size_t)t.resource].pool) continue;
+        size_t vb = 0, mb = 0;
+        tensor_bytes(t, &vb, &mb);
+        if (pool_add_range(t.resource, t.vals, vb) != 0 || (t.scales && mb && pool_add_range(t.resource, t.scales, mb) != 0) ||
+            (t.biases && mb && pool_add_range(t.resource, t.biases, mb) != 0)) {
+            e.regions.clear();
+            return -1;
+        }
+    }
+    std::sort(e.regions.begin(), e.regions.end(), [](const Region &a, const Region &b) {
+        return a.resource != b.resource ? a.resource < b.resource : a.source_offset < b.source_offset;
+    });
+    return e.regions.empty() ? -1 : 0;
+}
+
+bool pool_covers(const void *p, size_t nbytes) {
+    for (const Region &g : g_engine.regions)
+        if (inside(g.host, g.nbytes, p, nbytes)) return true;
+    return false;
+}
+
+// Without a residency arena the regions get allocations of their own (the counterpart of the reference pinning
+// them at its first sync, gpu_hip.cpp:3573-3640 and 6917-6920).  A pool that holds no tensor yet is left alone.
+int pool_finalize() {
+    Engine &e = g_engine;
+    if (e.pool_final || !pool_resources_present()) return 0;
+    if (e.pool_span_count != 0) return 0;                    // laid out as permanent spans: the engine populates them
+    if (pool_build_regions() != 0) return 0;
+    uint64_t total = 0;
+    for (Region &g : e.regions) {
+        if (hip_ok(hipMalloc((void **)&g.owned, g.nbytes), "hipMalloc component pool") != 0) { g.owned = nullptr; total = UINT64_MAX; break; }
+        if (hip_ok(hipMemcpy(g.owned, g.host, g.nbytes, hipMemcpyHostToDevice), "component pool upload") != 0) { total = UINT64_MAX; break; }
+        g.device = g.owned;
+        total += g.nbytes;
+    }
+    if (total == UINT64_MAX) {
+        for (Region &g : e.regions) if (g.owned) (void)hipFree(g.owned);
+        e.regions.clear();
+        return -1;
+    }
+    e.pool_bytes = total;
+    if (total > e.pool_peak_bytes) e.pool_peak_bytes = total;
+    e.device_copied_bytes += total;
+    e.pool_final = 1;
+    return 0;
+}
+
+// Drops the regions of one resource (reference gpu_hip.cpp:3642-3684); the caller has drained the device.
+int pool_release_resource(int ri) {
+    Engine &e = g_engine;
+    int failed = 0;
+    for (size_t i = 0; i < e.regions.size();) {
+        Region &g = e.regions[i];
+        if (g.resource != ri) { ++i; continue; }
+        if (g.owned) { failed |= hip_ok(hipFree(g.owned), "hipFree component pool"); e.device_copied_bytes -= g.nbytes; }
+        e.regions.erase(e.regions.begin() + (long)i);
+    }
+    uint64_t total = 0;
+    for (const Region &g : e.regions) if (g.device) total += g.nbytes;
+    e.pool_bytes = total;
+    if (e.regions.empty()) e.pool_final = 0;
+    e.resources[(size_t)ri].pool = 0;
+    return failed ? -1 : 0;
+}
 
 int legacy_reserve(size_t nbytes) {
     Engine &e = g_engine;
@@ -313,6 +462,19 @@ int register_tensor(uint32_t kind, uint32_t id, const void *key, const void *val
                           old.biases == proto.biases && old.bits == proto.bits && old.R == proto.R && old.C == proto.C;
         if (!same) { set_error("tensor slot: key is already bound to a different tensor"); return -1; }
         return 0;
+    }
+    if (r.pool) {
+        // a pool that is laid out or resident no longer grows: the tensor must lie inside what it already holds
+        size_t vb = 0, mb = 0;
+        tensor_bytes(proto, &vb, &mb);
+        if (g_engine.pool_final || g_engine.pool_span_count != 0) {
+            if (!pool_covers(vals, vb) || (scales && mb && !pool_covers(scales, mb)) || (biases && mb && !pool_covers(biases, mb))) {
+                set_error("tensor slot: the component pool of resource (%u, %u) is already laid out without these bytes", kind, id);
+                return -1;
+            }
+        } else {
+            g_engine.regions.clear();                     // rebuilt from all tensors when next needed
+        }
     }
     g_engine.tensors.emplace(key, proto);
     return 0;
@@ -433,6 +595,7 @@ int salt_gpu_set_defer(int on) {
 int salt_gpu_sync(void) {
     Engine &e = g_engine;
     if (!g_state.ready) return e.pending.empty() ? 0 : -1;
+    if (pool_finalize() != 0) return -1;
     const int rc = hip_ok(hipStreamSynchronize(g_state.stream), "hipStreamSynchronize");
     if (rc == 0)
         for (const Pending &p : e.pending) memcpy(p.host, p.staged, p.nbytes);
@@ -509,7 +672,18 @@ int salt_gpu_weight_resource_activate(uint32_t kind, uint32_t resource_id, SaltG
 }
 
 int salt_gpu_weight_resource_pool_bind(uint32_t kind, uint32_t resource_id) {
-    return salt_gpu_weight_resource_activate(kind, resource_id, SALT_GPU_WEIGHT_ADDRESS_AUTO);
+    if (ready_or_fail("weight_resource_pool_bind") != 0) return -1;
+    const int ri = find_resource(kind, resource_id);
+    if (ri < 0) { set_error("pool bind: resource (%u, %u) was never described", kind, resource_id); return -1; }
+    Resource &r = g_engine.resources[(size_t)ri];
+    if (!r.active || r.device || r.window_device || r.policy != SALT_GPU_WEIGHT_ADDRESS_BOUNDED_WINDOW || r.pool ||
+        g_engine.pool_final || g_engine.pool_span_count != 0) {
+        set_error("pool bind: the resource must be active and window-addressed with nothing bound, and the pool not yet resident");
+        return -1;
+    }
+    r.pool = 1;
+    g_engine.regions.clear();
+    return 0;
 }
 
 int salt_gpu_weight_resource_deactivate(uint32_t kind, uint32_t resource_id) {
@@ -543,9 +717,9 @@ int salt_gpu_weight_window_bind(uint32_t kind, uint32_t resource_id, uint64_t of
     const int ri = find_resource(kind, resource_id);
     if (ri < 0) return -1;
     Resource &r = g_engine.resources[(size_t)ri];
-    if (!r.active || r.policy != SALT_GPU_WEIGHT_ADDRESS_BOUNDED_WINDOW || r.window_device || nbytes < 1 ||
+    if (!r.active || r.policy != SALT_GPU_WEIGHT_ADDRESS_BOUNDED_WINDOW || r.window_device || r.pool || nbytes < 1 ||
         offset > r.nbytes || nbytes > r.nbytes - offset) {
-        set_error("window bind: resource is not window-addressed, a window is already bound, or the range is bad");
+        set_error("window bind: resource is not window-addressed, is pool-bound, a window is already bound, or the range is bad");
         return -1;
     }
     if (hip_ok(hipMalloc((void **)&r.window_device, nbytes), "hipMalloc window") != 0) { r.window_device = nullptr; return -1; }
@@ -582,9 +756,13 @@ int salt_gpu_weight_resource_usage(SaltGpuWeightResourceUsage *usage, size_t usa
         usage->active_resources++;
         if (r.device) usage->registered_bytes += r.nbytes;
         if (r.window_device) { usage->active_window_bytes += r.window_bytes; usage->active_windows++; }
+        if (r.pool) usage->active_windows++;              // reference gpu_hip.cpp:4258-4272
     }
-    usage->peak_window_bytes = g_engine.peak_window_bytes;
+    usage->peak_window_bytes = g_engine.peak_window_bytes > g_engine.pool_peak_bytes ? g_engine.peak_window_bytes
+                                                                                     : g_engine.pool_peak_bytes;
     usage->device_copied_weight_bytes = g_engine.device_copied_bytes;
+    if (g_engine.residency.published) usage->device_copied_weight_bytes += g_engine.pool_bytes;
+    else usage->active_window_bytes += g_engine.pool_bytes;
     return 0;
 }
 
@@ -1544,6 +1722,13 @@ static int res_destroy(void *) {
     int failed = drain_device();
     for (Seat &s : g_engine.seats)
         if (s.active && s.resident) { g_engine.logical_seat[(size_t)s.logical_id] = -1; s = Seat(); }
+    if (r.published) {                                       // the spans leave with the arena (reference gpu_hip.cpp:750-769)
+        for (Region &g : g_engine.regions) { g.device = nullptr; g.arena_offset = 0; g.populated = 0; }
+        g_engine.pool_bytes = 0;
+        g_engine.pool_final = 0;
+    }
+    g_engine.pool_layout_bytes = g_engine.pool_layout_max_span = 0;
+    g_engine.pool_span_count = 0;
     for (hipEvent_t ev : r.events) if (ev) failed |= hip_ok(hipEventDestroy(ev), "hipEventDestroy");
     if (r.stream) failed |= hip_ok(hipStreamDestroy(r.stream), "hipStreamDestroy");
     if (r.staging) failed |= hip_ok(hipHostFree(r.staging), "hipHostFree");
@@ -1552,15 +1737,105 @@ static int res_destroy(void *) {
     return failed ? -1 : 0;
 }
 
-static int res_permanent_layout(void *, SaltGpuResidencyPermanentLayout *layout, size_t layout_size) {
-    if (!layout || layout_size != sizeof *layout) return -1;
-    memset(layout, 0, sizeof *layout);
-    layout->alignment = 256;
+// Permanent spans: the regions of the component pool, laid out at the front of the arena (reference
+// gpu_hip.cpp:3429-3571).  The engine reads each span through the callback below into a staging slot and has it
+// copied chunk by chunk; publish makes the tensors inside resolvable.
+static int pool_source_read(void *context, uint64_t source_offset, void *destination, size_t nbytes) {
+    const size_t index = (size_t)(uintptr_t)context - 1;          // the span index travels in the pointer
+    if (!context || index >= g_engine.regions.size() || !destination || nbytes == 0) return -1;
+    const Region &g = g_engine.regions[index];
+    if (!g.host || source_offset < g.source_offset) return -1;
+    const uint64_t local = source_offset - g.source_offset;
+    if (local > g.nbytes || nbytes > g.nbytes - local) return -1;
+    memcpy(destination, g.host + local, nbytes);
     return 0;
 }
-static int res_permanent_span(void *, uint32_t, SaltGpuResidencyPermanentSpan *, size_t) { return -1; }
-static int res_permanent_copy(void *, uint32_t, uint64_t, uint32_t, size_t, uint64_t) { return -1; }
-static int res_permanent_publish(void *) { return g_engine.residency.ready ? 0 : -1; }
+
+static int res_permanent_layout(void *, SaltGpuResidencyPermanentLayout *layout, size_t layout_size) {
+    Engine &e = g_engine;
+    if (!g_state.ready || !layout || layout_size != sizeof *layout || e.pool_final) return -1;
+    if (e.pool_span_count == 0) {
+        if (pool_build_regions() != 0) {
+            set_error("permanent layout: no tensor is registered in a pool-bound resource");
+            return -1;
+        }
+        uint64_t cursor = 0, maximum = 0;
+        for (Region &g : e.regions) {
+            cursor = (cursor + POOL_ALIGN - 1) / POOL_ALIGN * POOL_ALIGN;
+            g.arena_offset = cursor;
+            g.populated = 0;
+            g.device = nullptr;
+            cursor += g.nbytes;
+            if (g.nbytes > maximum) maximum = g.nbytes;
+        }
+        e.pool_layout_bytes = cursor;
+        e.pool_layout_max_span = maximum;
+        e.pool_span_count = (uint32_t)e.regions.size();
+    }
+    layout->permanent_bytes = e.pool_layout_bytes;
+    layout->maximum_span_bytes = e.pool_layout_max_span;
+    layout->span_count = e.pool_span_count;
+    layout->alignment = (uint32_t)POOL_ALIGN;
+    return 0;
+}
+
+static int res_permanent_span(void *, uint32_t span_index, SaltGpuResidencyPermanentSpan *span, size_t span_size) {
+    Engine &e = g_engine;
+    if (!span || span_size != sizeof *span || span_index >= e.pool_span_count || span_index >= e.regions.size()) return -1;
+    const Region &g = e.regions[span_index];
+    if (g.resource < 0 || (size_t)g.resource >= e.resources.size()) return -1;
+    const Resource &r = e.resources[(size_t)g.resource];
+    if (!r.active || !r.pool) return -1;
+    memset(span, 0, sizeof *span);
+    span->source.resource.kind = r.kind;
+    span->source.resource.resource_id = r.id;
+    span->source.source_offset = g.source_offset;
+    span->source.nbytes = g.nbytes;
+    span->source.read = pool_source_read;
+    span->source.read_context = (void *)(uintptr_t)(span_index + 1u);
+    span->device_offset = g.arena_offset;
+    return 0;
+}
+
+static int res_permanent_copy(void *, uint32_t span_index, uint64_t device_offset, uint32_t staging_slot, size_t nbytes,
+                              uint64_t ticket) {
+    Engine &e = g_engine;
+    Residency &r = e.residency;
+    if (!r.ready || r.poisoned || r.published || ticket == 0 || nbytes == 0 || span_index >= e.pool_span_count ||
+        span_index >= e.regions.size() || staging_slot >= r.plan.staging_count || nbytes > r.plan.staging_bytes)
+        return -1;
+    Region &g = e.regions[span_index];
+    if (device_offset != g.arena_offset + g.populated || nbytes > g.nbytes - g.populated ||
+        device_offset > r.plan.permanent_bytes || nbytes > r.plan.permanent_bytes - device_offset) {
+        set_error("permanent copy: chunks of a span arrive in order and stay inside the permanent part of the arena");
+        return -1;
+    }
+    if (hip_ok(hipMemcpyAsync(r.arena + device_offset, r.staging + (size_t)staging_slot * r.plan.staging_bytes, nbytes,
+                              hipMemcpyHostToDevice, r.stream), "permanent span copy") != 0)
+        return -1;
+    if (hip_ok(hipStreamSynchronize(r.stream), "permanent span copy") != 0) { r.poisoned = 1; return -1; }
+    g.populated += nbytes;                                   // the staging slot is free again on return
+    return 0;
+}
+
+static int res_permanent_publish(void *) {
+    Engine &e = g_engine;
+    Residency &r = e.residency;
+    if (!r.ready || r.poisoned || r.published || e.pool_span_count == 0 || e.pool_span_count != e.regions.size()) return -1;
+    uint64_t total = 0;
+    for (const Region &g : e.regions)
+        if (g.populated != g.nbytes || g.arena_offset > r.plan.permanent_bytes ||
+            g.nbytes > r.plan.permanent_bytes - g.arena_offset) {
+            set_error("permanent publish: a span is not fully populated");
+            return -1;
+        }
+    for (Region &g : e.regions) { g.device = r.arena + g.arena_offset; total += g.nbytes; }
+    e.pool_bytes = total;
+    if (total > e.pool_peak_bytes) e.pool_peak_bytes = total;
+    e.pool_final = 1;
+    r.published = 1;
+    return 0;
+}
 
 static const SaltGpuResidencyBackendOps residency_ops = {
     SALT_GPU_RESIDENCY_ABI_VERSION, sizeof(SaltGpuResidencyBackendOps),

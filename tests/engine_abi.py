@@ -57,6 +57,15 @@ class PermanentLayout(C.Structure):
     _fields_ = [("permanent_bytes", u64), ("maximum_span_bytes", u64), ("span_count", u32), ("alignment", u32)]
 
 
+RESIDENCY_READ = C.CFUNCTYPE(i32, vp, u64, vp, sz)
+
+
+class PermanentSpan(C.Structure):      # reference gpu_residency.h:40-62
+    _fields_ = [("kind", u32), ("resource_id", u32), ("value_offset", u64), ("scale_offset", u64), ("bias_offset", u64),
+                ("logical_resource_id", u64), ("source_offset", u64), ("nbytes", u64), ("read", RESIDENCY_READ),
+                ("read_context", vp), ("device_offset", u64)]
+
+
 class ResidencyOps(C.Structure):
     _fields_ = [("abi_version", u32), ("ops_size", sz),
                 ("create", C.CFUNCTYPE(i32, vp, C.POINTER(ResidencyPlan))),
@@ -67,7 +76,7 @@ class ResidencyOps(C.Structure):
                 ("retire", C.CFUNCTYPE(i32, vp, u32, u64)),
                 ("destroy", C.CFUNCTYPE(i32, vp)),
                 ("permanent_layout", C.CFUNCTYPE(i32, vp, C.POINTER(PermanentLayout), sz)),
-                ("permanent_span", C.CFUNCTYPE(i32, vp, u32, vp, sz)),
+                ("permanent_span", C.CFUNCTYPE(i32, vp, u32, C.POINTER(PermanentSpan), sz)),
                 ("permanent_copy", C.CFUNCTYPE(i32, vp, u32, u64, u32, sz, u64)),
                 ("permanent_publish", C.CFUNCTYPE(i32, vp))]
 

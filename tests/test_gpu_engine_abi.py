@@ -290,7 +290,7 @@ def test_expert_seats_through_residency_and_selected_chain(eng, oracle, pkg):
     assert ops.create(None, C.byref(plan)) == -1                      # one arena at a time
     assert eng.salt_gpu_free() == -1                                  # refused while residency is live
     layout = abi.PermanentLayout()
-    assert ops.permanent_layout(None, C.byref(layout), C.sizeof(layout)) == 0 and layout.span_count == 0
+    assert ops.permanent_layout(None, C.byref(layout), C.sizeof(layout)) == -1     # no pool-bound resource: no spans
     assert eng.salt_gpu_selected_resources_prepare(seats, 30 * 128) == 0
     assert eng.salt_gpu_selected_resources_prepare(seats, 30 * 128) == 0
     assert eng.salt_gpu_selected_resources_prepare(seats + 1, 30 * 128) == -1
@@ -405,6 +405,109 @@ def test_expert_seats_through_residency_and_selected_chain(eng, oracle, pkg):
         assert eng.salt_gpu_shared_buffer_free(C.byref(b)) == 0 and not b.contents
     assert ops.destroy(None) == 0
     assert ops.destroy(None) == -1
+
+
+def test_component_pool_without_and_with_permanent_spans(eng, oracle, pkg):
+    """A pool-bound resource (reference gpu_hip.cpp:4208-4217): only the bytes its tensors occupy become resident,
+    at the first sync when no residency arena runs, as permanent spans of the arena when one does
+    (reference gpu_hip.cpp:3429-3571, gpu_residency.c:334-406)."""
+    shapes = [(128, 256), (64, 256), (96, 512)]
+    trunk = Trunk(shapes, 61)
+    gap = 3 * 4096 + 40                                   # unrelated bytes ahead of the tensors and between two of them
+    first = trunk.views[2][2][0]                          # offset of the third tensor: the gap goes in front of it
+    image = np.concatenate([np.full(gap, 0xA5, np.uint8), trunk.blob[:first], np.full(5 * 4096, 0x5A, np.uint8),
+                            trunk.blob[first:]])
+    def pointers(k):
+        offs = trunk.views[k][2]
+        return [image.ctypes.data + gap + o + (5 * 4096 if k == 2 else 0) for o in offs]
+    TR = 7
+    assert eng.salt_gpu_weight_resource_describe(TRUNK, TR, image.ctypes.data, image.nbytes) == 0
+    assert eng.salt_gpu_weight_resource_pool_bind(TRUNK, TR) == -1                  # not active
+    assert eng.salt_gpu_weight_resource_activate(TRUNK, TR, 1) == 0
+    assert eng.salt_gpu_weight_resource_pool_bind(TRUNK, TR) == 0, err(pkg)
+    assert eng.salt_gpu_weight_resource_pool_bind(TRUNK, TR) == -1                  # once
+    assert eng.salt_gpu_weight_window_bind(TRUNK, TR, 0, 4096) == -1                # no windows into a pool
+    for k, (R, Cc) in enumerate(shapes):
+        v, s, b = pointers(k)
+        assert eng.salt_gpu_weight_resource_slot(TRUNK, TR, v, v, s, b, 4, R, Cc) == 0, err(pkg)
+    eng.salt_gpu_set_mapped_only(1)
+
+    def check_all():
+        for k, (R, Cc) in enumerate(shapes):
+            v, s, b = pointers(k)
+            x = synth.activations(Cc, 1, 70 + k)[0]; y = np.zeros(R, np.float32)
+            assert eng.salt_gpu_q4_matvec(v, s, b, R, Cc, ptr(x), ptr(y)) == 0, err(pkg)
+            assert np.array_equal(bits(y), bits(q4_want(oracle, *trunk.views[k][3:], R, Cc, x)[0]))
+
+    # 1. no arena: resident from the first sync on
+    v, s, b = pointers(0)
+    x = synth.activations(256, 1, 1)[0]; y = np.zeros(128, np.float32)
+    assert eng.salt_gpu_q4_matvec(v, s, b, 128, 256, ptr(x), ptr(y)) == -1          # nothing resident before the sync
+    assert eng.salt_gpu_sync() == 0, err(pkg)
+    check_all()
+    usage = abi.ResourceUsage()
+    assert eng.salt_gpu_weight_resource_usage(C.byref(usage), C.sizeof(usage)) == 0
+    tensor_bytes = sum(a.nbytes for view in trunk.views for a in view[3:])
+    assert usage.active_windows >= 1 and tensor_bytes <= usage.active_window_bytes < image.nbytes - 4 * 4096
+    # a tensor registered after the pool became resident must lie inside it
+    assert eng.salt_gpu_weight_resource_slot(TRUNK, TR, image.ctypes.data + gap + first + 4096,
+                                             image.ctypes.data + gap + first + 4096, image.ctypes.data + gap + first + 8192,
+                                             image.ctypes.data + gap + first + 8192 + 64, 4, 8, 64) == -1
+    assert eng.salt_gpu_weight_resource_deactivate(TRUNK, TR) == 0
+    assert eng.salt_gpu_q4_matvec(v, s, b, 128, 256, ptr(x), ptr(y)) == -1
+
+    # 2. with an arena: the same regions as permanent spans, copied through staging in chunks
+    assert eng.salt_gpu_weight_resource_activate(TRUNK, TR, 1) == 0
+    assert eng.salt_gpu_weight_resource_pool_bind(TRUNK, TR) == 0, err(pkg)
+    ops = eng.salt_gpu_residency_backend_ops().contents
+    layout = abi.PermanentLayout()
+    assert ops.permanent_layout(None, C.byref(layout), C.sizeof(layout)) == 0, err(pkg)
+    assert layout.span_count == 2 and layout.alignment == 256
+    assert layout.maximum_span_bytes <= layout.permanent_bytes < image.nbytes - 4 * 4096
+    assert eng.salt_gpu_weight_resource_pool_bind(TRUNK, TR) == -1
+    staging_bytes, seat_bytes = 16384, 8192
+    base = (layout.permanent_bytes + 255) // 256 * 256
+    plan = abi.ResidencyPlan(base + 2 * seat_bytes, layout.permanent_bytes, base, seat_bytes, staging_bytes, 2, 2, 256, 0)
+    assert ops.create(None, C.byref(plan)) == 0, err(pkg)
+    assert eng.salt_gpu_sync() == 0                                                 # does not make the pool resident by itself
+    assert eng.salt_gpu_q4_matvec(v, s, b, 128, 256, ptr(x), ptr(y)) == -1
+    assert ops.permanent_publish(None) == -1                                        # nothing populated yet
+    ticket = 0
+    previous_end = 0
+    for index in range(layout.span_count):
+        span = abi.PermanentSpan()
+        assert ops.permanent_span(None, index, C.byref(span), C.sizeof(span)) == 0
+        assert span.kind == TRUNK and span.resource_id == TR and span.device_offset % 256 == 0
+        assert span.device_offset >= previous_end and span.source_offset % 4096 == 0
+        previous_end = span.device_offset + span.nbytes
+        done = 0
+        while done < span.nbytes:
+            st = ticket % 2
+            address, capacity = C.c_void_p(), C.c_size_t()
+            assert ops.staging(None, st, C.byref(address), C.byref(capacity)) == 0 and capacity.value == staging_bytes
+            chunk = min(capacity.value, span.nbytes - done)
+            assert span.read(span.read_context, span.source_offset + done, address, chunk) == 0
+            assert span.read(span.read_context, span.source_offset + span.nbytes, address, 1) == -1
+            ticket += 1
+            if done == 0:
+                assert ops.permanent_copy(None, index, span.device_offset + 256, st, chunk, ticket) == -1   # out of order
+                assert ops.permanent_copy(None, index, span.device_offset, st, chunk, 0) == -1             # ticket 0
+            assert ops.permanent_copy(None, index, span.device_offset + done, st, chunk, ticket) == 0, err(pkg)
+            done += chunk
+            if index == 0 and done >= span.nbytes:
+                assert ops.permanent_publish(None) == -1                            # the second span is still empty
+    span = abi.PermanentSpan()
+    assert ops.permanent_span(None, layout.span_count, C.byref(span), C.sizeof(span)) == -1
+    assert ops.permanent_publish(None) == 0, err(pkg)
+    assert ops.permanent_publish(None) == -1
+    assert ops.permanent_layout(None, C.byref(layout), C.sizeof(layout)) == -1      # resident: the layout is closed
+    check_all()
+    assert eng.salt_gpu_weight_resource_usage(C.byref(usage), C.sizeof(usage)) == 0
+    assert usage.device_copied_weight_bytes >= tensor_bytes and usage.active_window_bytes == 0
+    assert ops.destroy(None) == 0
+    assert eng.salt_gpu_q4_matvec(v, s, b, 128, 256, ptr(x), ptr(y)) == -1          # the spans left with the arena
+    assert eng.salt_gpu_weight_resource_unbind(TRUNK, TR) == 0
+    eng.salt_gpu_set_mapped_only(0)
 
 
 def test_nvfp4_engine_entry_points(eng, oracle, pkg):
