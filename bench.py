@@ -333,6 +333,30 @@ def main():
                 extra["ffn_block_graph_us"] = round(ms_g * 1e3, 2)
                 lib.salt_mi355_graph_destroy(graph)
         del block, residuals
+        # BASELINE configs[0]: one 4096 x 4096 Q4 matvec per launch, batch 1, rotating through 64 weight instances (606 MB)
+        R = Cc = 4096
+        vals, scales, biases = synth.q4_tensor(R, Cc, 60)
+        G = 64
+        per = vals.nbytes + scales.nbytes + biases.nbytes
+        w0 = gpu.DeviceBuffer(per * G)
+        for g in range(G):
+            w0.upload(vals, g * per)
+            w0.upload(scales, g * per + vals.nbytes)
+            w0.upload(biases, g * per + vals.nbytes + scales.nbytes)
+        x0 = gpu.DeviceBuffer.from_host(synth.activations(Cc, 1, 61))
+        y0 = gpu.DeviceBuffer(R * 4)
+
+        def q4_single_step(s):
+            for g in range(G):
+                at = g * per
+                if lib.salt_mi355_q4_matvec_dev(w0.at(at), w0.at(at + vals.nbytes), w0.at(at + vals.nbytes + scales.nbytes),
+                                                R, Cc, 1, x0.ptr, y0.ptr, 0, s) != 0:
+                    raise RuntimeError(lib.salt_mi355_last_error().decode())
+
+        ms_q0 = timed(lib, stream, events, q4_single_step, 2, 10) / G
+        extra["q4_4096_matvec_us"] = round(ms_q0 * 1e3, 2)
+        extra["q4_4096_matvec_gbps"] = round(synth.q4_bytes(R, Cc, 1) / (ms_q0 * 1e-3) / 1e9, 1)
+        del w0, x0, y0
         # NVFP4 8192 x 8192, batch 1, reference semantics (activation Q/DQ inside the rows' launch), 16 instances
         R = Cc = 8192
         packed, fscales = synth.nvfp4_tensor(R, Cc, 40)

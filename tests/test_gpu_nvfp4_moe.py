@@ -242,6 +242,15 @@ def test_moe_decode_step_fresh_logits_and_rejection(gpu, oracle):
         assert np.array_equal(bits(eo), bits(oeo)) and np.array_equal(bits(y), bits(oy))
     logits = synth.router_logits(E, 1).copy(); logits[3] = np.inf
     assert layer.step(logits, scale, x)[0] == -1
+    # many steps in a row on one workspace, each checked against the sum of its own expert outputs in place order
+    for it in range(40):
+        logits = synth.router_logits(E, 900 + it); x = synth.activations(H, 1, 950 + it)[0]
+        st, sel, w, eo, y = layer.step(logits, scale, x)
+        assert st == 0
+        acc = np.zeros(H, np.float32)
+        for i in range(K):
+            acc = (acc + (eo[i] * w[i]).astype(np.float32)).astype(np.float32)
+        assert np.array_equal(bits(y), bits(acc)), it
 
 
 def test_moe_decode_step_behind_a_pool_file_header(gpu, oracle):
@@ -267,6 +276,7 @@ def test_moe_decode_step_behind_a_pool_file_header(gpu, oracle):
     (520, 4, 128, 64, "more experts than the fused prologue holds: router, gate/up, activate, down, reduce as five launches"),
     (16, 16, 2816, 2048, "more than two tiles per compute unit: eight waves per tile in both fused launches"),
     (24, 5, 192, 4160, "d_ff beyond the LDS activation buffer of the fused down launch: five launches"),
+    (16, 4, 4160, 128, "65 row tiles in the down launch, two tiles in each gate and up projection"),
 ])
 def test_moe_decode_step_other_launch_shapes(gpu, oracle, E, K, H, F, why):
     print(f"moe step E={E} K={K} H={H} F={F}: {why}", flush=True)
