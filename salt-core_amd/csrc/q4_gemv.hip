@@ -68,7 +68,7 @@ static_assert(sizeof(Q4Job) == 56 && offsetof(Q4Job, rows) == 40 && offsetof(Q4J
               "find_job reads a job record as seven 64-bit words");
 
 __device__ __forceinline__ Q4Job find_job(const Q4Launch &L, int tile) {
-    if (L.njobs <= 1) return L.one;
+    if (L.njobs <= 1 && L.table == nullptr) return L.one;     // a table of one job (written on the device) is read like any other
     // 7 words per record, in a device table or inside the kernel arguments (the launch record is the kernel's only
     // argument, so the inline records sit at their offset in the kernarg segment)
     const uniform_u64_ptr words =

@@ -277,6 +277,7 @@ def test_moe_decode_step_behind_a_pool_file_header(gpu, oracle):
     (16, 16, 2816, 2048, "more than two tiles per compute unit: eight waves per tile in both fused launches"),
     (24, 5, 192, 4160, "d_ff beyond the LDS activation buffer of the fused down launch: five launches"),
     (16, 4, 4160, 128, "65 row tiles in the down launch, two tiles in each gate and up projection"),
+    (580, 1, 384, 320, "five launches with a single selected expert: the down launch's table holds one job"),
 ])
 def test_moe_decode_step_other_launch_shapes(gpu, oracle, E, K, H, F, why):
     print(f"moe step E={E} K={K} H={H} F={F}: {why}", flush=True)
