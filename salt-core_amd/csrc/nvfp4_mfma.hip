@@ -199,6 +199,8 @@ int fp4_mfma_splits(int rows, int cols, int tokens) {
     int splits = (512 + tiles - 1) / tiles;            // aim at two workgroups per compute unit
     if (splits > 8) splits = 8;
     if (splits > chunks / 4) splits = chunks / 4;      // at least four chunks per split
+    // with chunks shared out in equal runs the last split must still own one (30 chunks in 7 splits of 5 would not)
+    while (splits > 1 && (splits - 1) * ((chunks + splits - 1) / splits) >= chunks) --splits;
     return splits < 1 ? 1 : splits;
 }
 

@@ -35,7 +35,8 @@ def reference(oracle, packed, scales, divisor, g, R, Cc, xs):
 
 
 @pytest.mark.parametrize("R,Cc,B,g", [(128, 64, 128, 64.0), (192, 256, 37, 8.0), (70, 128, 1, 64.0),
-                                      (512, 2048, 256, 100.0), (1000, 1024, 130, 1.0)])
+                                      (512, 2048, 256, 100.0), (1000, 1024, 130, 1.0),
+                                      (295, 1920, 191, 17.5)])     # 30 column chunks over 6 tiles: an uneven split of K
 def test_matmul_within_stated_tolerance(pkg, oracle, R, Cc, B, g):
     print(f"nvfp4 mfma R={R} C={Cc} B={B}", flush=True)
     packed, scales = synth.nvfp4_tensor(R, Cc, R + Cc + B)
