@@ -407,7 +407,9 @@ __global__ __launch_bounds__(256) void fp4_qdq_kernel(const float *__restrict__ 
 int fp4_launch(const Fp4Launch &L, int chains_per_lane, hipStream_t stream) {
     if (L.total_tiles < 1 || L.tokens < 1 || L.tokens > 4 || L.cols < 32 || (L.cols & 31)) return -1;
     int S = chains_per_lane;
-    if (S == 0) S = L.total_tiles > 512 ? 4 : 2;      // as for the affine-Q4 kernel: sixteen waves per tile up to two tiles per unit
+    // as for the affine-Q4 kernel: sixteen waves per tile up to one tile per compute unit, eight beyond (8192 columns,
+    // one token: 23.9 against 30.2 us at 256 tiles, 42.5 against 36.0 at 320, 48.5 against 43.8 at 512)
+    if (S == 0) S = L.total_tiles > 256 ? 4 : 2;
     switch (S) {
         case 8: return launch_tiles<8>(L, stream);
         case 4: return launch_tiles<4>(L, stream);

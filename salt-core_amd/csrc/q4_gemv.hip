@@ -621,9 +621,11 @@ int q4_moe_gate_up_launch(const Q4Launch &launch, hipStream_t stream) {
     L.table = nullptr; L.njobs = 1; L.cols = m.hidden; L.tokens = 1; L.fused = 0;
     L.total_tiles = 2 * m.topk * ((m.routed + TILE_ROWS - 1) / TILE_ROWS);
     const dim3 grid(L.total_tiles + 1);                         // the extra workgroup publishes the router's outputs
-    if (L.total_tiles <= env_wide_limit())
+    // measured at 176 tiles (eight experts of 704 rows): 1024-column steps 29.4 us per decode step, 512-column steps 29.1,
+    // four chains per lane 30.4 and 33.4; the wide step is kept for launches that leave half the compute units idle
+    if (L.total_tiles <= env_wide_limit() / 2)
         hipLaunchKernelGGL((q4_tile_kernel<2, 1, false, 32, 1>), grid, dim3(1024), 0, stream, L);
-    else if (L.total_tiles <= 512)
+    else if (L.total_tiles <= env_wide_limit())
         hipLaunchKernelGGL((q4_tile_kernel<2, 1, false, 16, 1>), grid, dim3(1024), 0, stream, L);
     else
         hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 16, 1>), grid, dim3(512), 0, stream, L);
@@ -639,10 +641,10 @@ int q4_moe_down_launch(const Q4Launch &launch, hipStream_t stream) {
     L.table = nullptr; L.njobs = 1; L.cols = m.routed; L.tokens = 1; L.fused = 0;
     L.total_tiles = m.topk * ((m.hidden + TILE_ROWS - 1) / TILE_ROWS);
     const dim3 grid(L.total_tiles);
+    // measured at 352 tiles (eight experts of 2816 rows): two chains per lane 31.4 us per decode step, four 29.4,
+    // eight 31.4, wide steps 32.7 and 34.5
     if (L.total_tiles <= env_wide_limit())
         hipLaunchKernelGGL((q4_tile_kernel<2, 1, false, 32, 2>), grid, dim3(1024), 0, stream, L);
-    else if (L.total_tiles <= 512)
-        hipLaunchKernelGGL((q4_tile_kernel<2, 1, false, 16, 2>), grid, dim3(1024), 0, stream, L);
     else
         hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 16, 2>), grid, dim3(512), 0, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
@@ -652,10 +654,10 @@ int q4_launch(const Q4Launch &L, int chains_per_lane, hipStream_t stream) {
     if (L.total_tiles < 1 || L.tokens < 1 || L.tokens > 4 || L.cols < 64 || (L.cols & 63)) return -1;
     int S = chains_per_lane ? chains_per_lane : env_chains();
     if (S == 0) {
-        // Four chains per lane (eight waves per tile) measured fastest once every
-        // compute unit holds three tiles; up to two tiles per unit, sixteen
-        // waves per tile hide more of the LDS and scalar-load latency.
-        S = L.total_tiles > 512 ? 4 : 2;
+        // Up to one tile per compute unit, sixteen waves per tile (two chains per lane) hide more of the LDS and
+        // scalar-load latency; beyond that four chains per lane win (one token, 2816 columns: 12.4 against 15.5 us at
+        // 256 tiles, 20.7 against 15.2 at 320, 23.3 against 17.6 at 512; eight chains per lane never do).
+        S = L.total_tiles > env_wide_limit() ? 4 : 2;
     }
     if (L.fused) {
         switch (S) {
