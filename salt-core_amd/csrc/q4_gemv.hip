@@ -158,8 +158,8 @@ constexpr int x_batch_groups(int S, int NB) {
 // PRO selects a prologue of the MoE decode step (0: none, jobs come from the
 // launch): 1 = router top-k, the workgroup derives its gate or up job from the
 // selection; 2 = the down projection of one selected expert, whose activations
-// gelu_tanh(gate) * up are computed into LDS and reach the VALU through
-// v_readfirstlane instead of scalar loads.
+// gelu_tanh(gate) * up are computed into LDS and reach the VALU in vector
+// registers (every lane reads the same words) instead of through scalar loads.
 template <int S, int NB, bool FUSED, int CB, int PRO = 0>
 __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L) {
     constexpr int CHUNK_BLOCKS = CB;
@@ -174,7 +174,7 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
     constexpr int ITEMS = (TILE_ROWS * CHUNK_GROUPS + THREADS - 1) / THREADS;
     constexpr int FOLD_BYTES = NB * TILE_ROWS * FOLD_PITCH * 4;
     constexpr int W_BYTES = 2 * W_STAGE > FOLD_BYTES ? 2 * W_STAGE : FOLD_BYTES;
-    constexpr int XG = x_batch_groups(S, NB);
+    constexpr int XG = PRO == 2 ? 2 : x_batch_groups(S, NB);        // LDS-fed activations sit in vector registers: short batches
     constexpr int XN = XG * 2 * S;
     static_assert(THREADS >= NB * TILE_ROWS, "fold needs one thread per (token, row)");
 
@@ -350,12 +350,11 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
 
     // x of `groups` consecutive scale groups starting at group g0 of the row
     auto load_x = [&](int g0, float (&xq)[NB][XN], int groups) {
-        if (PRO == 2) {                   // wave-uniform LDS reads, broadcast into scalar registers
+        if (PRO == 2) {                   // every lane reads the same LDS words: the activations travel in vector registers
             const float *xl = x_lds + g0 * 64 + S * wave;
 #pragma unroll
             for (int k = 0; k < XN; ++k)
-                if (k < groups * 2 * S)
-                    xq[0][k] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(xl[(k / S) * 32 + (k % S)])));
+                if (k < groups * 2 * S) xq[0][k] = xl[(k / S) * 32 + (k % S)];
             return;
         }
         const uniform_f32_ptr xg = xbase + (size_t)g0 * 64;
