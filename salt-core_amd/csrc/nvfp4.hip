@@ -136,8 +136,8 @@ constexpr int x_batch_blocks(int S, int NB) {
 
 // QDQ: the launch's single token is quantised and dequantised by every
 // workgroup in its prologue (the activation pass of the reference matvec,
-// nvfp4.c:228-256) into LDS, and the rows read it from there through
-// v_readfirstlane; workgroup 0 reports a non-finite activation (-1 into a
+// nvfp4.c:228-256) into LDS, and the rows read it from there into vector
+// registers (every lane the same words); workgroup 0 reports a non-finite activation (-1 into a
 // status word the caller cleared) and nothing is published then.
 template <int S, int NB, bool QDQ = false>
 __global__ __launch_bounds__((32 / S) * 64) void fp4_tile_kernel(const Fp4Launch L) {
@@ -146,7 +146,7 @@ __global__ __launch_bounds__((32 / S) * 64) void fp4_tile_kernel(const Fp4Launch
     constexpr int PIECES = (TILE_ROWS * CHUNK_BLOCKS) / THREADS;     // 16-byte pieces == (row, block) items
     constexpr int FOLD_BYTES = NB * TILE_ROWS * FOLD_PITCH * 4;
     constexpr int W_BYTES = 2 * W_STAGE > FOLD_BYTES ? 2 * W_STAGE : FOLD_BYTES;
-    constexpr int XB = x_batch_blocks(S, NB);
+    constexpr int XB = QDQ ? 2 : x_batch_blocks(S, NB);      // LDS-fed activations sit in vector registers: short batches
     constexpr int XN = XB * S;
     constexpr int W_ROW_STEP = THREADS / 16;
     static_assert(THREADS >= NB * TILE_ROWS, "fold needs one thread per (token, row)");
@@ -241,12 +241,11 @@ __global__ __launch_bounds__((32 / S) * 64) void fp4_tile_kernel(const Fp4Launch
     issue(0);
 
     auto load_x = [&](int blk0, float (&xq)[NB][XN], int blocks) {
-        if (QDQ) {                        // wave-uniform LDS reads, broadcast into scalar registers
+        if (QDQ) {                        // every lane reads the same LDS words: the activations travel in vector registers
             const float *xl = x_lds + blk0 * 32 + S * wave;
 #pragma unroll
             for (int k = 0; k < XN; ++k)
-                if (k < blocks * S)
-                    xq[0][k] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(xl[(k / S) * 32 + (k % S)])));
+                if (k < blocks * S) xq[0][k] = xl[(k / S) * 32 + (k % S)];
             return;
         }
         const uniform_f32_ptr xg = xbase + (size_t)blk0 * 32;
