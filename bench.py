@@ -435,6 +435,34 @@ def main():
                 abi_call()
             extra["abi_q4_matvec_4096_host_pointers_us"] = round((time.perf_counter() - t0) / 200 * 1e6, 1)
             lib.salt_gpu_weight_resource_deactivate(1, 900)
+            # the engine's decode call for the routed experts: salt_gpu_q4_moe_chain over eight experts, one row each
+            import engine_abi
+            eabi = engine_abi.bind(lib)
+            if eabi.salt_gpu_expert_resource_bind(901, pool.ctypes.data, pool.nbytes) == 0:
+                proj, n = synth.expert_proj_bytes(H, F), H * F
+                recs = (engine_abi.MoeExpert * K)()
+                for i, e8 in enumerate(range(3, 3 + 15 * K, 15)):
+                    at = pool.ctypes.data + e8 * 3 * proj
+                    for p_, name in enumerate(("gate", "up", "down")):
+                        setattr(recs[i], name + "_vals", at + p_ * proj)
+                        setattr(recs[i], name + "_scales", at + p_ * proj + n // 2)
+                        setattr(recs[i], name + "_biases", at + p_ * proj + n // 2 + (n // 64) * 2)
+                        setattr(recs[i], name + "_id", at + p_ * proj)
+                    recs[i].group, recs[i].resource_slot, recs[i].logical_resource_id = 1, -1, 0
+                xin = np.tile(synth.activations(H, 1, 7)[0], (K, 1)).astype(np.float32)
+                yout, scr = np.zeros((K, H), np.float32), np.zeros((2, K * F), np.float32)
+
+                def chain_call():
+                    if eabi.salt_gpu_q4_moe_chain(recs, K, H, F, xin.ctypes.data, yout.ctypes.data, scr[0].ctypes.data,
+                                                  scr[1].ctypes.data, K * F) != 0:
+                        raise RuntimeError(lib.salt_mi355_last_error().decode())
+                for _ in range(20):
+                    chain_call()
+                t0 = time.perf_counter()
+                for _ in range(200):
+                    chain_call()
+                extra["abi_q4_moe_chain_8_experts_us"] = round((time.perf_counter() - t0) / 200 * 1e6, 1)
+                eabi.salt_gpu_expert_resource_unbind(901)
         # MoE prefill, 2048 tokens through one layer (E = 128, top-8, Zipf 1.1), grouped per expert, matrix cores
         T = 2048
         sel, wts = synth.zipf_selection(T, E, K, 1.1, 60)

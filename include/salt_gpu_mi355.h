@@ -100,6 +100,13 @@ typedef struct SaltMi355Q4Job {
 } SaltMi355Q4Job;
 int salt_mi355_q4_jobs_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tokens,
                            int chains_per_lane, void *stream);
+/* The down projections of a decode-shaped expert chain in one launch, without a launch for the activation: every
+ * job has one token, and its activation row is gelu_tanh(g[i]) * u[i] (reference gemma4.c:80-83,
+ * gemma4_text.c:7608-7649) where g = job.xs and u = job.xs + up_offset_floats, both [C] floats on the device.  C a
+ * multiple of 64 up to 4096; pointers as the tiled kernel needs them (values 4-byte, scales and biases 2-byte
+ * aligned), else -1.  ys[j] is bit-identical to salt_mi355_moe_activate_dev followed by salt_mi355_q4_jobs_dev. */
+int salt_mi355_q4_jobs_activated_dev(const SaltMi355Q4Job *jobs, int njobs, int C, long long up_offset_floats,
+                                     void *stream);
 /* Accumulation mode of the tiled Q4 kernel for later launches; returns the
  * previous mode.  0 (default): acc = fl(acc + fl(w * x)), bit-identical to the
  * reference.  1: acc = fma(w, x, acc) in the same chain order, one rounding

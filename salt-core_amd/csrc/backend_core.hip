@@ -251,10 +251,13 @@ int salt_mi355_graph_destroy(void *graph_exec) {
 
 // ---------------------------------------------------------------- Q4, device-resident
 
-int salt_mi355_q4_jobs_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tokens, int chains,
-                           void *stream_handle) {
+}  // extern "C"
+
+// Shared by the plain and the activated multi-job entry points.  activated: one token per job, whose activation row
+// is gelu_tanh(xs[i]) * xs[i + act_delta].
+static int q4_jobs_common(const SaltMi355Q4Job *jobs, int njobs, int C, int tokens, int chains, bool activated,
+                          long long act_delta, hipStream_t stream) {
     State &s = g_state;
-    hipStream_t stream = (hipStream_t)stream_handle;
     if (!s.ready) { set_error("q4: library not initialised"); return -1; }
     if (!jobs || njobs < 1 || C < 1 || tokens < 1) { set_error("q4: bad arguments"); return -1; }
     if (chains != 0 && chains != 8 && chains != 4 && chains != 2) { set_error("q4: chains_per_lane %d", chains); return -1; }
@@ -299,11 +302,29 @@ int salt_mi355_q4_jobs_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tok
             if (!slot) return -1;
             launch.table = (const Q4Job *)slot->device;
         }
-        const int rc = tileable ? q4_launch(launch, chains, stream) : q4_launch_generic(launch, stream);
+        launch.act_delta = act_delta;
+        if (activated && !tileable) { table_release(slot, stream); set_error("q4 activated: the jobs do not meet the tiled kernel's needs"); return -1; }
+        const int rc = activated ? q4_activated_launch(launch, stream)
+                                 : (tileable ? q4_launch(launch, chains, stream) : q4_launch_generic(launch, stream));
         table_release(slot, stream);
         if (rc != 0) { set_error("q4: kernel launch failed: %s", hipGetErrorString(hipGetLastError())); return -1; }
     }
     return 0;
+}
+
+extern "C" {
+
+int salt_mi355_q4_jobs_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tokens, int chains, void *stream) {
+    return q4_jobs_common(jobs, njobs, C, tokens, chains, false, 0, (hipStream_t)stream);
+}
+
+int salt_mi355_q4_jobs_activated_dev(const SaltMi355Q4Job *jobs, int njobs, int C, long long up_offset_floats,
+                                     void *stream) {
+    if (C < 64 || (C & 63) || C > MOE_FUSE_MAX_ROUTED) {
+        set_error("q4 activated: C must be a multiple of 64 up to %d", MOE_FUSE_MAX_ROUTED);
+        return -1;
+    }
+    return q4_jobs_common(jobs, njobs, C, 1, 0, true, up_offset_floats, (hipStream_t)stream);
 }
 
 int salt_mi355_q4_matvec_dev(const void *vals, const void *scales, const void *biases, int R, int C, int B,

@@ -1059,6 +1059,30 @@ int moe_chain(const SaltGpuMoeExpert *experts, int count, int hidden, int routed
     }
     std::vector<OutputCopy> none;
     if (run_q4_jobs(jobs, hidden, &none) != 0) { (void)salt_gpu_sync(); return -1; }
+    // Decode shape (one row per expert): gelu_tanh(gate) * up is computed in the prologue of the down launch.
+    bool one_row_each = (routed & 63) == 0 && routed <= 4096 && !g_state.q4_fused;
+    for (int i = 0; i < count && one_row_each; ++i)
+        one_row_each = experts[i].group == 1 && ((uintptr_t)down[(size_t)i].vals & 3) == 0 &&
+                       ((uintptr_t)down[(size_t)i].scales & 1) == 0 && ((uintptr_t)down[(size_t)i].biases & 1) == 0;
+    if (one_row_each) {
+        std::vector<SaltMi355Q4Job> activated((size_t)count);
+        for (int i = 0; i < count; ++i) {
+            SaltMi355Q4Job &q = activated[(size_t)i];
+            q.vals = down[(size_t)i].vals; q.scales = down[(size_t)i].scales; q.biases = down[(size_t)i].biases;
+            q.xs = gate_dev + (size_t)i * routed;
+            q.ys = (float *)out_dev + (size_t)i * hidden;
+            q.rows = hidden;
+        }
+        if (salt_mi355_q4_jobs_activated_dev(activated.data(), count, routed, (long long)(up_dev - gate_dev), g_state.stream) != 0) {
+            (void)salt_gpu_sync();
+            return -1;
+        }
+        e.pending.push_back({out_pin, outputs, in_floats * 4});
+        std::vector<OutputCopy> copies;
+        if (!out_in_place) copies.push_back(OutputCopy{out_dev, out_pin, in_floats * 4});
+        count_batch(experts[0].gate_vals, any_legacy);
+        return finish_call(copies);
+    }
     if (salt_mi355_moe_activate_dev(gate_dev, up_dev, act_dev, mid_floats, g_state.stream) != 0) { (void)salt_gpu_sync(); return -1; }
     jobs.clear();
     row = 0;

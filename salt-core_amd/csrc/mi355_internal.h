@@ -55,6 +55,7 @@ struct Q4Launch {
     int tiles_per_job;        // > 0 when every job of the table has this many tiles (tile -> job by division), else 0
     int fused;                // 0: separately rounded multiply and add (bit-exact); 1: fma accumulate
     MoeFuse moe;              // only read by q4_moe_gate_up_launch / q4_moe_down_launch
+    long long act_delta;      // q4_activated_launch: floats from a job's gate row (its x) to its up row
     // Up to Q4_INLINE_JOBS job records inside the kernel arguments: a decode-sized batch (the gate and up projections
     // of eight experts) then needs no table upload.  Must stay the last member.
     Q4Job inline_jobs[Q4_INLINE_JOBS];
@@ -66,6 +67,9 @@ int q4_moe_down_launch(const Q4Launch &launch, hipStream_t stream);
 int q4_launch(const Q4Launch &launch, int chains_per_lane, hipStream_t stream);
 // Any C, any byte alignment: one wave64 computes two rows, lane = chain.
 int q4_launch_generic(const Q4Launch &launch, hipStream_t stream);
+// One token per job; a job's activations are gelu_tanh(x[i]) * x[i + act_delta], computed in every workgroup's
+// prologue (cols <= MOE_FUSE_MAX_ROUTED, tileable jobs).
+int q4_activated_launch(const Q4Launch &launch, hipStream_t stream);
 // true when every pointer and the column count meet the tiled kernel's needs
 bool q4_job_is_tileable(const Q4Job &job, int cols);
 

@@ -159,7 +159,8 @@ constexpr int x_batch_groups(int S, int NB) {
 // launch): 1 = router top-k, the workgroup derives its gate or up job from the
 // selection; 2 = the down projection of one selected expert, whose activations
 // gelu_tanh(gate) * up are computed into LDS and reach the VALU in vector
-// registers (every lane reads the same words) instead of through scalar loads.
+// registers (every lane reads the same words) instead of through scalar loads;
+// 3 = the same activation prologue for jobs of the launch (one token each).
 template <int S, int NB, bool FUSED, int CB, int PRO = 0>
 __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L) {
     constexpr int CHUNK_BLOCKS = CB;
@@ -174,13 +175,13 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
     constexpr int ITEMS = (TILE_ROWS * CHUNK_GROUPS + THREADS - 1) / THREADS;
     constexpr int FOLD_BYTES = NB * TILE_ROWS * FOLD_PITCH * 4;
     constexpr int W_BYTES = 2 * W_STAGE > FOLD_BYTES ? 2 * W_STAGE : FOLD_BYTES;
-    constexpr int XG = PRO == 2 ? 2 : x_batch_groups(S, NB);        // LDS-fed activations sit in vector registers: short batches
+    constexpr int XG = PRO >= 2 ? 2 : x_batch_groups(S, NB);        // LDS-fed activations sit in vector registers: short batches
     constexpr int XN = XG * 2 * S;
     static_assert(THREADS >= NB * TILE_ROWS, "fold needs one thread per (token, row)");
 
     __shared__ __attribute__((aligned(16))) uint8_t w_lds[W_BYTES];
     __shared__ __attribute__((aligned(16))) float m_lds[2 * M_STAGE];
-    __shared__ __attribute__((aligned(16))) float x_lds[PRO == 2 ? MOE_FUSE_MAX_ROUTED : 4];
+    __shared__ __attribute__((aligned(16))) float x_lds[PRO >= 2 ? MOE_FUSE_MAX_ROUTED : 4];
     __shared__ int slow_flag;
     static_assert(PRO == 0 || (NB == 1 && !FUSED), "the MoE prologues serve the single-token bit-exact kernel");
     static_assert(PRO != 1 || (sizeof(RouterShared) <= W_BYTES && THREADS >= MOE_FUSE_MAX_EXPERTS),
@@ -193,6 +194,11 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
     Q4Job job;
     if (PRO == 0) {
         job = find_job(L, blockIdx.x);
+    } else if (PRO == 3) {
+        // the job's activation row is gelu_tanh(gate) * up of the two rows its x names: x[i] and x[i + act_delta]
+        job = find_job(L, blockIdx.x);
+        const float *gate = job.x, *up = job.x + L.act_delta;
+        for (int i = tid; i < L.cols; i += THREADS) x_lds[i] = det_gelu_tanh(gate[i]) * up[i];
     } else {
         const MoeFuse &m = L.moe;
         const size_t n = (size_t)m.hidden * (size_t)m.routed;
@@ -350,7 +356,7 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
 
     // x of `groups` consecutive scale groups starting at group g0 of the row
     auto load_x = [&](int g0, float (&xq)[NB][XN], int groups) {
-        if (PRO == 2) {                   // every lane reads the same LDS words: the activations travel in vector registers
+        if (PRO >= 2) {                   // every lane reads the same LDS words: the activations travel in vector registers
             const float *xl = x_lds + g0 * 64 + S * wave;
 #pragma unroll
             for (int k = 0; k < XN; ++k)
@@ -646,6 +652,16 @@ int q4_moe_down_launch(const Q4Launch &launch, hipStream_t stream) {
         hipLaunchKernelGGL((q4_tile_kernel<2, 1, false, 32, 2>), grid, dim3(1024), 0, stream, L);
     else
         hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 16, 2>), grid, dim3(512), 0, stream, L);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int q4_activated_launch(const Q4Launch &L, hipStream_t stream) {
+    if (L.total_tiles < 1 || L.tokens != 1 || L.fused || L.cols < 64 || (L.cols & 63) || L.cols > MOE_FUSE_MAX_ROUTED) return -1;
+    const dim3 grid(L.total_tiles);
+    if (L.total_tiles <= env_wide_limit())
+        hipLaunchKernelGGL((q4_tile_kernel<2, 1, false, 32, 3>), grid, dim3(1024), 0, stream, L);
+    else
+        hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 16, 3>), grid, dim3(512), 0, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

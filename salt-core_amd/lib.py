@@ -89,6 +89,7 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_event_elapsed_ms, i, vp, vp, C.POINTER(f))
     _sig(lib.salt_mi355_q4_matvec_dev, i, vp, vp, vp, i, i, i, vp, vp, i, vp)
     _sig(lib.salt_mi355_q4_jobs_dev, i, C.POINTER(Q4Job), i, i, i, i, vp)
+    _sig(lib.salt_mi355_q4_jobs_activated_dev, i, C.POINTER(Q4Job), i, i, C.c_longlong, vp)
     _sig(lib.salt_mi355_set_q4_accumulate, i, i)
     _sig(lib.salt_mi355_q4_matmul_workspace_bytes, sz, i, i)
     _sig(lib.salt_mi355_q4_matmul_dev, i, vp, vp, vp, i, i, i, vp, vp, vp, vp)

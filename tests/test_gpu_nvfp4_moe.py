@@ -211,6 +211,37 @@ def test_activation_and_reduce_match_checker(gpu, oracle):
     assert np.array_equal(bits(do.to_host(np.float32)), bits(acc))
 
 
+@pytest.mark.parametrize("njobs,Cc,rows", [(1, 704, 2816), (8, 704, 2816), (20, 64, 130), (3, 4096, 65), (16, 1088, 200)])
+def test_activated_down_jobs(gpu, oracle, pkg, njobs, Cc, rows):
+    """Down projections whose activation row gelu_tanh(gate) * up is computed in the launch's prologue: one record, inline
+    records and a device table; bit for bit the activation kernel followed by the plain multi-job launch."""
+    print("activated jobs", njobs, Cc, rows, flush=True)
+    lib = gpu.load()
+    gate = (synth.activations(Cc, njobs, 61) * 2).astype(np.float32)
+    up = synth.activations(Cc, njobs, 62)
+    both = gpu.DeviceBuffer.from_host(np.concatenate([gate.ravel(), np.zeros(32, np.float32), up.ravel()]))
+    up_offset = gate.size + 32
+    hold, jobs, want = [], (pkg.lib.Q4Job * njobs)(), []
+    for j in range(njobs):
+        vals, scales, biases = synth.q4_tensor(rows, Cc, 700 + j)
+        bufs = [pkg.lib.DeviceBuffer.from_host(a) for a in (vals, scales, biases)]
+        out = pkg.lib.DeviceBuffer(rows * 4, fill=0xFF)
+        hold.append((bufs, out))
+        jobs[j] = pkg.lib.Q4Job(bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, both.at(j * Cc * 4), out.ptr, rows)
+        act = np.array([np.float32(oracle.orc_gelu_tanh(float(a))) * b for a, b in zip(gate[j], up[j])], np.float32)
+        y = np.zeros(rows, np.float32)
+        assert oracle.orc_q4_matvec_threads(ptr(vals), ptr(scales), ptr(biases), rows, Cc, ptr(act), ptr(y), host_threads()) == 0
+        want.append(y)
+    stream = lib.salt_mi355_stream()
+    assert lib.salt_mi355_q4_jobs_activated_dev(jobs, njobs, Cc, up_offset, stream) == 0, lib.salt_mi355_last_error()
+    assert lib.salt_mi355_stream_sync(stream) == 0
+    for j in range(njobs):
+        assert np.array_equal(bits(hold[j][1].to_host(np.float32)), bits(want[j])), j
+    # column counts the prologue does not hold, or that are no multiple of 64
+    assert lib.salt_mi355_q4_jobs_activated_dev(jobs, njobs, 4160, up_offset, stream) == -1
+    assert lib.salt_mi355_q4_jobs_activated_dev(jobs, njobs, 100, up_offset, stream) == -1
+
+
 @pytest.mark.parametrize("case", cases.MOE_CASES, ids=lambda c: c[0])
 def test_moe_decode_step_reference_fixtures(gpu, case):
     name, E, K, H, F, pseed, lseed, xseed = case
