@@ -574,6 +574,51 @@ def test_nvfp4_engine_entry_points(eng, oracle, pkg):
     assert eng.salt_gpu_nvfp4_matvec(key, R, Cc, ptr(xs[0]), ptr(y)) == -1
 
 
+def test_nvfp4_mixed_batch_of_two_tensors(eng, oracle, pkg):
+    """salt_gpu_nvfp4_mixed_batch (reference gpu.h:56-59): jobs on tensors of different heights that share the column
+    count, several tokens per job, one call."""
+    Cc = 1024
+    shapes = [96, 200]
+    tensors = [synth.nvfp4_tensor(R, Cc, 300 + R) for R in shapes]
+    globals_ = [np.array([2688.0, 64.0], np.float32), np.array([0.37, 64.0], np.float32)]
+    parts, at, offs = [], 0, []
+    for (packed, scales), g in zip(tensors, globals_):
+        o = []
+        for a in (packed, scales, g.view(np.uint8)):
+            o.append(at); parts.append(a.view(np.uint8)); at += a.nbytes
+            pad = (-at) % 16; parts.append(np.zeros(pad, np.uint8)); at += pad
+        offs.append(o)
+    blob = np.concatenate(parts); base = blob.ctypes.data
+    assert eng.salt_gpu_weight_resource_bind(TRUNK, 13, base, blob.nbytes) == 0, err(pkg)
+    keys = [0x8801, 0x8802]
+    for k, (R, o) in enumerate(zip(shapes, offs)):
+        assert eng.salt_gpu_nvfp4_resource_slot(TRUNK, 13, keys[k], base + o[0], base + o[1], base + o[2], base + o[2] + 4,
+                                                R, Cc) == 0, err(pkg)
+
+    def want(k, xs):
+        packed, scales = tensors[k]
+        out = np.zeros((xs.shape[0], shapes[k]), np.float32)
+        for t in range(xs.shape[0]):
+            s = (np.zeros(Cc // 2, np.uint8), np.zeros(Cc // 16, np.uint8), np.zeros(Cc, np.float32))
+            assert oracle.orc_nvfp4_matvec(ptr(packed), ptr(scales), float(globals_[k][0]), 64.0, shapes[k], Cc,
+                                           ptr(np.ascontiguousarray(xs[t])), ptr(out[t]), ptr(s[0]), ptr(s[1]), ptr(s[2])) == 0
+        return out
+
+    plan = [(0, 2), (1, 1), (0, 1), (1, 3)]                       # (tensor, tokens)
+    xs = [synth.activations(Cc, n, 400 + j) for j, (_, n) in enumerate(plan)]
+    ys = [np.full((n, shapes[k]), 7.0, np.float32) for k, n in plan]
+    rc = eng.salt_gpu_nvfp4_mixed_batch(abi.ptr_array([keys[k] for k, _ in plan]), abi.ptr_array(xs), abi.ptr_array(ys),
+                                        (C.c_int * 4)(*[n for _, n in plan]), (C.c_int * 4)(*[shapes[k] for k, _ in plan]),
+                                        Cc, 4)
+    assert rc == 0, err(pkg)
+    for (k, n), x, y in zip(plan, xs, ys):
+        assert np.array_equal(bits(y), bits(want(k, x))), (k, n)
+    # a height that is not the key's
+    assert eng.salt_gpu_nvfp4_mixed_batch(abi.ptr_array([keys[0]]), abi.ptr_array(xs[:1]), abi.ptr_array(ys[:1]),
+                                          (C.c_int * 1)(2), (C.c_int * 1)(shapes[1]), Cc, 1) == -1
+    assert eng.salt_gpu_weight_resource_unbind(TRUNK, 13) == 0
+
+
 def test_router_gate_and_head_through_the_engine(eng, oracle, pkg):
     """An 8-bit router gate (one job per token of the same matrix, the way the engine batches it) and the bf16 head,
     both inside one described trunk resource."""
