@@ -107,13 +107,24 @@ int salt_mi355_q4_jobs_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tok
  * aligned), else -1.  ys[j] is bit-identical to salt_mi355_moe_activate_dev followed by salt_mi355_q4_jobs_dev. */
 int salt_mi355_q4_jobs_activated_dev(const SaltMi355Q4Job *jobs, int njobs, int C, long long up_offset_floats,
                                      void *stream);
-/* Accumulation mode of the tiled Q4 kernel for later launches; returns the
- * previous mode.  0 (default): acc = fl(acc + fl(w * x)), bit-identical to the
- * reference.  1: acc = fma(w, x, acc) in the same chain order, one rounding
- * fewer per element: not bit-identical, within a few ulp of the sum of
- * magnitudes.  The environment variable SALT_MI355_Q4_FUSED=1 selects mode 1
- * at initialisation. */
-int salt_mi355_set_q4_accumulate(int fused);
+/* Tolerance-class decode matvec: the memory-bound kernel.  Same layouts and
+ * shapes as salt_mi355_q4_matvec_dev / salt_mi355_q4_jobs_dev, but NOT
+ * bit-identical to the reference row (kernels.c:220-250), whose 32-chain order
+ * with four roundings per weight costs more vector instructions than the
+ * memory system leaves time for.  Per 64-column scale group the kernel forms
+ *   scale * sum_c q_c * x_c + bias * sum_c x_c
+ * with the integer-by-activation sums exact (activations in block fixed point
+ * of 31 bits below each group's largest magnitude) and a few fp32 roundings per
+ * group.  Bound, per output:
+ *   |y - y_ref| <= 2^-20 * sum_c (|q_c s| + 16 |s| + |b|) |x_c| + 1e-6.
+ * A non-finite activation makes every output of its token non-finite (the
+ * reference: the rows that touch it).  C a multiple of 64, at least 512, and
+ * dword-aligned values take the streaming kernel; anything else runs on the
+ * bit-exact kernels.  The reference has no counterpart (north star: "otherwise
+ * within a stated max-abs/relative fp32 tolerance"). */
+int salt_mi355_q4_matvec_t_dev(const void *vals, const void *scales, const void *biases,
+                               int R, int C, int B, const float *xs, float *ys, void *stream);
+int salt_mi355_q4_jobs_t_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tokens, void *stream);
 
 /* Prefill-sized variant on the matrix cores: ys[t*R + r] for B tokens against
  * one matrix, fp32-accurate but NOT bit-identical to the reference (different

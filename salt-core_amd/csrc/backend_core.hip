@@ -86,6 +86,11 @@ int verify_converters() {
 
 State::TableSlot *table_acquire(const void *host_table, size_t nbytes, hipStream_t stream) {
     State &s = g_state;
+    // A decode loop sends the same tables token after token: a slot that already holds these bytes, uploaded on this
+    // stream, is used again without a copy (stream order puts the earlier upload before the new reader).
+    for (State::TableSlot &held : s.tables)
+        if (held.device && held.valid_bytes == nbytes && held.stream == stream && memcmp(held.pinned, host_table, nbytes) == 0)
+            return &held;
     State::TableSlot *slot = &s.tables[s.next_table];
     s.next_table = (s.next_table + 1) % State::kTableSlots;
     if (slot->busy) {
@@ -105,10 +110,13 @@ State::TableSlot *table_acquire(const void *host_table, size_t nbytes, hipStream
     }
     if (!slot->done && hip_ok(hipEventCreateWithFlags(&slot->done, hipEventDisableTiming), "hipEventCreate") != 0)
         return nullptr;
+    slot->valid_bytes = 0;
     memcpy(slot->pinned, host_table, nbytes);
     if (hip_ok(hipMemcpyAsync(slot->device, slot->pinned, nbytes, hipMemcpyHostToDevice, stream),
                "job table upload") != 0)
         return nullptr;
+    slot->valid_bytes = nbytes;
+    slot->stream = stream;
     return slot;
 }
 
@@ -155,8 +163,6 @@ int salt_mi355_init(void) {
         s.fork = s.join = nullptr;
         return -1;
     }
-    const char *fused = getenv("SALT_MI355_Q4_FUSED");
-    s.q4_fused = fused && *fused == '1';
     s.ready = 1;
     if (getenv("SALT_GPU_DIAG"))
         fprintf(stderr, "salt-mi355: ready on %s, %d CUs, fp8 code scale %g\n", prop.gcnArchName,
@@ -184,12 +190,6 @@ int salt_mi355_shutdown(void) {
 }
 
 const char *salt_mi355_last_error(void) { return g_state.last_error; }
-
-int salt_mi355_set_q4_accumulate(int fused) {
-    const int before = g_state.q4_fused;
-    g_state.q4_fused = fused ? 1 : 0;
-    return before;
-}
 
 int salt_mi355_converter_tables(float *fp8, float *fp4) {
     if (!g_state.ready || !fp8 || !fp4) return -1;
@@ -291,7 +291,6 @@ static int q4_jobs_common(const SaltMi355Q4Job *jobs, int njobs, int C, int toke
         launch.cols = C;
         launch.tokens = group;
         launch.code_scale = s.code_scale;
-        launch.fused = s.q4_fused;
         State::TableSlot *slot = nullptr;
         if (njobs == 1) {
             launch.one = table[0];
@@ -325,6 +324,76 @@ int salt_mi355_q4_jobs_activated_dev(const SaltMi355Q4Job *jobs, int njobs, int 
         return -1;
     }
     return q4_jobs_common(jobs, njobs, C, 1, 0, true, up_offset_floats, (hipStream_t)stream);
+}
+
+// Tolerance-class decode matvec: jobs the streaming kernel cannot take (short or ragged rows, misaligned tensors)
+// run on the bit-exact kernels, whose result is inside any tolerance.
+int salt_mi355_q4_jobs_t_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tokens, void *stream_) {
+    State &s = g_state;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (!s.ready) { set_error("q4 t: library not initialised"); return -1; }
+    if (!jobs || njobs < 1 || C < 1 || tokens < 1) { set_error("q4 t: bad arguments"); return -1; }
+    bool streamable = q4_dot_takes(C) && q4_dot_tokens_per_pass(C) > 0;
+    for (int j = 0; j < njobs && streamable; ++j) {
+        const SaltMi355Q4Job &q = jobs[j];
+        if (!q.vals || !q.scales || !q.xs || !q.ys || q.rows < 1 || (size_t)q.rows > SIZE_MAX / (size_t)C) {
+            set_error("q4 t: job %d is malformed", j);
+            return -1;
+        }
+        streamable = ((uintptr_t)q.vals & 3) == 0 && ((uintptr_t)q.scales & 1) == 0 && ((uintptr_t)q.biases & 1) == 0 &&
+                     ((uintptr_t)q.xs & 3) == 0 && ((uintptr_t)q.ys & 3) == 0 &&
+                     (uint64_t)DOT_BLOCK_ROWS * (uint64_t)C / 2u < (1ull << 31);
+    }
+    if (!streamable) return q4_jobs_common(jobs, njobs, C, tokens, 0, false, 0, stream);
+    const int per_pass = q4_dot_tokens_per_pass(C);
+    std::vector<Q4Job> table((size_t)njobs);
+    for (int first = 0; first < tokens; first += per_pass) {
+        const int group = tokens - first < per_pass ? tokens - first : per_pass;
+        Q4DotLaunch launch;
+        memset(&launch, 0, sizeof launch);
+        const DotShape shape = q4_dot_shape(C, group);
+        const int rows_per_wg = shape.waves * DOT_BLOCK_ROWS;
+        int wgs = 0;
+        bool uniform = true;
+        for (int j = 0; j < njobs; ++j) {
+            Q4Job &q = table[(size_t)j];
+            q.vals = (const uint8_t *)jobs[j].vals;
+            q.scales = (const uint8_t *)jobs[j].scales;
+            q.biases = (const uint8_t *)jobs[j].biases;
+            q.x = jobs[j].xs + (size_t)first * (size_t)C;
+            q.y = jobs[j].ys + (size_t)first * (size_t)jobs[j].rows;
+            q.rows = jobs[j].rows;
+            q.x_stride = C;
+            q.y_stride = jobs[j].rows;
+            q.tile0 = wgs;
+            wgs += (jobs[j].rows + rows_per_wg - 1) / rows_per_wg;
+            uniform = uniform && jobs[j].rows == jobs[0].rows;
+        }
+        launch.wgs_per_job = uniform ? wgs / njobs : 0;
+        launch.njobs = njobs;
+        launch.cols = C;
+        launch.tokens = group;
+        launch.total_wgs = wgs;
+        State::TableSlot *slot = nullptr;
+        if (njobs == 1) {
+            launch.one = table[0];
+        } else {
+            slot = table_acquire(table.data(), table.size() * sizeof(Q4Job), stream);
+            if (!slot) return -1;
+            launch.table = (const Q4Job *)slot->device;
+        }
+        const int rc = q4_dot_launch(launch, shape, stream);
+        table_release(slot, stream);
+        if (rc != 0) { set_error("q4 t: kernel launch failed: %s", hipGetErrorString(hipGetLastError())); return -1; }
+    }
+    return 0;
+}
+
+int salt_mi355_q4_matvec_t_dev(const void *vals, const void *scales, const void *biases, int R, int C, int B,
+                               const float *xs, float *ys, void *stream) {
+    SaltMi355Q4Job job;
+    job.vals = vals; job.scales = scales; job.biases = biases; job.xs = xs; job.ys = ys; job.rows = R;
+    return salt_mi355_q4_jobs_t_dev(&job, 1, C, B, stream);
 }
 
 int salt_mi355_q4_matvec_dev(const void *vals, const void *scales, const void *biases, int R, int C, int B,

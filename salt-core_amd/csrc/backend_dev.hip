@@ -393,7 +393,7 @@ int salt_mi355_ffn_block_dev(const SaltMi355FfnLayer *layer, const float *residu
     gate_up.tiles_per_job = q4_uniform_tiles(dense, 2);
     memcpy(gate_up.inline_jobs, dense, sizeof dense);
     gate_up.table = nullptr; gate_up.njobs = 2; gate_up.cols = L.hidden; gate_up.tokens = 1;
-    gate_up.code_scale = g_state.code_scale; gate_up.fused = g_state.q4_fused;
+    gate_up.code_scale = g_state.code_scale;
     const bool tileable = q4_job_is_tileable(dense[0], L.hidden) && q4_job_is_tileable(dense[1], L.hidden);
 
     if (ffn_pre_launch(residual, L.pre_norm, L.pre_norm_2, L.router_scale, ws.norm_a, ws.norm_b, ws.router_in, L.hidden, L.eps,

@@ -106,8 +106,13 @@ struct Engine {
     uint8_t *pinned_dev = nullptr;    // the pinned region as kernels address it (zero-copy for small calls)
     size_t staging_capacity = 0, pinned_used = 0, device_used = 0;
     // scratch for weights that arrive without a resident resource
-    uint8_t *legacy = nullptr;
-    size_t legacy_capacity = 0, legacy_used = 0;
+    // (chunks: a call that needs more than the current chunk holds gets another one; nothing that an earlier job of
+    // the same call points at is ever moved or freed before the call ends)
+    struct LegacyChunk { uint8_t *base; size_t capacity; };
+    std::vector<LegacyChunk> legacy_chunks;
+    size_t legacy_used = 0;           // bytes used of the last chunk
+    int legacy_dirty = 0;             // some chunk holds weights of an earlier call
+    int legacy_depth = 0;             // nesting of the entry points that may copy weights
     std::vector<Pending> pending;
     Residency residency;
     // component pool
@@ -368,26 +373,47 @@ int pool_release_resource(int ri) {
     return failed ? -1 : 0;
 }
 
+// Weights that arrive outside every resident resource are copied per call.  The copies of one call stay where they
+// are until the call has ended: a job enqueued early must not see a later job's weights.  The next call that copies
+// weights first waits for the device (the earlier call's kernels may be deferred) and starts over.
+struct LegacyScope {
+    LegacyScope() {
+        Engine &e = g_engine;
+        if (e.legacy_depth++ == 0 && e.legacy_dirty && g_state.ready) {
+            if (drain_device() == 0) {
+                // keep the largest chunk, free the others
+                size_t keep = 0;
+                for (size_t i = 1; i < e.legacy_chunks.size(); ++i)
+                    if (e.legacy_chunks[i].capacity > e.legacy_chunks[keep].capacity) keep = i;
+                for (size_t i = 0; i < e.legacy_chunks.size(); ++i)
+                    if (i != keep) (void)hipFree(e.legacy_chunks[i].base);
+                const Engine::LegacyChunk kept = e.legacy_chunks[keep];
+                e.legacy_chunks.assign(1, kept);
+                e.legacy_used = 0;
+                e.legacy_dirty = 0;
+            }
+        }
+    }
+    ~LegacyScope() { g_engine.legacy_depth--; }
+};
+
 int legacy_reserve(size_t nbytes) {
     Engine &e = g_engine;
-    if (e.legacy_used + nbytes <= e.legacy_capacity) return 0;
-    if (salt_gpu_sync() != 0 || drain_device() != 0) return -1;
-    e.legacy_used = 0;
-    if (nbytes <= e.legacy_capacity) return 0;
-    if (e.legacy) (void)hipFree(e.legacy);
-    e.legacy = nullptr;
-    e.legacy_capacity = 0;
+    if (!e.legacy_chunks.empty() && e.legacy_used + nbytes <= e.legacy_chunks.back().capacity) return 0;
     size_t capacity = 64u << 20;
     while (capacity < nbytes) capacity *= 2;
-    if (hip_ok(hipMalloc((void **)&e.legacy, capacity), "hipMalloc legacy weights") != 0) return -1;
-    e.legacy_capacity = capacity;
+    uint8_t *base = nullptr;
+    if (hip_ok(hipMalloc((void **)&base, capacity), "hipMalloc legacy weights") != 0) return -1;
+    e.legacy_chunks.push_back(Engine::LegacyChunk{base, capacity});
+    e.legacy_used = 0;
     return 0;
 }
 
 const uint8_t *legacy_upload(const void *host, size_t nbytes) {
     Engine &e = g_engine;
-    uint8_t *dst = e.legacy + e.legacy_used;
+    uint8_t *dst = e.legacy_chunks.back().base + e.legacy_used;
     e.legacy_used += align_up(nbytes, 256);
+    e.legacy_dirty = 1;
     // pageable source: the runtime stages it; the copy is complete on return
     if (hip_ok(hipMemcpy(dst, host, nbytes, hipMemcpyHostToDevice), "legacy weight upload") != 0) return nullptr;
     return dst;
@@ -572,7 +598,7 @@ int salt_gpu_free(void) {
         for (Seat &s : e.seats) if (s.owned) failed |= hip_ok(hipFree(s.owned), "hipFree seat");
         for (SaltGpuSharedBuffer &b : e.shared) if (b.contents) failed |= hip_ok(hipHostFree(b.contents), "hipHostFree");
         if (e.pinned) { failed |= hip_ok(hipHostFree(e.pinned), "hipHostFree"); failed |= hip_ok(hipFree(e.device), "hipFree"); }
-        if (e.legacy) failed |= hip_ok(hipFree(e.legacy), "hipFree");
+        for (const Engine::LegacyChunk &c : e.legacy_chunks) failed |= hip_ok(hipFree(c.base), "hipFree");
     }
     e = Engine();
     failed |= salt_mi355_shutdown();
@@ -867,6 +893,7 @@ extern "C" {
 
 int salt_gpu_q4_matvec(const uint32_t *vals, const uint16_t *scales, const uint16_t *biases, int R, int C,
                        const float *x, float *y) {
+    LegacyScope weights_of_this_call;
     if (ready_or_fail("q4_matvec") != 0) return -1;
     if (!vals || !scales || !x || !y || R < 1 || C < 1 || C > MAX_C || (size_t)R > MAX_OUTPUT_FLOATS) {
         set_error("q4_matvec: bad arguments");
@@ -886,6 +913,7 @@ int salt_gpu_q4_matvec(const uint32_t *vals, const uint16_t *scales, const uint1
 int salt_gpu_q4_batch(const uint32_t *const *vals, const uint16_t *const *scales, const uint16_t *const *biases,
                       const float *const *xs, float *const *ys, const void *const *ids, const int *Rj, int C,
                       int njobs) {
+    LegacyScope weights_of_this_call;
     if (ready_or_fail("q4_batch") != 0) return -1;
     if (!vals || !scales || !xs || !ys || !Rj || njobs < 1 || (uint32_t)njobs > MAX_BATCH_JOBS || C < 1 || C > MAX_C) {
         set_error("q4_batch: bad arguments");
@@ -925,6 +953,7 @@ int salt_gpu_q4_batch(const uint32_t *const *vals, const uint16_t *const *scales
 
 int salt_gpu_proj_batch(const uint32_t *vals, const uint16_t *scales, const uint16_t *biases, int R, int C, int B,
                         const float *const *xs, float *const *ys, const void *id) {
+    LegacyScope weights_of_this_call;
     if (ready_or_fail("proj_batch") != 0) return -1;
     if (!vals || !scales || !xs || !ys || R < 1 || C < 1 || C > MAX_C || B < 1 || B > MAX_PROJ_BATCH ||
         (uint64_t)B * (uint64_t)R > MAX_OUTPUT_FLOATS) {
@@ -952,6 +981,7 @@ int salt_gpu_proj_batch(const uint32_t *vals, const uint16_t *scales, const uint
 int salt_gpu_proj_batch_indexed(const uint32_t *vals, const uint16_t *scales, const uint16_t *biases, int R, int C,
                                 int B, int first_job, int job_count, const float *xs, SaltGpuSharedBuffer *output,
                                 size_t y_float_offset, const void *id) {
+    LegacyScope weights_of_this_call;
     if (ready_or_fail("proj_batch_indexed") != 0) return -1;
     if (!vals || !scales || !xs || !output || !output->contents || R < 1 || C < 1 || C > MAX_C || B < 2 ||
         B > MAX_PROJ_BATCH || first_job < 0 || job_count < 1 || first_job > B - job_count) {
@@ -995,6 +1025,7 @@ namespace {
 // `seats_only` makes every expert resolve through its bound cache seat.
 int moe_chain(const SaltGpuMoeExpert *experts, int count, int hidden, int routed, const float *inputs,
               float *outputs, float *gate_scratch, float *up_scratch, size_t scratch_capacity, int seats_only) {
+    LegacyScope weights_of_this_call;
     if (ready_or_fail("q4_moe_chain") != 0) return -1;
     if (!experts || !inputs || !outputs || !gate_scratch || !up_scratch || scratch_capacity < 1 || count < 1 ||
         count > 128 || hidden < 1 || routed < 1 || hidden > MAX_C || routed > MAX_C) {
@@ -1060,7 +1091,7 @@ int moe_chain(const SaltGpuMoeExpert *experts, int count, int hidden, int routed
     std::vector<OutputCopy> none;
     if (run_q4_jobs(jobs, hidden, &none) != 0) { (void)salt_gpu_sync(); return -1; }
     // Decode shape (one row per expert): gelu_tanh(gate) * up is computed in the prologue of the down launch.
-    bool one_row_each = (routed & 63) == 0 && routed <= 4096 && !g_state.q4_fused;
+    bool one_row_each = (routed & 63) == 0 && routed <= 4096;
     for (int i = 0; i < count && one_row_each; ++i)
         one_row_each = experts[i].group == 1 && ((uintptr_t)down[(size_t)i].vals & 3) == 0 &&
                        ((uintptr_t)down[(size_t)i].scales & 1) == 0 && ((uintptr_t)down[(size_t)i].biases & 1) == 0;
@@ -1128,6 +1159,7 @@ int salt_gpu_q4_moe_chain_selected(const SaltGpuMoeExpert *experts, int count, i
 }
 
 int salt_gpu_q4_selected_shared(const SaltGpuSelectedProjectionJob *jobs, int job_count, SaltGpuSharedBuffer *arena) {
+    LegacyScope weights_of_this_call;
     if (ready_or_fail("q4_selected_shared") != 0) return -1;
     if (!jobs || job_count < 1 || job_count > 256 || !arena || !arena->contents ||
         !shared_device_view(arena->contents, arena->nbytes)) {
@@ -1455,6 +1487,7 @@ int salt_gpu_nvfp4_batch(const void *const *keys, const float *const *inputs, fl
 int salt_gpu_q8_batch(const uint32_t *const *vals, const uint16_t *const *scales, const uint16_t *const *biases,
                       const float *const *xs, float *const *ys, const void *const *ids, const int *Rj, int C,
                       int njobs) {
+    LegacyScope weights_of_this_call;
     if (ready_or_fail("q8_batch") != 0) return -1;
     if (!vals || !scales || !xs || !ys || !Rj || njobs < 1 || (uint32_t)njobs > MAX_BATCH_JOBS || C < 1 || C > MAX_C) {
         set_error("q8_batch: bad arguments");
@@ -1508,6 +1541,7 @@ int salt_gpu_q8_batch(const uint32_t *const *vals, const uint16_t *const *scales
 
 int salt_gpu_q8_matvec(const uint32_t *vals, const uint16_t *scales, const uint16_t *biases, int R, int C,
                        const float *x, float *y) {
+    LegacyScope weights_of_this_call;
     const void *id = vals;
     return salt_gpu_q8_batch(&vals, &scales, &biases, &x, &y, &id, &R, C, 1);
 }

@@ -16,7 +16,6 @@ struct State {
     hipStream_t side = nullptr;         // second branch of a forked sequence (default priority, like every stream)
     hipEvent_t fork = nullptr, join = nullptr;
     float code_scale = 0.0f;            // 1 / fp8_table[1]
-    int q4_fused = 0;                   // 1: fma accumulate (tolerance class) instead of mul + add
     int fp8_is_ocp = 0;                 // the converter decodes every byte as OCP E4M3FN
     float fp8_table[256] = {0};
     float fp4_table[512] = {0};
@@ -27,6 +26,8 @@ struct State {
         void *device = nullptr;
         void *pinned = nullptr;
         size_t capacity = 0;
+        size_t valid_bytes = 0;         // bytes of `pinned` that the device copy mirrors (0: none)
+        hipStream_t stream = nullptr;   // the stream that carried the upload
         hipEvent_t done = nullptr;
         int busy = 0;
     };

@@ -53,7 +53,6 @@ struct Q4Launch {
     int total_tiles;
     float code_scale;         // 1 / (value the fp8 converter gives byte 1)
     int tiles_per_job;        // > 0 when every job of the table has this many tiles (tile -> job by division), else 0
-    int fused;                // 0: separately rounded multiply and add (bit-exact); 1: fma accumulate
     MoeFuse moe;              // only read by q4_moe_gate_up_launch / q4_moe_down_launch
     long long act_delta;      // q4_activated_launch: floats from a job's gate row (its x) to its up row
     // Up to Q4_INLINE_JOBS job records inside the kernel arguments: a decode-sized batch (the gate and up projections
@@ -77,6 +76,32 @@ bool q4_job_is_tileable(const Q4Job &job, int cols);
 int q4_assign_tiles(Q4Job *table, int njobs);
 // the common tile count of the jobs, or 0 when they differ
 int q4_uniform_tiles(const Q4Job *table, int njobs);
+
+// ---------------------------------------------------------------- affine Q4 decode matvec, tolerance class
+// (q4_dot.hip): per scale group  scale * sum q*x + bias * sum x  with the integer dot products exact.
+
+constexpr int DOT_BLOCK_ROWS = 32;         // rows per block; a wave walks whole blocks
+constexpr int DOT_MIN_COLS = 512;          // the streaming kernel takes 512 .. 8192 columns in multiples of 256;
+constexpr int DOT_MAX_COLS = 8192;         // callers send everything else to the exact kernel
+constexpr int DOT_LDS_LIMIT = 160 * 1024;
+
+// How a launch is cut: waves per workgroup (a wave owns one block of 32 rows), steps of LDS per wave.
+struct DotShape { int waves, stages; };
+
+struct Q4DotLaunch {
+    Q4Job one;                // used when table == nullptr; tile0 = index of the job's first workgroup
+    const Q4Job *table;       // device array of njobs jobs sorted by tile0
+    int njobs;
+    int cols;
+    int tokens;               // 1..4, at most q4_dot_tokens_per_pass(cols)
+    int total_wgs;
+    int wgs_per_job;          // > 0 when every job of the table has this many workgroups (workgroup -> job by division)
+    int debug;
+};
+bool q4_dot_takes(int cols);
+int q4_dot_tokens_per_pass(int cols);      // 0: the column count does not fit at all
+DotShape q4_dot_shape(int cols, int tokens);
+int q4_dot_launch(const Q4DotLaunch &launch, const DotShape &shape, hipStream_t stream);
 
 // ---------------------------------------------------------------- affine Q4 on MFMA (tolerance class)
 

@@ -1,0 +1,527 @@
+// Affine-Q4 matvec for gfx950, tolerance class: the HBM-bound decode kernel.
+//
+// The reference row (src/kernels.c:220-250) rounds every weight, product and sum and fixes the order of 32 chains;
+// reproducing that costs about four vector instructions per weight, which caps a bit-exact kernel below the memory
+// system.  This kernel computes the same sum in a different association, per 64-column scale group g of a row:
+//
+//     y = sum_g ( scale_g * sum_{c in g} q_c * x_c  +  bias_g * sum_{c in g} x_c )
+//
+// and evaluates the inner integer-by-activation dot products exactly:
+//  * each activation group is turned into block fixed point once per workgroup: I_c = rint(x_c * 2^k_g) with k_g
+//    chosen so that |I_c| < 2^30, split into four signed 8-bit digit planes  I = d0 + 2^8 d1 + 2^16 d2 + 2^24 d3.
+//    The error of x against its fixed-point image is at most 2^-31 of the group's largest magnitude.
+//  * the codes q (0..15) are 8-bit integers after two masks and a shift, so  sum_c q_c * d_p,c  is an integer dot
+//    product: v_mfma_i32_32x32x32_i8 computes it for 32 rows at a time.  The matrix instruction is used as a bank
+//    of dot-product units: its N side holds 32 weight rows, its M side the digit planes of up to four tokens, its K
+//    side sixteen columns of each of two groups.  Digit planes of the "other" group are zero, which keeps the two
+//    groups' sums apart in different output rows.
+//  * the four plane sums (each below 2^17) are recombined in integers and converted to fp32 once per group; the
+//    group's scale, its power of two and the bias term follow as two fused multiply-adds per (row, group, token).
+//    sum_c x_c of a group is accumulated in double and rounded once.
+// Everything except the last two steps is exact, so the result differs from the infinitely precise sum by a few
+// fp32 roundings per group.  Stated bound (tests): |y - y_ref| <= 2^-20 * sum_c (|q_c s| + 16|s| + |b|) |x_c| + 1e-6.
+//
+// Data movement: a wave owns blocks of 32 rows and walks each in two strips (halves of the row) at once, 128 bytes
+// of each strip and row per step: 8 KiB per step, fetched straight into LDS with eight 16-byte-per-lane loads
+// (contiguous 128-byte pieces in memory, non-temporal).  Several steps are in flight per wave and there is no
+// barrier after the prologue.  Lane (row n, strip h) reads its
+// 32 bytes of a group back with two 16-byte LDS reads (slots swizzled by the row so that the lanes of a read phase
+// hit different bank groups).  The scales and biases of a block do not travel with the steps: a lane fetches the
+// scales and biases of its row and strip for the whole block into registers before the stream starts, and picks
+// the step's four by register indexing.  (Fetching them per step with direct-to-LDS loads of 16 bytes per lane
+// costs a quarter of the stream's rate: 64 scattered pieces per load.  Loads that return to registers are kept out
+// of the loop on purpose: on this device they do not complete in issue order with direct-to-LDS loads, so a partial
+// s_waitcnt vmcnt(n) cannot tell which of the two kinds has landed.)
+#include "mi355_internal.h"
+
+#ifndef DOT_SWIZZLE_LOW
+#define DOT_SWIZZLE_LOW 0
+#endif
+
+#include <stddef.h>
+#include <stdio.h>
+#include <stdlib.h>
+
+#include <type_traits>
+#include <utility>
+
+namespace mi355 {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef const u32x4 __attribute__((address_space(1))) *global_u128_ptr;
+typedef __attribute__((address_space(3))) void *lds_void_ptr;
+typedef const uint64_t __attribute__((address_space(4))) *uniform_u64_ptr;
+
+constexpr int BLOCK_ROWS = DOT_BLOCK_ROWS;   // rows per block = N of the matrix instruction
+constexpr int STAGE_BYTES = 8192;            // 2 strips x 32 rows x 128 bytes
+constexpr int STAGE_GROUPS = 4;              // scale groups per strip and step
+constexpr int STEP_LDS = STAGE_BYTES;
+constexpr int LOADS_PER_STEP = 8;            // weight pieces
+constexpr int ZERO_BYTES = 1024 + 256;       // what lanes without a digit plane read instead
+constexpr int GROUP_IMAGE = 256;             // bytes of digits per group: 4 quarters x 4 planes x 16
+#ifndef DOT_STREAMING
+#define DOT_STREAMING 2
+#endif
+constexpr int STREAMING = DOT_STREAMING;     // 2 = non-temporal: every weight byte is read once
+
+__device__ __forceinline__ int swizzle(int piece) { return DOT_SWIZZLE_LOW ? (piece & 7) : ((piece >> 1) & 7); }
+
+// steps per strip: half of the row's groups, in whole steps
+__host__ __device__ __forceinline__ int dot_steps(int ngrp) { return ((ngrp + 1) / 2 + STAGE_GROUPS - 1) / STAGE_GROUPS; }
+
+// f(integral_constant<int, 0>), f(<1>), ... until one returns false; true when all ran
+template <int... I, class F>
+__device__ __forceinline__ bool static_steps(std::integer_sequence<int, I...>, F &&f) {
+    return (f(std::integral_constant<int, I>{}) && ...);
+}
+
+// A lane's scales (or biases) of one block: MD dwords = 2 * MD groups of its strip, in registers.
+template <int MD> struct MetaRegs { u32x4 q[MD / 4]; };
+
+// Written in assembly so that the compiler neither moves the load nor waits for it on its own: the one wait that
+// covers it names the registers (wait_meta).
+__device__ __forceinline__ u32x4 load_meta16(const uint8_t *address) {
+    u32x4 value;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(value) : "v"(address) : "memory");
+    return value;
+}
+__device__ __forceinline__ void wait_meta(u32x4 &value) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(value) : : "memory"); }
+
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ Q4Job dot_find_job(const Q4DotLaunch &L, int wg) {
+    if (L.table == nullptr) return L.one;
+    const uniform_u64_ptr words = (uniform_u64_ptr)(uintptr_t)L.table;
+    int lo = 0, hi = L.njobs - 1;
+    if (L.wgs_per_job > 0) {               // every job has the same number of workgroups: no search
+        lo = wg / L.wgs_per_job;
+    } else {
+        while (lo < hi) {                  // last job whose first workgroup is <= wg
+            const int mid = (lo + hi + 1) >> 1;
+            if ((int)(words[7 * mid + 5] >> 32) <= wg) lo = mid; else hi = mid - 1;
+        }
+    }
+    const uniform_u64_ptr rec = words + 7 * lo;
+    Q4Job job;
+    job.vals = (const uint8_t *)rec[0];
+    job.scales = (const uint8_t *)rec[1];
+    job.biases = (const uint8_t *)rec[2];
+    job.x = (const float *)rec[3];
+    job.y = (float *)rec[4];
+    job.rows = (int)(uint32_t)rec[5];
+    job.tile0 = (int)(rec[5] >> 32);
+    job.x_stride = (int)(uint32_t)rec[6];
+    job.y_stride = (int)(rec[6] >> 32);
+    return job;
+}
+
+// T tokens per pass (1..4), WAVES waves per workgroup, STAGES steps of LDS per wave (one being consumed, the others
+// in flight), MD dwords of scales per lane (two groups each: 16 serves rows of up to 4096 columns, 32 up to 8192).
+// A workgroup owns WAVES consecutive blocks of 32 rows of one job, one per wave.
+template <int T, int WAVES, int STAGES, int MD>
+__global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L) {
+    static_assert(T >= 1 && T <= 4 && STAGES >= 2 && STAGES <= 4 && (MD == 16 || MD == 32), "tokens per pass, steps per wave");
+    constexpr int WAVE_LDS = STAGES * STEP_LDS;
+    constexpr int AHEAD = STAGES - 1;                // steps in flight behind the one being consumed
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr int THREADS = WAVES * 64;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const Q4Job job = dot_find_job(L, blockIdx.x);
+
+    const int C = L.cols;
+    const int ngrp = C >> 6;
+    // Groups per strip: half the row, rounded up to whole steps so that strip 1 starts on a 128-byte boundary of the
+    // row (a piece that straddles two memory lines is fetched twice by loads that bypass the caches).  Strip 1 holds
+    // the remaining ngrp - SG groups.
+    const int nstage = dot_steps(ngrp);
+    const int SG = nstage * STAGE_GROUPS;
+    const uint32_t row_bytes = (uint32_t)C >> 1;
+    const int whole_steps = (ngrp - SG) / STAGE_GROUPS;            // steps that lie inside the row for both strips
+    // A lane holds the scales of 2 * MD consecutive groups of its row: strip 0 from group 0, strip 1 the row's last
+    // 2 * MD (both cover their strip; the launcher sees to it that the difference is a whole number of steps)
+    const int meta_groups = 2 * MD < ngrp ? 2 * MD : ngrp & ~7;
+    const int strip1_start = ngrp - meta_groups;
+    const int strip1_shift = (SG - strip1_start) / STAGE_GROUPS;   // steps by which strip 1's registers lead its steps
+
+    uint8_t *const w_lds = lds;                                            // [WAVES][STAGES][STEP_LDS]
+    uint8_t *const zero_lds = lds + WAVES * WAVE_LDS;                      // ZERO_BYTES
+    uint8_t *const img_lds = zero_lds + ZERO_BYTES;                        // [T][2 * SG][GROUP_IMAGE]
+    float *const xm_lds = (float *)(img_lds + (size_t)T * 2 * SG * GROUP_IMAGE);   // [T][2 * SG] (power of two, sum)
+
+    // the wave's block and its stream of steps
+    const int row_base = (((int)blockIdx.x - job.tile0) * WAVES + wave) * BLOCK_ROWS;
+    const bool has_rows = row_base < job.rows;       // a wave without rows still helps with the activations
+    const int rows_here = !has_rows ? 1 : (job.rows - row_base < BLOCK_ROWS ? job.rows - row_base : BLOCK_ROWS);
+    const int total_steps = has_rows ? nstage : 0;
+
+    // ---------------------------------------------------------------- per-lane geometry
+    // weights: load k of a step covers strip k / 4, rows 8 (k % 4) .. + 7 of the block; lane i lands in slot 64 k + i,
+    // that is piece (strip * 32 + row), position i % 8, which receives segment (i % 8) ^ swizzle(piece) of the piece
+    uint8_t *const my_lds = w_lds + (size_t)wave * WAVE_LDS;
+    int src_rowi[8];
+    uint32_t src_col[8], src_off[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const int strip = k >> 2;
+        const int row = (k & 3) * 8 + (lane >> 3);
+        const int piece = strip * 32 + row;
+        const int seg = (lane & 7) ^ swizzle(piece);
+        src_rowi[k] = row;
+        src_col[k] = (uint32_t)(strip * SG) * 32u + (uint32_t)seg * 16u;
+        src_off[k] = (uint32_t)row * row_bytes + src_col[k];
+    }
+    // reads: lane (n, h) owns piece h * 32 + n
+    const int n = lane & 31, h = lane >> 5;
+    const int my_piece = h * 32 + n;
+    uint32_t rd_off[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) rd_off[s] = (uint32_t)my_piece * 128u + (uint32_t)(s ^ swizzle(my_piece)) * 16u;
+    const bool no_bias = job.biases == nullptr;      // the load still happens (the waits count it); its result is dropped
+    const uint8_t *const bias_src = no_bias ? job.scales : job.biases;
+    // digit planes: row m = l % 32 of the M side is (token m / 8, strip (m / 4) % 2, plane m % 4); it carries digits
+    // only in the lanes of its own strip (l / 32)
+    const int m_tok = n >> 3, m_strip = (n >> 2) & 1, m_plane = n & 3;
+    const bool has_digits = m_tok < T && m_strip == h;
+    const uint8_t *const a_base = has_digits
+        ? img_lds + ((size_t)(m_tok * 2 * SG + m_strip * SG) * 16 + m_plane) * 16
+        : zero_lds + 64;              // a bank group that no digit plane of the same read occupies
+    const uint32_t a_step = has_digits ? STAGE_GROUPS * GROUP_IMAGE : 0u;
+    const float *const xm_ptr = xm_lds + 2 * (h * SG);
+
+    // ---------------------------------------------------------------- loads
+    // The block's scales and biases: lane (n, h) fetches 2 * MD groups of row n, 16 bytes at a time.
+    typedef uint32_t MetaVec __attribute__((ext_vector_type(MD)));
+    MetaRegs<MD> scales_r, biases_r;
+    MetaVec scales_v, biases_v;                      // the same registers as one indexable vector, valid after the wait
+    auto issue_meta = [&]() {
+        const int row = n < rows_here ? n : rows_here - 1;
+        const size_t at = ((size_t)(row_base + row) * ngrp + (h ? strip1_start : 0)) * 2;
+#pragma unroll
+        for (int q = 0; q < MD / 4; ++q) {
+            // pieces past the row's groups are not fetched (and never read): the address repeats the last real one
+            const int piece = 8 * q < meta_groups ? q : (meta_groups - 1) / 8;
+            scales_r.q[q] = load_meta16(job.scales + at + 16 * piece);
+            biases_r.q[q] = load_meta16(bias_src + at + 16 * piece);
+        }
+    };
+    // Step st into ring slot `slot`: eight weight pieces.
+    const uint8_t *const block_vals = job.vals + (size_t)row_base * row_bytes;
+    auto issue_step = [&](int st, int slot) {
+        uint8_t *const stage = my_lds + slot * STEP_LDS;
+        const uint32_t advance = (uint32_t)st * (STAGE_GROUPS * 32);
+        if (rows_here == BLOCK_ROWS && st < whole_steps) {
+            // a wave-uniform base that advances with the step plus a fixed 32-bit offset per lane
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                __builtin_amdgcn_global_load_lds((global_u128_ptr)(uintptr_t)(block_vals + advance + src_off[k]),
+                                                 (lds_void_ptr)(stage + k * 1024), 16, 0, STREAMING);
+        } else {
+            // the matrix ends inside this block, or strip 1 ends inside this step or before it: stay inside
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int row = src_rowi[k] < rows_here ? src_rowi[k] : rows_here - 1;
+                uint32_t col = src_col[k] + advance;
+                col = col <= row_bytes - 16 ? col : row_bytes - 16;
+                __builtin_amdgcn_global_load_lds((global_u128_ptr)(uintptr_t)(block_vals + ((uint32_t)row * row_bytes + col)),
+                                                 (lds_void_ptr)(stage + k * 1024), 16, 0, STREAMING);
+            }
+        }
+    };
+
+    // ---------------------------------------------------------------- arithmetic of one step
+    float acc[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) acc[t] = 0.0f;
+    // A step's weights leave LDS for registers in one go: its slot is then free for the loads of a later step while
+    // the arithmetic runs.
+    struct StepWeights { uint32_t raw[STAGE_GROUPS][8]; };
+    auto fetch = [&](int slot, StepWeights &w) {
+        const uint8_t *stage = my_lds + slot * STEP_LDS;
+#pragma unroll
+        for (int u = 0; u < STAGE_GROUPS; ++u) {
+            const u32x4 w0 = *(const u32x4 *)(stage + rd_off[2 * u]);
+            const u32x4 w1 = *(const u32x4 *)(stage + rd_off[2 * u + 1]);
+            w.raw[u][0] = w0.x; w.raw[u][1] = w0.y; w.raw[u][2] = w0.z; w.raw[u][3] = w0.w;
+            w.raw[u][4] = w1.x; w.raw[u][5] = w1.y; w.raw[u][6] = w1.z; w.raw[u][7] = w1.w;
+        }
+    };
+    auto consume = [&](int st, const StepWeights &w) {
+        const uint8_t *a_ptr = a_base + (uint32_t)st * a_step;
+        // the step's four scales and four biases: two dwords each out of the lane's registers, at a wave-uniform
+        // index for either strip (groups past the row's end have zero digits; they take whatever the clamped index
+        // yields, a finite value of the row)
+        float scale[STAGE_GROUPS], bias[STAGE_GROUPS];
+        {
+            // register indexing by a wave-uniform index
+            auto pick = [&](const MetaVec &m, int dword) -> uint32_t { return m[dword]; };
+            const int last = MD - 2;
+            const int i0 = 2 * st < last ? 2 * st : last;
+            const int i1 = 2 * (st + strip1_shift) < last ? 2 * (st + strip1_shift) : last;
+            uint32_t s_lo = pick(scales_v, i0), s_hi = pick(scales_v, i0 + 1);
+            uint32_t b_lo = pick(biases_v, i0), b_hi = pick(biases_v, i0 + 1);
+            if (i1 != i0) {                        // uniform
+                const uint32_t s_lo1 = pick(scales_v, i1), s_hi1 = pick(scales_v, i1 + 1);
+                const uint32_t b_lo1 = pick(biases_v, i1), b_hi1 = pick(biases_v, i1 + 1);
+                s_lo = h ? s_lo1 : s_lo; s_hi = h ? s_hi1 : s_hi;
+                b_lo = h ? b_lo1 : b_lo; b_hi = h ? b_hi1 : b_hi;
+            }
+            scale[0] = __uint_as_float(s_lo << 16); scale[1] = __uint_as_float(s_lo & 0xffff0000u);
+            scale[2] = __uint_as_float(s_hi << 16); scale[3] = __uint_as_float(s_hi & 0xffff0000u);
+            bias[0] = __uint_as_float(b_lo << 16); bias[1] = __uint_as_float(b_lo & 0xffff0000u);
+            bias[2] = __uint_as_float(b_hi << 16); bias[3] = __uint_as_float(b_hi & 0xffff0000u);
+        }
+        // (power of two, sum) of the step's four groups, per token.  Read as native vectors: an LDS read without type
+        // information (a struct such as float4, or reads the compiler merged itself) is made to wait for every
+        // outstanding direct-to-LDS load
+        float xm[T][2 * STAGE_GROUPS];
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const f32x4 lo4 = *(const f32x4 *)(xm_ptr + 2 * (t * 2 * SG + st * STAGE_GROUPS));
+            const f32x4 hi4 = *(const f32x4 *)(xm_ptr + 2 * (t * 2 * SG + st * STAGE_GROUPS) + 4);
+            xm[t][0] = lo4.x; xm[t][1] = lo4.y; xm[t][2] = lo4.z; xm[t][3] = lo4.w;
+            xm[t][4] = hi4.x; xm[t][5] = hi4.y; xm[t][6] = hi4.z; xm[t][7] = hi4.w;
+        }
+        // The four groups advance together through the four quarters, so that consecutive matrix instructions belong
+        // to different accumulators and never wait for each other.
+        v16i d[STAGE_GROUPS];
+#pragma unroll
+        for (int u = 0; u < STAGE_GROUPS; ++u)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) d[u][i] = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v4i a[STAGE_GROUPS];
+#pragma unroll
+            for (int u = 0; u < STAGE_GROUPS; ++u) a[u] = *(const v4i *)(a_ptr + u * GROUP_IMAGE + j * 64);
+#pragma unroll
+            for (int u = 0; u < STAGE_GROUPS; ++u) {
+                const uint32_t lo = w.raw[u][2 * j], hi = w.raw[u][2 * j + 1];
+                v4i b;
+                b.x = (int)(lo & 0x0f0f0f0fu);
+                b.y = (int)((lo >> 4) & 0x0f0f0f0fu);
+                b.z = (int)(hi & 0x0f0f0f0fu);
+                b.w = (int)((hi >> 4) & 0x0f0f0f0fu);
+                d[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[u], b, d[u], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < STAGE_GROUPS; ++u) {
+            const float bias_u = no_bias ? 0.0f : bias[u];
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                const int lo = d[u][4 * t] + (d[u][4 * t + 1] << 8);
+                const int hi = d[u][4 * t + 2] + (d[u][4 * t + 3] << 8);
+                const float f = __builtin_fmaf((float)hi, 65536.0f, (float)lo);
+                acc[t] = __builtin_fmaf(scale[u] * xm[t][2 * u], f, acc[t]);
+                acc[t] = __builtin_fmaf(bias_u, xm[t][2 * u + 1], acc[t]);
+            }
+        }
+    };
+
+    // the two strips of a row meet
+    auto finish_block = [&]() {
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const float other = __shfl_xor(acc[t], 32, 64);
+            if (lane < rows_here) job.y[(size_t)t * job.y_stride + row_base + lane] = acc[t] + other;
+        }
+    };
+
+    // ---------------------------------------------------------------- activations -> digit planes (all waves)
+    auto build_image = [&]() {
+        for (int i = tid; i < ZERO_BYTES / 4; i += THREADS) ((uint32_t *)zero_lds)[i] = 0u;
+        // one thread per four columns; the sixteen threads of a group are sixteen neighbouring lanes
+        const int items = T * 2 * SG * 16;
+        // items is a multiple of 64, so a wave is inside or outside the loop as a whole (the shuffles need that)
+        for (int item = tid; item < items; item += THREADS) {
+            const int q16 = item & 15;
+            const int g = (item >> 4) % (2 * SG);      // slot of the group in the image = its index in the row
+            const int t = (item >> 4) / (2 * SG);
+            const bool valid = g < ngrp;               // slots past the row's end hold zero digits
+            float xv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (valid) {
+                const float *src = job.x + (size_t)t * job.x_stride + (size_t)g * 64 + 4 * q16;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) xv[k] = src[k];
+            }
+            float gmax = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(xv[0]), __builtin_fabsf(xv[1])),
+                                         __builtin_fmaxf(__builtin_fabsf(xv[2]), __builtin_fabsf(xv[3])));
+            double gsum = ((double)xv[0] + (double)xv[1]) + ((double)xv[2] + (double)xv[3]);
+            // a NaN does not survive the maximum, but the sum keeps it, and with it every output of the token
+#pragma unroll
+            for (int d = 1; d < 16; d <<= 1) {
+                gmax = __builtin_fmaxf(gmax, __shfl_xor(gmax, d, 64));
+                gsum = gsum + __shfl_xor(gsum, d, 64);
+            }
+            // gmax in [2^E, 2^(E+1)): digits of rint(x * 2^(29 - E)); tiny groups are pinned at E = -97
+            int eb = (int)((__float_as_uint(gmax) >> 23) & 0xffu);
+            eb = eb < 30 ? 30 : (eb > 254 ? 254 : eb);
+            const float up = __uint_as_float((uint32_t)(283 - eb) << 23);      // 2^(29 - E)
+            const float down = __uint_as_float((uint32_t)(eb - 29) << 23);     // 2^(E - 29)
+            int d0[4], d1[4], d2[4], d3[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                float scaled = xv[k] * up;
+                scaled = __builtin_fminf(__builtin_fmaxf(scaled, -1073741824.0f), 1073741824.0f);   // non-finite input: any digits
+                int I = __float2int_rn(scaled);
+                d0[k] = (int)(int8_t)I; I = (I - d0[k]) >> 8;
+                d1[k] = (int)(int8_t)I; I = (I - d1[k]) >> 8;
+                d2[k] = (int)(int8_t)I; I = (I - d2[k]) >> 8;
+                d3[k] = I;
+            }
+            // byte order inside a sixteen-column quarter = the order the code extraction yields:
+            // columns 0 2 4 6 | 1 3 5 7 | 8 10 12 14 | 9 11 13 15
+            const int j = q16 >> 2, c4 = (q16 & 3) * 4;
+            const int pos = (c4 & 8) + ((c4 & 4) >> 1);
+            uint8_t *slot = img_lds + ((size_t)(t * 2 * SG + g) * 16 + j * 4) * 16 + pos;
+            const int *planes[4] = {d0, d1, d2, d3};
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const int *d = planes[p];
+                *(uint16_t *)(slot + p * 16) = (uint16_t)((d[0] & 0xff) | ((d[2] & 0xff) << 8));
+                *(uint16_t *)(slot + p * 16 + 4) = (uint16_t)((d[1] & 0xff) | ((d[3] & 0xff) << 8));
+            }
+            if (q16 == 0) {
+                xm_lds[2 * (t * 2 * SG + g)] = valid ? down : 0.0f;
+                xm_lds[2 * (t * 2 * SG + g) + 1] = valid ? (float)gsum : 0.0f;
+            }
+        }
+    };
+
+    // ---------------------------------------------------------------- main loop
+    // Weight loads go out in step order, LOADS_PER_STEP per step, STAGES steps ahead: a step's slot is refilled as
+    // soon as its weights sit in registers, before its arithmetic.  When step g is waited for, what may still be in
+    // flight is exactly the steps behind it: direct-to-LDS loads complete in issue order.  The first loads do not
+    // depend on the activations: they are on their way while the digit planes are built.  The scales and biases, the
+    // only loads that return to registers, are waited for with everything that is in flight at that moment, once.
+    // Blocks start their walk over the row at different steps: rows whose length is a power of two put the same
+    // step of every row on the same memory channels, and waves that all began at step 0 would queue there.
+    const int first_step = (int)(((unsigned)blockIdx.x * WAVES + wave) % (unsigned)nstage);
+    auto step_of = [&](int g) { const int st = g + first_step; return st < nstage ? st : st - nstage; };
+    if (has_rows) {
+        issue_meta();
+#pragma unroll
+        for (int g = 0; g < STAGES; ++g)
+            if (g < total_steps) issue_step(step_of(g), g);
+    }
+    if (!(L.debug & 2)) build_image();
+    __syncthreads();
+    if (!has_rows) return;                           // no barrier below
+#pragma unroll
+    for (int q = 0; q < MD / 4; ++q) {
+        wait_meta(scales_r.q[q]);
+        wait_meta(biases_r.q[q]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            scales_v[4 * q + e] = scales_r.q[q][e];
+            biases_v[4 * q + e] = biases_r.q[q][e];
+        }
+    }
+
+    for (int base = 0; base < total_steps; base += STAGES) {
+        const bool more = static_steps(std::make_integer_sequence<int, STAGES>{}, [&](auto step_in_turn) {
+            constexpr int r = decltype(step_in_turn)::value;       // ring slot of step base + r
+            const int g = base + r;
+            if (g >= total_steps) return false;
+            if (!(L.debug & 4)) {
+                const int behind = total_steps - 1 - g < STAGES - 1 ? total_steps - 1 - g : STAGES - 1;
+                if (L.debug & 1) wait_vm<0>();
+                else if (behind == 0) wait_vm<0>();
+                else if (behind == 1) wait_vm<LOADS_PER_STEP>();
+                else if (behind == 2) wait_vm<2 * LOADS_PER_STEP>();
+                else wait_vm<3 * LOADS_PER_STEP>();
+            }
+            StepWeights w;
+            fetch(r, w);
+            // the reads have returned before the slot is written again
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (!(L.debug & 4) && g + STAGES < total_steps) issue_step(step_of(g + STAGES), r);
+            if (!(L.debug & 8)) consume(step_of(g), w);
+            return true;
+        });
+        if (!more) break;
+    }
+    finish_block();
+}
+
+size_t dot_lds_bytes(int cols, int tokens, int waves, int stages) {
+    const int sg = dot_steps(cols >> 6) * STAGE_GROUPS;
+    return (size_t)waves * stages * STEP_LDS + ZERO_BYTES + (size_t)tokens * 2 * sg * (GROUP_IMAGE + 8);
+}
+
+template <int T, int WAVES, int STAGES, int MD>
+int launch_shape(const Q4DotLaunch &L, hipStream_t stream) {
+    const size_t lds = dot_lds_bytes(L.cols, T, WAVES, STAGES);
+    static size_t raised = 0;                 // per instantiation: the largest dynamic LDS size asked for so far
+    if (lds > raised) {
+        if (hipFuncSetAttribute((const void *)q4_dot_kernel<T, WAVES, STAGES, MD>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds) != hipSuccess)
+            return -1;
+        raised = lds;
+    }
+    hipLaunchKernelGGL((q4_dot_kernel<T, WAVES, STAGES, MD>), dim3(L.total_wgs), dim3(WAVES * 64), lds, stream, L);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int env_int(const char *name, int fallback) {
+    const char *e = getenv(name);
+    return e ? atoi(e) : fallback;
+}
+
+// (waves per workgroup, steps of LDS per wave); `resident` workgroups share a compute unit's LDS
+struct Candidate { int waves, stages, resident; };
+constexpr Candidate CANDIDATES[] = {{4, 2, 2}, {3, 2, 2}, {8, 2, 1}, {7, 2, 1}, {6, 2, 1}, {5, 3, 1}, {4, 4, 1}, {4, 3, 1},
+                                    {4, 2, 1}, {2, 2, 2}};
+
+}  // namespace
+
+bool q4_dot_takes(int cols) { return cols >= DOT_MIN_COLS && cols <= DOT_MAX_COLS && (cols & 255) == 0; }
+
+int q4_dot_tokens_per_pass(int cols) {
+    // what fits beside four waves' weight steps in 160 KiB of LDS
+    for (int t = 4; t >= 1; --t)
+        if (dot_lds_bytes(cols, t, 4, 2) <= DOT_LDS_LIMIT) return t;
+    return 0;
+}
+
+DotShape q4_dot_shape(int cols, int tokens) {
+    static const int want_waves = env_int("SALT_MI355_DOT_WAVES", 0), want_stages = env_int("SALT_MI355_DOT_STAGES", 0);
+    // in order of preference; the first that fits the LDS beside the digit planes is taken
+    for (const Candidate &c : CANDIDATES)
+        if ((want_waves == 0 || want_waves == c.waves) && (want_stages == 0 || want_stages == c.stages) &&
+            dot_lds_bytes(cols, tokens, c.waves, c.stages) * c.resident <= DOT_LDS_LIMIT)
+            return DotShape{c.waves, c.stages};
+    return DotShape{4, 2};
+}
+
+int q4_dot_launch(const Q4DotLaunch &launch, const DotShape &shape, hipStream_t stream) {
+    Q4DotLaunch L = launch;
+    if (L.total_wgs < 1 || L.tokens < 1 || L.tokens > 4 || !q4_dot_takes(L.cols)) return -1;
+    if (dot_lds_bytes(L.cols, L.tokens, shape.waves, shape.stages) > DOT_LDS_LIMIT) return -1;
+    static const int debug_env = env_int("SALT_MI355_DOT_DEBUG", 0);
+    L.debug = debug_env;
+    const int md = L.cols <= 4096 ? 16 : 32;
+#define DOT_CASE(TT, WW, SS) \
+    if (L.tokens == TT && shape.waves == WW && shape.stages == SS) \
+        return md == 16 ? launch_shape<TT, WW, SS, 16>(L, stream) : launch_shape<TT, WW, SS, 32>(L, stream)
+#define DOT_CASES(TT) DOT_CASE(TT, 8, 2); DOT_CASE(TT, 7, 2); DOT_CASE(TT, 6, 2); DOT_CASE(TT, 5, 3); DOT_CASE(TT, 4, 4); \
+                      DOT_CASE(TT, 4, 3); DOT_CASE(TT, 4, 2); DOT_CASE(TT, 3, 2); DOT_CASE(TT, 2, 2)
+    DOT_CASES(1); DOT_CASES(2); DOT_CASES(3); DOT_CASES(4);
+#undef DOT_CASES
+#undef DOT_CASE
+    return -1;
+}
+
+}  // namespace mi355

@@ -114,7 +114,7 @@ __device__ __forceinline__ void nibbles_to_f32(uint32_t w, float (&q)[8]) {
 // One packed word of a lane.  Nibble n belongs to block (first_block + n / S)
 // of its scale group and to the lane's chain (n % S).  x holds the wave's
 // activations in SGPRs: x[token][xbase + block * S + chain].
-template <int S, int NB, int XN, int NNIB, bool SLOW, bool FUSED>
+template <int S, int NB, int XN, int NNIB, bool SLOW>
 __device__ __forceinline__ void consume_word(uint32_t w, int first_block, int xbase, float scale, float bias,
                                              const float (&x)[NB][XN], float code_scale, float (&acc)[NB][S]) {
     float q[8];
@@ -134,12 +134,8 @@ __device__ __forceinline__ void consume_word(uint32_t w, int first_block, int xb
 #pragma unroll
         for (int t = 0; t < NB; ++t) {
             const float xv = x[t][xbase + blk * S + ch];
-            if (FUSED) {
-                acc[t][ch] = __builtin_fmaf(wgt, xv, acc[t][ch]);
-            } else {
-                const float p = wgt * xv;
-                acc[t][ch] = acc[t][ch] + p;
-            }
+            const float p = wgt * xv;
+            acc[t][ch] = acc[t][ch] + p;
         }
     }
 }
@@ -161,7 +157,7 @@ constexpr int x_batch_groups(int S, int NB) {
 // gelu_tanh(gate) * up are computed into LDS and reach the VALU in vector
 // registers (every lane reads the same words) instead of through scalar loads;
 // 3 = the same activation prologue for jobs of the launch (one token each).
-template <int S, int NB, bool FUSED, int CB, int PRO = 0>
+template <int S, int NB, int CB, int PRO = 0>
 __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L) {
     constexpr int CHUNK_BLOCKS = CB;
     constexpr int CHUNK_GROUPS = CB / 2;                   // 64-column scale groups per step
@@ -183,7 +179,7 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
     __shared__ __attribute__((aligned(16))) float m_lds[2 * M_STAGE];
     __shared__ __attribute__((aligned(16))) float x_lds[PRO >= 2 ? MOE_FUSE_MAX_ROUTED : 4];
     __shared__ int slow_flag;
-    static_assert(PRO == 0 || (NB == 1 && !FUSED), "the MoE prologues serve the single-token bit-exact kernel");
+    static_assert(PRO == 0 || NB == 1, "the MoE prologues serve the single-token kernel");
     static_assert(PRO != 1 || (sizeof(RouterShared) <= W_BYTES && THREADS >= MOE_FUSE_MAX_EXPERTS),
                   "the router prologue borrows the weight staging memory and one thread per expert");
 
@@ -421,10 +417,10 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
                     float scale, bias;
                     fetch(batch * XG + gl, w0, w1, scale, bias);
                     if (S == 8) {
-                        consume_word<S, NB, XN, 8, false, FUSED>(w0, 0, gl * 2 * S, scale, bias, xq, L.code_scale, acc);
-                        consume_word<S, NB, XN, 8, false, FUSED>(w1, 1, gl * 2 * S, scale, bias, xq, L.code_scale, acc);
+                        consume_word<S, NB, XN, 8, false>(w0, 0, gl * 2 * S, scale, bias, xq, L.code_scale, acc);
+                        consume_word<S, NB, XN, 8, false>(w1, 1, gl * 2 * S, scale, bias, xq, L.code_scale, acc);
                     } else {
-                        consume_word<S, NB, XN, (S == 4 ? 8 : 4), false, FUSED>(w0, 0, gl * 2 * S, scale, bias, xq,
+                        consume_word<S, NB, XN, (S == 4 ? 8 : 4), false>(w0, 0, gl * 2 * S, scale, bias, xq,
                                                                                  L.code_scale, acc);
                     }
                 }
@@ -442,10 +438,10 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
                         float scale, bias;
                         fetch(g + gl, w0, w1, scale, bias);
                         if (S == 8) {
-                            consume_word<S, NB, XN, 8, false, FUSED>(w0, 0, gl * 2 * S, scale, bias, xq, L.code_scale, acc);
-                            consume_word<S, NB, XN, 8, false, FUSED>(w1, 1, gl * 2 * S, scale, bias, xq, L.code_scale, acc);
+                            consume_word<S, NB, XN, 8, false>(w0, 0, gl * 2 * S, scale, bias, xq, L.code_scale, acc);
+                            consume_word<S, NB, XN, 8, false>(w1, 1, gl * 2 * S, scale, bias, xq, L.code_scale, acc);
                         } else {
-                            consume_word<S, NB, XN, (S == 4 ? 8 : 4), false, FUSED>(w0, 0, gl * 2 * S, scale, bias, xq,
+                            consume_word<S, NB, XN, (S == 4 ? 8 : 4), false>(w0, 0, gl * 2 * S, scale, bias, xq,
                                                                                      L.code_scale, acc);
                         }
                     }
@@ -459,18 +455,18 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
                 if (slow) {
                     scale = bf16_to_f32(scales16[(uint32_t)my_row * ngrp + ck * CHUNK_GROUPS + g]);
                     if (S == 8) {
-                        consume_word<S, NB, XN, 8, true, FUSED>(w0, 0, 0, scale, bias, xq, L.code_scale, acc);
-                        consume_word<S, NB, XN, 8, true, FUSED>(w1, 1, 0, scale, bias, xq, L.code_scale, acc);
+                        consume_word<S, NB, XN, 8, true>(w0, 0, 0, scale, bias, xq, L.code_scale, acc);
+                        consume_word<S, NB, XN, 8, true>(w1, 1, 0, scale, bias, xq, L.code_scale, acc);
                     } else {
-                        consume_word<S, NB, XN, (S == 4 ? 8 : 4), true, FUSED>(w0, 0, 0, scale, bias, xq,
+                        consume_word<S, NB, XN, (S == 4 ? 8 : 4), true>(w0, 0, 0, scale, bias, xq,
                                                                                 L.code_scale, acc);
                     }
                 } else {
                     if (S == 8) {
-                        consume_word<S, NB, XN, 8, false, FUSED>(w0, 0, 0, scale, bias, xq, L.code_scale, acc);
-                        consume_word<S, NB, XN, 8, false, FUSED>(w1, 1, 0, scale, bias, xq, L.code_scale, acc);
+                        consume_word<S, NB, XN, 8, false>(w0, 0, 0, scale, bias, xq, L.code_scale, acc);
+                        consume_word<S, NB, XN, 8, false>(w1, 1, 0, scale, bias, xq, L.code_scale, acc);
                     } else {
-                        consume_word<S, NB, XN, (S == 4 ? 8 : 4), false, FUSED>(w0, 0, 0, scale, bias, xq,
+                        consume_word<S, NB, XN, (S == 4 ? 8 : 4), false>(w0, 0, 0, scale, bias, xq,
                                                                                  L.code_scale, acc);
                     }
                 }
@@ -566,19 +562,19 @@ int env_wide_limit() {
     return cached;
 }
 
-template <int S, bool FUSED>
+template <int S>
 int launch_tiles(const Q4Launch &L, hipStream_t stream) {
     const dim3 grid(L.total_tiles), block((32 / S) * 64);
     // One token with few tiles: a workgroup has its compute unit to itself and stages twice as much per step.
-    if (L.tokens == 1 && !FUSED && S <= 4 && L.total_tiles <= env_wide_limit()) {
-        hipLaunchKernelGGL((q4_tile_kernel<S, 1, false, 32>), grid, block, 0, stream, L);
+    if (L.tokens == 1 && S <= 4 && L.total_tiles <= env_wide_limit()) {
+        hipLaunchKernelGGL((q4_tile_kernel<S, 1, 32>), grid, block, 0, stream, L);
         return hipGetLastError() == hipSuccess ? 0 : -1;
     }
     switch (L.tokens) {
-        case 1: hipLaunchKernelGGL((q4_tile_kernel<S, 1, FUSED, 16>), grid, block, 0, stream, L); break;
-        case 2: hipLaunchKernelGGL((q4_tile_kernel<S, 2, FUSED, 16>), grid, block, 0, stream, L); break;
-        case 3: hipLaunchKernelGGL((q4_tile_kernel<S, 3, FUSED, 16>), grid, block, 0, stream, L); break;
-        case 4: hipLaunchKernelGGL((q4_tile_kernel<S, 4, FUSED, 16>), grid, block, 0, stream, L); break;
+        case 1: hipLaunchKernelGGL((q4_tile_kernel<S, 1, 16>), grid, block, 0, stream, L); break;
+        case 2: hipLaunchKernelGGL((q4_tile_kernel<S, 2, 16>), grid, block, 0, stream, L); break;
+        case 3: hipLaunchKernelGGL((q4_tile_kernel<S, 3, 16>), grid, block, 0, stream, L); break;
+        case 4: hipLaunchKernelGGL((q4_tile_kernel<S, 4, 16>), grid, block, 0, stream, L); break;
         default: return -1;
     }
     return hipGetLastError() == hipSuccess ? 0 : -1;
@@ -623,17 +619,17 @@ int q4_moe_gate_up_launch(const Q4Launch &launch, hipStream_t stream) {
     if (m.n_experts < 1 || m.n_experts > MOE_FUSE_MAX_EXPERTS || m.topk < 1 || m.topk > m.n_experts ||
         m.topk > ROUTER_MAX_TOPK || m.hidden < 64 || (m.hidden & 63) || m.routed < 64 || (m.routed & 63))
         return -1;
-    L.table = nullptr; L.njobs = 1; L.cols = m.hidden; L.tokens = 1; L.fused = 0;
+    L.table = nullptr; L.njobs = 1; L.cols = m.hidden; L.tokens = 1;
     L.total_tiles = 2 * m.topk * ((m.routed + TILE_ROWS - 1) / TILE_ROWS);
     const dim3 grid(L.total_tiles + 1);                         // the extra workgroup publishes the router's outputs
     // measured at 176 tiles (eight experts of 704 rows): 1024-column steps 29.4 us per decode step, 512-column steps 29.1,
     // four chains per lane 30.4 and 33.4; the wide step is kept for launches that leave half the compute units idle
     if (L.total_tiles <= env_wide_limit() / 2)
-        hipLaunchKernelGGL((q4_tile_kernel<2, 1, false, 32, 1>), grid, dim3(1024), 0, stream, L);
+        hipLaunchKernelGGL((q4_tile_kernel<2, 1, 32, 1>), grid, dim3(1024), 0, stream, L);
     else if (L.total_tiles <= env_wide_limit())
-        hipLaunchKernelGGL((q4_tile_kernel<2, 1, false, 16, 1>), grid, dim3(1024), 0, stream, L);
+        hipLaunchKernelGGL((q4_tile_kernel<2, 1, 16, 1>), grid, dim3(1024), 0, stream, L);
     else
-        hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 16, 1>), grid, dim3(512), 0, stream, L);
+        hipLaunchKernelGGL((q4_tile_kernel<4, 1, 16, 1>), grid, dim3(512), 0, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -643,25 +639,25 @@ int q4_moe_down_launch(const Q4Launch &launch, hipStream_t stream) {
     if (m.topk < 1 || m.hidden < 64 || (m.hidden & 63) || m.routed < 64 || (m.routed & 63) ||
         m.routed > MOE_FUSE_MAX_ROUTED)
         return -1;
-    L.table = nullptr; L.njobs = 1; L.cols = m.routed; L.tokens = 1; L.fused = 0;
+    L.table = nullptr; L.njobs = 1; L.cols = m.routed; L.tokens = 1;
     L.total_tiles = m.topk * ((m.hidden + TILE_ROWS - 1) / TILE_ROWS);
     const dim3 grid(L.total_tiles);
     // measured at 352 tiles (eight experts of 2816 rows): two chains per lane 31.4 us per decode step, four 29.4,
     // eight 31.4, wide steps 32.7 and 34.5
     if (L.total_tiles <= env_wide_limit())
-        hipLaunchKernelGGL((q4_tile_kernel<2, 1, false, 32, 2>), grid, dim3(1024), 0, stream, L);
+        hipLaunchKernelGGL((q4_tile_kernel<2, 1, 32, 2>), grid, dim3(1024), 0, stream, L);
     else
-        hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 16, 2>), grid, dim3(512), 0, stream, L);
+        hipLaunchKernelGGL((q4_tile_kernel<4, 1, 16, 2>), grid, dim3(512), 0, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
 int q4_activated_launch(const Q4Launch &L, hipStream_t stream) {
-    if (L.total_tiles < 1 || L.tokens != 1 || L.fused || L.cols < 64 || (L.cols & 63) || L.cols > MOE_FUSE_MAX_ROUTED) return -1;
+    if (L.total_tiles < 1 || L.tokens != 1 || L.cols < 64 || (L.cols & 63) || L.cols > MOE_FUSE_MAX_ROUTED) return -1;
     const dim3 grid(L.total_tiles);
     if (L.total_tiles <= env_wide_limit())
-        hipLaunchKernelGGL((q4_tile_kernel<2, 1, false, 32, 3>), grid, dim3(1024), 0, stream, L);
+        hipLaunchKernelGGL((q4_tile_kernel<2, 1, 32, 3>), grid, dim3(1024), 0, stream, L);
     else
-        hipLaunchKernelGGL((q4_tile_kernel<4, 1, false, 16, 3>), grid, dim3(512), 0, stream, L);
+        hipLaunchKernelGGL((q4_tile_kernel<4, 1, 16, 3>), grid, dim3(512), 0, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -674,18 +670,10 @@ int q4_launch(const Q4Launch &L, int chains_per_lane, hipStream_t stream) {
         // 256 tiles, 20.7 against 15.2 at 320, 23.3 against 17.6 at 512; eight chains per lane never do).
         S = L.total_tiles > env_wide_limit() ? 4 : 2;
     }
-    if (L.fused) {
-        switch (S) {
-            case 8: return launch_tiles<8, true>(L, stream);
-            case 4: return launch_tiles<4, true>(L, stream);
-            case 2: return launch_tiles<2, true>(L, stream);
-            default: return -1;
-        }
-    }
     switch (S) {
-        case 8: return launch_tiles<8, false>(L, stream);
-        case 4: return launch_tiles<4, false>(L, stream);
-        case 2: return launch_tiles<2, false>(L, stream);
+        case 8: return launch_tiles<8>(L, stream);
+        case 4: return launch_tiles<4>(L, stream);
+        case 2: return launch_tiles<2>(L, stream);
         default: return -1;
     }
 }

@@ -89,8 +89,9 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_event_elapsed_ms, i, vp, vp, C.POINTER(f))
     _sig(lib.salt_mi355_q4_matvec_dev, i, vp, vp, vp, i, i, i, vp, vp, i, vp)
     _sig(lib.salt_mi355_q4_jobs_dev, i, C.POINTER(Q4Job), i, i, i, i, vp)
+    _sig(lib.salt_mi355_q4_matvec_t_dev, i, vp, vp, vp, i, i, i, vp, vp, vp)
+    _sig(lib.salt_mi355_q4_jobs_t_dev, i, C.POINTER(Q4Job), i, i, i, vp)
     _sig(lib.salt_mi355_q4_jobs_activated_dev, i, C.POINTER(Q4Job), i, i, C.c_longlong, vp)
-    _sig(lib.salt_mi355_set_q4_accumulate, i, i)
     _sig(lib.salt_mi355_q4_matmul_workspace_bytes, sz, i, i)
     _sig(lib.salt_mi355_q4_matmul_dev, i, vp, vp, vp, i, i, i, vp, vp, vp, vp)
     _sig(lib.salt_mi355_nvfp4_qdq_dev, i, vp, i, i, f, vp, vp, vp, vp, vp)
@@ -176,10 +177,10 @@ class DeviceBuffer:
 
 
 def q4_matvec(vals: np.ndarray, scales: np.ndarray, biases: np.ndarray | None, R: int, C_: int,
-              xs: np.ndarray, chains: int = 0, value_offset: int = 0) -> np.ndarray:
-    """Host-array convenience around salt_mi355_q4_matvec_dev: uploads, runs on
-    the library stream, downloads ys[B, R].  value_offset shifts the packed values by that many bytes inside their
-    device allocation (alignment cases)."""
+              xs: np.ndarray, chains: int = 0, value_offset: int = 0, tolerance_class: bool = False) -> np.ndarray:
+    """Host-array convenience around salt_mi355_q4_matvec_dev (or, with tolerance_class, salt_mi355_q4_matvec_t_dev):
+    uploads, runs on the library stream, downloads ys[B, R].  value_offset shifts the packed values by that many bytes
+    inside their device allocation (alignment cases)."""
     lib = init()
     xs = np.ascontiguousarray(xs, np.float32).reshape(-1, C_)
     B = xs.shape[0]
@@ -189,8 +190,12 @@ def q4_matvec(vals: np.ndarray, scales: np.ndarray, biases: np.ndarray | None, R
     dx = DeviceBuffer.from_host(xs)
     dy = DeviceBuffer(B * R * 4, fill=0xFF)
     stream = lib.salt_mi355_stream()
-    check(lib.salt_mi355_q4_matvec_dev(dv.at(value_offset), ds.ptr, db.ptr if db else None, R, C_, B, dx.ptr, dy.ptr,
-                                       chains, stream), "q4_matvec_dev")
+    if tolerance_class:
+        check(lib.salt_mi355_q4_matvec_t_dev(dv.at(value_offset), ds.ptr, db.ptr if db else None, R, C_, B, dx.ptr,
+                                             dy.ptr, stream), "q4_matvec_t_dev")
+    else:
+        check(lib.salt_mi355_q4_matvec_dev(dv.at(value_offset), ds.ptr, db.ptr if db else None, R, C_, B, dx.ptr, dy.ptr,
+                                           chains, stream), "q4_matvec_dev")
     check(lib.salt_mi355_stream_sync(stream), "sync")
     return dy.to_host(np.float32).reshape(B, R)
 

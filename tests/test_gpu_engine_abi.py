@@ -149,6 +149,27 @@ def test_resource_lifecycle_matvec_batch_and_stats(eng, oracle, pkg):
     assert usage.described_resources == 0 and usage.device_copied_weight_bytes == 0
 
 
+def test_batch_of_unregistered_matrices_larger_than_one_copy_chunk(eng, oracle, pkg):
+    """Three matrices outside every resource, 78 MB together: each is copied for the call, and the copy of the first
+    must still be in place when the launch runs although the third does not fit the chunk that holds the first."""
+    R, Cc = 16384, 2816
+    eng.salt_gpu_set_mapped_only(0)
+    tensors = [synth.q4_tensor(R, Cc, 300 + j) for j in range(3)]
+    xs = synth.activations(Cc, 3, 310)
+    ys = [np.zeros(R, np.float32) for _ in range(3)]
+    rc = eng.salt_gpu_q4_batch(abi.ptr_array([t[0] for t in tensors]), abi.ptr_array([t[1] for t in tensors]),
+                               abi.ptr_array([t[2] for t in tensors]), abi.ptr_array([xs[j] for j in range(3)]),
+                               abi.ptr_array(ys), abi.ptr_array([t[0] for t in tensors]), (C.c_int * 3)(R, R, R), Cc, 3)
+    assert rc == 0, err(pkg)
+    for j, (vals, scales, biases) in enumerate(tensors):
+        assert np.array_equal(bits(ys[j]), bits(q4_want(oracle, vals, scales, biases, R, Cc, xs[j])[0])), j
+    # the next call starts over in the copy memory and still computes from its own weights
+    lv, ls, lb = synth.q4_tensor(64, 128, 3)
+    lx = synth.activations(128, 1, 4)[0]; ly = np.zeros(64, np.float32)
+    assert eng.salt_gpu_q4_matvec(ptr(lv), ptr(ls), ptr(lb), 64, 128, ptr(lx), ptr(ly)) == 0, err(pkg)
+    assert np.array_equal(bits(ly), bits(q4_want(oracle, lv, ls, lb, 64, 128, lx)[0]))
+
+
 def test_bounded_window_and_expert_layer_resource(eng, oracle, pkg):
     trunk = Trunk([(128, 256), (64, 256)], 21)
     assert eng.salt_gpu_weight_resource_describe(TRUNK, 3, trunk.base, trunk.blob.nbytes) == 0
