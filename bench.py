@@ -3,7 +3,9 @@
 
 A step is one pass of the decode-shape sweep (BASELINE.json configs[1], batch
 1): for each (K, N) in {(2816, 2816), (2816, 16384), (8192, 2816)} one launch
-of the bit-exact Q4 kernel over G distinct weight instances resident in HBM
+of the tolerance-class Q4 kernel (per-group affine form with exact integer dot
+products; stated bound in include/salt_gpu_mi355.h) over G distinct weight
+instances resident in HBM
 (G chosen so that every launch streams more than the 256 MB Infinity Cache can
 hold), the way the engine's batched entry point dispatches many matrices at
 once (reference salt_gpu_q4_batch, include/salt/gpu.h:83).  `value` is the
@@ -14,8 +16,11 @@ region starts.
 The JSON line also carries the roofline of the dominant kernel (achieved HBM
 GB/s against 8 TB/s), the same sweep timed on the host cores with the
 reference's own C kernel when oracle/_ref is present (else the checker's
-port), and, under "extra", the MoE decode layer-step, the NVFP4 matvec and the
-batch-4 sweep.
+port), and, under "extra", the same sweep on the bit-exact kernel, the MoE
+decode layer-step, the NVFP4 matvec and the batch-4 sweeps.
+
+--only NAME runs a single leg (sweep, sweep-exact, moe, nvfp4, nvfp4-t, copy): what the
+rocprofv3 commands in profiles/ use.
 """
 from __future__ import annotations
 
@@ -36,9 +41,13 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
 SWEEP = [(2816, 2816), (16384, 2816), (2816, 8192)]        # (R, C) = (N, K)
 INSTANCE_BYTES = 640e6                                      # distinct weight bytes per launch
-# HBM bytes one launch of the default workload moves, from FETCH_SIZE / WRITE_SIZE counter runs scaled by a copy of
-# known size (profiles/q4_tile_kernel_decode_sweep_b1.md); valid for the default instance counts only.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 661_320_000
+# HBM bytes one launch of the default workload moves (mean of the three launches), from FETCH_SIZE / WRITE_SIZE counter
+# runs scaled by a copy of known size; taken from the profile summary named beside it, for the default instance
+# counts only.  bench.py does not measure it: it reports it with its source.
+TRAFFIC_FROM_PROFILE = {
+    "q4_dot_kernel": (657_200_000, "profiles/q4_dot_kernel_decode_sweep_b1.md"),
+    "q4_tile_kernel": (661_320_000, "profiles/q4_tile_kernel_decode_sweep_b1.md"),
+}
 
 
 class Events:
@@ -59,9 +68,10 @@ class Events:
 class Q4Sweep:
     """The three decode shapes, G instances each, one multi-job launch per shape."""
 
-    def __init__(self, gpu, synth, tokens: int, distinct: int = 0):
-        """distinct > 0: the same number of jobs, but only that many weight instances in memory (cache-warm)."""
-        self.gpu, self.lib, self.tokens = gpu, gpu.load(), tokens
+    def __init__(self, gpu, synth, tokens: int, distinct: int = 0, exact: bool = False):
+        """distinct > 0: the same number of jobs, but only that many weight instances in memory (cache-warm).
+        exact: the bit-exact kernel (salt_mi355_q4_jobs_dev) instead of the tolerance-class one."""
+        self.gpu, self.lib, self.tokens, self.exact = gpu, gpu.load(), tokens, exact
         self.launches, self.keep = [], []
         self.bytes_per_step = 0
         for seed, (R, Cc) in enumerate(SWEEP):
@@ -88,7 +98,10 @@ class Q4Sweep:
 
     def step(self, stream):
         for jobs, G, Cc in self.launches:
-            rc = self.lib.salt_mi355_q4_jobs_dev(jobs, G, Cc, self.tokens, 0, stream)
+            if self.exact:
+                rc = self.lib.salt_mi355_q4_jobs_dev(jobs, G, Cc, self.tokens, 0, stream)
+            else:
+                rc = self.lib.salt_mi355_q4_jobs_t_dev(jobs, G, Cc, self.tokens, stream)
             if rc != 0:
                 raise RuntimeError(self.lib.salt_mi355_last_error().decode())
 
@@ -219,6 +232,60 @@ def cpu_other_configs(synth, pool, cores: int, budget_s: float = 3.0):
     return out
 
 
+def copy_leg(gpu, lib, stream, events):
+    """A 512 MiB device-to-device copy: the known-size transfer that calibrates FETCH_SIZE / WRITE_SIZE."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMemcpyAsync.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
+    n = 512 << 20
+    src, dst = gpu.DeviceBuffer(n, fill=1), gpu.DeviceBuffer(n, fill=0)
+    for _ in range(3):
+        assert hip.hipMemcpyAsync(dst.ptr, src.ptr, n, 3, stream) == 0
+    assert lib.salt_mi355_stream_sync(stream) == 0
+    return {"copy_bytes": n}
+
+
+def sweep_record(lib, sweep, ms, steps, warmup):
+    gbs = sweep.bytes_per_step / (ms * 1e-3) / 1e9
+    launches = len(sweep.launches)
+    bytes_per_launch = sweep.bytes_per_step / launches
+    launch_us = ms * 1e3 / launches
+    kernel = lib.salt_mi355_last_kernel().decode()
+    traffic, source = TRAFFIC_FROM_PROFILE.get(kernel.split("<")[0], (None, None))
+    klass = ("bit-exact kernel" if sweep.exact else
+             "tolerance-class kernel (|err| <= 2^-20 sum (|q s| + 16|s| + |b|)|x| + 1e-6 per output)")
+    return {
+        "metric": "q4_decode_matvec_hbm_gbps", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {
+            "workload": "BASELINE configs[1]: affine-Q4 group-64 decode matvec sweep, batch %d, "
+                        "(K,N) in {(2816,2816),(2816,16384),(8192,2816)}, %s" % (sweep.tokens, klass),
+            "instances_per_shape": [g for _, g, _ in sweep.launches],
+            "launches_per_step": launches,
+            "weights": "one seeded instance per shape replicated at distinct HBM addresses",
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": round(bytes_per_launch / (launch_us * 1e-6) / 1e9, 1),
+            "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(bytes_per_launch / (launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            "traffic": traffic, "traffic_source": source, "kernel": kernel,
+            "bytes_per_launch": int(bytes_per_launch), "launch_us": round(launch_us, 2),
+        },
+    }
+
+
+def run_only(args, gpu, synth, lib, stream, events):
+    """One leg on its own, for profiler runs: the kernels of that leg are the only matvec kernels in the trace."""
+    if args.only == "copy":
+        return copy_leg(gpu, lib, stream, events)
+    if args.only in ("sweep", "sweep-exact", "sweep-b4", "sweep-b4-exact"):
+        sweep = Q4Sweep(gpu, synth, tokens=4 if "b4" in args.only else 1, exact=args.only.endswith("exact"))
+        ms = timed(lib, stream, events, sweep.step, args.warmup, args.steps)
+        return sweep_record(lib, sweep, ms, args.steps, args.warmup)
+    sys.exit("unknown leg: " + args.only)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -226,6 +293,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the MoE / NVFP4 / batch-4 legs")
+    ap.add_argument("--only", default="", help="run one leg: sweep | sweep-exact | sweep-b4 | moe | moe-t | nvfp4 | nvfp4-t | copy")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU mode (run with --gpus 1)")
@@ -237,47 +305,37 @@ def main():
     stream = lib.salt_mi355_stream()
     events = Events(lib, stream)
 
+    if args.only:
+        print(json.dumps(run_only(args, gpu, synth, lib, stream, events)))
+        return
+
     sweep = Q4Sweep(gpu, synth, tokens=1)
     ms = timed(lib, stream, events, sweep.step, args.warmup, args.steps)
-    gbs = sweep.bytes_per_step / (ms * 1e-3) / 1e9
-    launches = len(sweep.launches)
-    bytes_per_launch = sweep.bytes_per_step / launches
-    launch_us = ms * 1e3 / launches
-    result = {
-        "metric": "q4_decode_matvec_hbm_gbps", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {
-            "workload": "BASELINE configs[1]: affine-Q4 group-64 decode matvec sweep, batch 1, "
-                        "(K,N) in {(2816,2816),(2816,16384),(8192,2816)}, bit-exact kernel",
-            "instances_per_shape": [g for _, g, _ in sweep.launches],
-            "launches_per_step": launches,
-            "weights": "one seeded instance per shape replicated at distinct HBM addresses",
-        },
-        "roofline": {
-            "bound": "hbm", "achieved": round(bytes_per_launch / (launch_us * 1e-6) / 1e9, 1),
-            "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(bytes_per_launch / (launch_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH, "kernel": "q4_tile_kernel<4,1,false,16,0>",
-            "bytes_per_launch": int(bytes_per_launch), "launch_us": round(launch_us, 2),
-        },
-    }
-    keep_sweep = sweep
+    result = sweep_record(lib, sweep, ms, args.steps, args.warmup)
 
     if not args.no_extra:
         extra = {}
-        del keep_sweep, sweep
-        # batch 4 of the same sweep
-        s4 = Q4Sweep(gpu, synth, tokens=4)
-        ms4 = timed(lib, stream, events, s4.step, 2, max(5, args.steps // 5))
-        extra["q4_sweep_batch4_gbps"] = round(s4.bytes_per_step / (ms4 * 1e-3) / 1e9, 1)
-        del s4
+        del sweep
+        extra["q4_sweep_class_t_gbps"] = result["value"]
+        # the same sweep on the bit-exact kernel (the reference's 32-chain order and rounding points)
+        sx = Q4Sweep(gpu, synth, tokens=1, exact=True)
+        ms_x = timed(lib, stream, events, sx.step, args.warmup, args.steps)
+        extra["q4_sweep_bit_exact_gbps"] = round(sx.bytes_per_step / (ms_x * 1e-3) / 1e9, 1)
+        extra["q4_sweep_bit_exact_kernel"] = lib.salt_mi355_last_kernel().decode()
+        del sx
+        # batch 4 of the same sweep, both kernels
+        for name, exact in (("q4_sweep_batch4_class_t_gbps", False), ("q4_sweep_batch4_bit_exact_gbps", True)):
+            s4 = Q4Sweep(gpu, synth, tokens=4, exact=exact)
+            ms4 = timed(lib, stream, events, s4.step, 2, max(5, args.steps // 5))
+            extra[name] = round(s4.bytes_per_step / (ms4 * 1e-3) / 1e9, 1)
+            del s4
         # the same batch-1 launches with every job reading one of two weight instances per shape (87 MB in all):
         # served by the 256 MB last-level cache instead of HBM
-        warm = Q4Sweep(gpu, synth, tokens=1, distinct=2)
-        ms_w = timed(lib, stream, events, warm.step, 5, max(20, args.steps))
-        extra["q4_sweep_cache_warm_gbps"] = round(warm.bytes_per_step / (ms_w * 1e-3) / 1e9, 1)
-        del warm
+        for name, exact in (("q4_sweep_cache_warm_class_t_gbps", False), ("q4_sweep_cache_warm_bit_exact_gbps", True)):
+            warm = Q4Sweep(gpu, synth, tokens=1, distinct=2, exact=exact)
+            ms_w = timed(lib, stream, events, warm.step, 5, max(20, args.steps))
+            extra[name] = round(warm.bytes_per_step / (ms_w * 1e-3) / 1e9, 1)
+            del warm
         # MoE decode layer-step, E = 128 top-8, d_model 2816, d_ff 704.  Two layer instances (857 MB of experts) and 32
         # logit vectors per layer taken in turn, so that the selection changes from step to step and the 256 MB
         # last-level cache cannot hold the experts a step reads.

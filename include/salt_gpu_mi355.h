@@ -45,6 +45,8 @@ int salt_mi355_init(void);
 int salt_mi355_shutdown(void);
 /* Last failure recorded by any entry point, for logs; never NULL. */
 const char *salt_mi355_last_error(void);
+/* Name and template arguments of the Q4 matvec kernel that the last launch used (for bench records); never NULL. */
+const char *salt_mi355_last_kernel(void);
 /* Raw decode tables measured at init: fp8[b] is what v_cvt_pk_f32_fp8 returns
  * for byte b; fp4[2*b], fp4[2*b+1] what v_cvt_scalef32_pk_f32_fp4 (scale 1)
  * returns for the low and high nibble of byte b.  Host arrays of 256 / 512. */

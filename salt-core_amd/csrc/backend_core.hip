@@ -20,6 +20,13 @@ void set_error(const char *format, ...) {
     if (getenv("SALT_GPU_DIAG")) fprintf(stderr, "salt-mi355: %s\n", g_state.last_error);
 }
 
+void note_kernel(const char *format, ...) {
+    va_list args;
+    va_start(args, format);
+    vsnprintf(g_state.last_kernel, sizeof g_state.last_kernel, format, args);
+    va_end(args);
+}
+
 int hip_ok(hipError_t status, const char *what) {
     if (status == hipSuccess) return 0;
     set_error("%s: %s", what, hipGetErrorString(status));
@@ -190,6 +197,7 @@ int salt_mi355_shutdown(void) {
 }
 
 const char *salt_mi355_last_error(void) { return g_state.last_error; }
+const char *salt_mi355_last_kernel(void) { return g_state.last_kernel; }
 
 int salt_mi355_converter_tables(float *fp8, float *fp4) {
     if (!g_state.ready || !fp8 || !fp4) return -1;

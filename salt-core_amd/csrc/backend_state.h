@@ -20,6 +20,7 @@ struct State {
     float fp8_table[256] = {0};
     float fp4_table[512] = {0};
     char last_error[256] = {0};
+    char last_kernel[96] = {0};
     // Ring of device + pinned copies of multi-job tables.  A slot is reused
     // only after the event recorded behind its last consumer has completed.
     struct TableSlot {

@@ -7,6 +7,9 @@
 
 namespace mi355 {
 
+// Name and template arguments of the matvec kernel launched last (diagnostics: salt_mi355_last_kernel).
+void note_kernel(const char *format, ...) __attribute__((format(printf, 1, 2)));
+
 // ---------------------------------------------------------------- affine Q4
 
 // One weight matrix against `tokens` activation rows.  All pointers are

@@ -471,6 +471,7 @@ int launch_shape(const Q4DotLaunch &L, hipStream_t stream) {
             return -1;
         raised = lds;
     }
+    note_kernel("q4_dot_kernel<%d,%d,%d,%d>", T, WAVES, STAGES, MD);
     hipLaunchKernelGGL((q4_dot_kernel<T, WAVES, STAGES, MD>), dim3(L.total_wgs), dim3(WAVES * 64), lds, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }

@@ -567,9 +567,11 @@ int launch_tiles(const Q4Launch &L, hipStream_t stream) {
     const dim3 grid(L.total_tiles), block((32 / S) * 64);
     // One token with few tiles: a workgroup has its compute unit to itself and stages twice as much per step.
     if (L.tokens == 1 && S <= 4 && L.total_tiles <= env_wide_limit()) {
+        note_kernel("q4_tile_kernel<%d,1,32,0>", S);
         hipLaunchKernelGGL((q4_tile_kernel<S, 1, 32>), grid, block, 0, stream, L);
         return hipGetLastError() == hipSuccess ? 0 : -1;
     }
+    note_kernel("q4_tile_kernel<%d,%d,16,0>", S, L.tokens);
     switch (L.tokens) {
         case 1: hipLaunchKernelGGL((q4_tile_kernel<S, 1, 16>), grid, block, 0, stream, L); break;
         case 2: hipLaunchKernelGGL((q4_tile_kernel<S, 2, 16>), grid, block, 0, stream, L); break;

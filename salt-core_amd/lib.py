@@ -71,6 +71,7 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_init, i)
     _sig(lib.salt_mi355_shutdown, i)
     _sig(lib.salt_mi355_last_error, C.c_char_p)
+    _sig(lib.salt_mi355_last_kernel, C.c_char_p)
     _sig(lib.salt_mi355_converter_tables, i, vp, vp)
     _sig(lib.salt_mi355_dev_alloc, vp, sz)
     _sig(lib.salt_mi355_dev_free, i, vp)
