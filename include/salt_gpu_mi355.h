@@ -302,6 +302,22 @@ int salt_mi355_moe_decode_step_dev(const void *pool, size_t expert_stride,
                                    const float *x, int *selected, float *weights,
                                    float *expert_out, float *out,
                                    void *workspace, void *stream);
+/* The same layer-step for callers that cannot allocate device memory or pass a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc): the workspace is a static array inside the library, one
+ * per device, SALT_MI355_MOE_STATIC_SCRATCH_BYTES large, and the call allocates
+ * nothing.  It has no counterpart in the reference.  Geometries whose
+ * salt_mi355_moe_workspace_bytes() exceeds the array are refused (-1).  Results
+ * are bit-identical to salt_mi355_moe_decode_step_dev.  status_dev (optional
+ * device int) receives the router status (0 / -1).  All calls on one device
+ * share the array: calls that overlap in time on one device (two streams) race. */
+#define SALT_MI355_MOE_STATIC_SCRATCH_BYTES (1 << 20)
+int salt_mi355_moe_decode_step_static_dev(const void *pool, size_t expert_stride,
+                                          int hidden, int routed, int n_experts, int topk,
+                                          const float *logits, const float *per_expert_scale,
+                                          const float *x, int *selected, float *weights,
+                                          float *expert_out, float *out,
+                                          int *status_dev, void *stream);
 /* Many tokens through the experts of one MoE layer, grouped per expert
  * (reference src/moe_group.c:24-97 validation, :138-184 grouping in ascending
  * expert / token / rank order, :211-224 weighted sum over ranks in rank order

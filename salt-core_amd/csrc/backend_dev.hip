@@ -522,6 +522,69 @@ int salt_mi355_moe_decode_step_dev(const void *pool, size_t expert_stride, int h
     return 0;
 }
 
+// ---------------------------------------------------------------- the same step without a workspace argument
+
+}  // extern "C"
+
+// The workspace of salt_mi355_moe_decode_step_static_dev: one array per device for as long as the process lives.  In
+// host code this name is only a handle for hipGetSymbolAddress; the address the kernels use is looked up once per
+// device and kept below.
+static __device__ __align__(256) unsigned char moe_static_scratch[SALT_MI355_MOE_STATIC_SCRATCH_BYTES];
+static void *moe_static_scratch_address[16];        // by device ordinal; nullptr = not looked up yet
+
+static void *moe_static_scratch_of_current_device() {
+    int device = -1;
+    if (hip_ok(hipGetDevice(&device), "hipGetDevice") != 0) return nullptr;
+    if (device < 0 || device >= 16) { set_error("moe static step: device ordinal %d is out of range", device); return nullptr; }
+    if (!moe_static_scratch_address[device]) {
+        void *address = nullptr;
+        if (hip_ok(hipGetSymbolAddress(&address, HIP_SYMBOL(moe_static_scratch)), "hipGetSymbolAddress") != 0 || !address)
+            return nullptr;
+        moe_static_scratch_address[device] = address;
+    }
+    return moe_static_scratch_address[device];
+}
+
+extern "C" {
+
+int salt_mi355_moe_decode_step_static_dev(const void *pool, size_t expert_stride, int hidden, int routed, int n_experts,
+                                          int topk, const float *logits, const float *per_expert_scale, const float *x,
+                                          int *selected, float *weights, float *expert_out, float *out,
+                                          int *status_dev, void *stream) {
+    if (!g_state.ready) { set_error("moe static step: library not initialised"); return -1; }
+    if (hidden < 1 || routed < 1 || n_experts < 1 || topk < 1) { set_error("moe static step: bad geometry"); return -1; }
+    const size_t need = salt_mi355_moe_workspace_bytes(hidden, routed, n_experts, topk);
+    if (need == 0 || need > (size_t)SALT_MI355_MOE_STATIC_SCRATCH_BYTES) {
+        set_error("moe static step: this geometry needs %zu bytes of workspace, the static one holds %d", need,
+                  SALT_MI355_MOE_STATIC_SCRATCH_BYTES);
+        return -1;
+    }
+    void *scratch = moe_static_scratch_of_current_device();
+    if (!scratch) return -1;
+    if (!pool || !logits || !per_expert_scale || !x || !selected || !weights || !out || ((uintptr_t)pool & 3) ||
+        (expert_stride & 15)) {
+        set_error("moe static step: bad arguments (pool 4-byte aligned, expert stride a multiple of 16)");
+        return -1;
+    }
+    const MoeGeometry g = {hidden, routed, n_experts, topk};
+    const size_t n = (size_t)hidden * (size_t)routed;
+    if (hidden < 64 || (hidden & 63) || routed < 64 || (routed & 63) || expert_stride < 3 * (n / 2 + 4 * (n / 64))) {
+        set_error("moe static step: hidden and routed must be multiples of 64 and the stride must cover a slot");
+        return -1;
+    }
+    MoeWorkspace ws;
+    moe_workspace_carve(g, scratch, &ws);
+    // Every word of the workspace that a launch reads is written earlier in the same step (the status word by the
+    // router, the job tables and the intermediate vectors by their producers): nothing has to start at zero.
+    if (status_dev) ws.status = status_dev;
+    if (moe_decode_step_launch(g, (const uint8_t *)pool, expert_stride, logits, per_expert_scale, x, selected, weights,
+                               expert_out, out, ws, g_state.code_scale, (hipStream_t)stream) != 0) {
+        set_error("moe static step: unsupported geometry or launch failure");
+        return -1;
+    }
+    return 0;
+}
+
 int salt_mi355_moe_activate_dev(const float *gate, const float *up, float *act, size_t n, void *stream) {
     if (!g_state.ready || !gate || !up || !act || n < 1) { set_error("moe activate: bad arguments"); return -1; }
     return moe_activate_launch(gate, up, act, n, (hipStream_t)stream);

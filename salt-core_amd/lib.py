@@ -109,6 +109,7 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_router_topk_dev, i, vp, vp, i, i, i, vp, vp, vp, vp)
     _sig(lib.salt_mi355_moe_workspace_bytes, sz, i, i, i, i)
     _sig(lib.salt_mi355_moe_decode_step_dev, i, vp, sz, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, vp, vp)
+    _sig(lib.salt_mi355_moe_decode_step_static_dev, i, vp, sz, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_moe_prefill_workspace_bytes, sz, i, i, i, i, i)
     _sig(lib.salt_mi355_moe_prefill_dev, i, vp, sz, i, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_moe_activate_dev, i, vp, vp, vp, sz, vp)
