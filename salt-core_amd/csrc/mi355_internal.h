@@ -84,12 +84,13 @@ int q4_uniform_tiles(const Q4Job *table, int njobs);
 // (q4_dot.hip): per scale group  scale * sum q*x + bias * sum x  with the integer dot products exact.
 
 constexpr int DOT_BLOCK_ROWS = 32;         // rows per block; a wave walks whole blocks
-constexpr int DOT_MIN_COLS = 512;          // the streaming kernel takes 512 .. 8192 columns in multiples of 256;
+constexpr int DOT_MIN_COLS = 512;          // the streaming kernel takes 512 .. 8192 columns in multiples of 64;
 constexpr int DOT_MAX_COLS = 8192;         // callers send everything else to the exact kernel
 constexpr int DOT_LDS_LIMIT = 160 * 1024;
 
-// How a launch is cut: waves per workgroup (a wave owns one block of 32 rows), steps of LDS per wave.
-struct DotShape { int waves, stages; };
+// How a launch is cut: waves per workgroup, steps of LDS per wave, parts a row is cut into along its columns
+// (ksplit waves share one block of 32 rows; a workgroup owns waves / ksplit blocks).
+struct DotShape { int waves, stages, ksplit; };
 
 struct Q4DotLaunch {
     Q4Job one;                // used when table == nullptr; tile0 = index of the job's first workgroup
@@ -98,12 +99,13 @@ struct Q4DotLaunch {
     int cols;
     int tokens;               // 1..4, at most q4_dot_tokens_per_pass(cols)
     int total_wgs;
+    int ksplit;               // filled by q4_dot_launch from the shape
     int wgs_per_job;          // > 0 when every job of the table has this many workgroups (workgroup -> job by division)
     int debug;
 };
 bool q4_dot_takes(int cols);
 int q4_dot_tokens_per_pass(int cols);      // 0: the column count does not fit at all
-DotShape q4_dot_shape(int cols, int tokens);
+DotShape q4_dot_shape(int cols, int tokens, long long total_blocks);
 int q4_dot_launch(const Q4DotLaunch &launch, const DotShape &shape, hipStream_t stream);
 
 // ---------------------------------------------------------------- affine Q4 on MFMA (tolerance class)

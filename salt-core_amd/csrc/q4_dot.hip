@@ -149,11 +149,19 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
     const int SG = nstage * STAGE_GROUPS;
     const uint32_t row_bytes = (uint32_t)C >> 1;
     const int whole_steps = (ngrp - SG) / STAGE_GROUPS;            // steps that lie inside the row for both strips
-    // A lane holds the scales of 2 * MD consecutive groups of its row: strip 0 from group 0, strip 1 the row's last
-    // 2 * MD (both cover their strip; the launcher sees to it that the difference is a whole number of steps)
-    const int meta_groups = 2 * MD < ngrp ? 2 * MD : ngrp & ~7;
-    const int strip1_start = ngrp - meta_groups;
-    const int strip1_shift = (SG - strip1_start) / STAGE_GROUPS;   // steps by which strip 1's registers lead its steps
+    // The row may be cut into L.ksplit parts along its columns (launches with few blocks): a wave then walks only the
+    // steps [step_lo, step_hi) of its block, and the parts of a block are added in order at the end.
+    const int ksplit = L.ksplit;
+    const int blocks_per_wg = WAVES / ksplit;
+    const int my_block = wave / ksplit, my_part = wave - my_block * ksplit;
+    const int step_lo = my_part * nstage / ksplit, step_hi = (my_part + 1) * nstage / ksplit;
+    // A lane holds the scales (and biases) of meta_groups consecutive groups of its row in registers: a window that
+    // starts at its strip's first group of the wave's steps, moved left where it would pass the row's end.
+    const int meta_groups = 2 * MD < (ngrp & ~7) ? 2 * MD : ngrp & ~7;
+    const int want0 = step_lo * STAGE_GROUPS, want1 = SG + step_lo * STAGE_GROUPS;
+    const int window0 = want0 <= ngrp - meta_groups ? want0 : ngrp - meta_groups;
+    const int window1 = want1 <= ngrp - meta_groups ? want1 : ngrp - meta_groups;
+    const int shift0 = want0 - window0, shift1 = want1 - window1;  // groups between the window's start and the first step's
 
     uint8_t *const w_lds = lds;                                            // [WAVES][STAGES][STEP_LDS]
     uint8_t *const zero_lds = lds + WAVES * WAVE_LDS;                      // ZERO_BYTES
@@ -161,10 +169,10 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
     float *const xm_lds = (float *)(img_lds + (size_t)T * 2 * SG * GROUP_IMAGE);   // [T][2 * SG] (power of two, sum)
 
     // the wave's block and its stream of steps
-    const int row_base = (((int)blockIdx.x - job.tile0) * WAVES + wave) * BLOCK_ROWS;
-    const bool has_rows = row_base < job.rows;       // a wave without rows still helps with the activations
+    const int row_base = (((int)blockIdx.x - job.tile0) * blocks_per_wg + my_block) * BLOCK_ROWS;
+    const bool has_rows = my_block < blocks_per_wg && row_base < job.rows;   // a wave without rows still helps with the activations
     const int rows_here = !has_rows ? 1 : (job.rows - row_base < BLOCK_ROWS ? job.rows - row_base : BLOCK_ROWS);
-    const int total_steps = has_rows ? nstage : 0;
+    const int total_steps = has_rows ? step_hi - step_lo : 0;
 
     // ---------------------------------------------------------------- per-lane geometry
     // weights: load k of a step covers strip k / 4, rows 8 (k % 4) .. + 7 of the block; lane i lands in slot 64 k + i,
@@ -207,10 +215,10 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
     MetaVec scales_v, biases_v;                      // the same registers as one indexable vector, valid after the wait
     auto issue_meta = [&]() {
         const int row = n < rows_here ? n : rows_here - 1;
-        const size_t at = ((size_t)(row_base + row) * ngrp + (h ? strip1_start : 0)) * 2;
+        const size_t at = ((size_t)(row_base + row) * ngrp + (h ? window1 : window0)) * 2;
 #pragma unroll
         for (int q = 0; q < MD / 4; ++q) {
-            // pieces past the row's groups are not fetched (and never read): the address repeats the last real one
+            // pieces past the window are not fetched (and never read): the address repeats the last real one
             const int piece = 8 * q < meta_groups ? q : (meta_groups - 1) / 8;
             scales_r.q[q] = load_meta16(job.scales + at + 16 * piece);
             biases_r.q[q] = load_meta16(bias_src + at + 16 * piece);
@@ -267,8 +275,9 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
             // register indexing by a wave-uniform index
             auto pick = [&](const MetaVec &m, int dword) -> uint32_t { return m[dword]; };
             const int last = MD - 2;
-            const int i0 = 2 * st < last ? 2 * st : last;
-            const int i1 = 2 * (st + strip1_shift) < last ? 2 * (st + strip1_shift) : last;
+            const int at0 = 2 * (st - step_lo) + (shift0 >> 1), at1 = 2 * (st - step_lo) + (shift1 >> 1);
+            const int i0 = at0 < last ? at0 : last;
+            const int i1 = at1 < last ? at1 : last;
             uint32_t s_lo = pick(scales_v, i0), s_hi = pick(scales_v, i0 + 1);
             uint32_t b_lo = pick(biases_v, i0), b_hi = pick(biases_v, i0 + 1);
             if (i1 != i0) {                        // uniform
@@ -330,12 +339,31 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
         }
     };
 
-    // the two strips of a row meet
+    // The two strips of a row meet; with the row cut into parts, every wave leaves its sums in its own (now idle)
+    // LDS and the first wave of the block adds them in part order.
     auto finish_block = [&]() {
+        float sum[T];
 #pragma unroll
-        for (int t = 0; t < T; ++t) {
-            const float other = __shfl_xor(acc[t], 32, 64);
-            if (lane < rows_here) job.y[(size_t)t * job.y_stride + row_base + lane] = acc[t] + other;
+        for (int t = 0; t < T; ++t) sum[t] = acc[t] + __shfl_xor(acc[t], 32, 64);
+        if (ksplit > 1) {
+            float *mine = (float *)my_lds;
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+                if (lane < 32) mine[t * 32 + lane] = sum[t];
+            __syncthreads();
+            if (my_part != 0) return;
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                float total = 0.0f;
+                for (int p = 0; p < ksplit; ++p)
+                    total = total + ((const float *)(w_lds + (size_t)(my_block * ksplit + p) * WAVE_LDS))[t * 32 + (lane & 31)];
+                sum[t] = total;
+            }
+        }
+        if (has_rows && lane < rows_here) {
+#pragma unroll
+            for (int t = 0; t < T; ++t) job.y[(size_t)t * job.y_stride + row_base + lane] = sum[t];
         }
     };
 
@@ -408,8 +436,8 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
     // only loads that return to registers, are waited for with everything that is in flight at that moment, once.
     // Blocks start their walk over the row at different steps: rows whose length is a power of two put the same
     // step of every row on the same memory channels, and waves that all began at step 0 would queue there.
-    const int first_step = (int)(((unsigned)blockIdx.x * WAVES + wave) % (unsigned)nstage);
-    auto step_of = [&](int g) { const int st = g + first_step; return st < nstage ? st : st - nstage; };
+    const int first_step = total_steps > 0 ? (int)(((unsigned)blockIdx.x * WAVES + wave) % (unsigned)total_steps) : 0;
+    auto step_of = [&](int g) { const int st = g + first_step; return step_lo + (st < total_steps ? st : st - total_steps); };
     if (has_rows) {
         issue_meta();
 #pragma unroll
@@ -418,7 +446,7 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
     }
     if (!(L.debug & 2)) build_image();
     __syncthreads();
-    if (!has_rows) return;                           // no barrier below
+    if (has_rows) {
 #pragma unroll
     for (int q = 0; q < MD / 4; ++q) {
         wait_meta(scales_r.q[q]);
@@ -427,6 +455,19 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
         for (int e = 0; e < 4; ++e) {
             scales_v[4 * q + e] = scales_r.q[q][e];
             biases_v[4 * q + e] = biases_r.q[q][e];
+        }
+    }
+    if ((shift0 | shift1) & 1) {
+        // a window that starts an odd number of groups before the strip's first step: move the lane's values down by
+        // one group (16 bits), so that a step's four again fill two whole registers
+        const bool odd = ((h ? shift1 : shift0) & 1) != 0;
+#pragma unroll
+        for (int i = 0; i < MD; ++i) {
+            const uint32_t s_next = i + 1 < MD ? scales_v[i + 1] : 0u, b_next = i + 1 < MD ? biases_v[i + 1] : 0u;
+            const uint32_t s_moved = __builtin_amdgcn_alignbit(s_next, scales_v[i], 16);
+            const uint32_t b_moved = __builtin_amdgcn_alignbit(b_next, biases_v[i], 16);
+            scales_v[i] = odd ? s_moved : scales_v[i];
+            biases_v[i] = odd ? b_moved : biases_v[i];
         }
     }
 
@@ -453,6 +494,7 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
         });
         if (!more) break;
     }
+    }   // has_rows
     finish_block();
 }
 
@@ -488,7 +530,7 @@ constexpr Candidate CANDIDATES[] = {{4, 2, 2}, {3, 2, 2}, {8, 2, 1}, {7, 2, 1}, 
 
 }  // namespace
 
-bool q4_dot_takes(int cols) { return cols >= DOT_MIN_COLS && cols <= DOT_MAX_COLS && (cols & 255) == 0; }
+bool q4_dot_takes(int cols) { return cols >= DOT_MIN_COLS && cols <= DOT_MAX_COLS && (cols & 63) == 0; }
 
 int q4_dot_tokens_per_pass(int cols) {
     // what fits beside four waves' weight steps in 160 KiB of LDS
@@ -497,23 +539,35 @@ int q4_dot_tokens_per_pass(int cols) {
     return 0;
 }
 
-DotShape q4_dot_shape(int cols, int tokens) {
+DotShape q4_dot_shape(int cols, int tokens, long long total_blocks) {
     static const int want_waves = env_int("SALT_MI355_DOT_WAVES", 0), want_stages = env_int("SALT_MI355_DOT_STAGES", 0);
+    static const int want_ksplit = env_int("SALT_MI355_DOT_KSPLIT", 0);
+    const int nstage = dot_steps(cols >> 6);
+    // Few blocks: cut the rows along their columns until the launch has about a thousand waves
+    int ksplit = 1;
+    while (ksplit < 8 && total_blocks * ksplit < 1024 && nstage >= 2 * ksplit) ksplit *= 2;
+    if (want_ksplit == 1 || want_ksplit == 2 || want_ksplit == 4 || want_ksplit == 8) ksplit = want_ksplit;
+    while (ksplit > 1 && ksplit > nstage) ksplit /= 2;
     // in order of preference; the first that fits the LDS beside the digit planes is taken
     for (const Candidate &c : CANDIDATES)
         if ((want_waves == 0 || want_waves == c.waves) && (want_stages == 0 || want_stages == c.stages) &&
+            c.waves % ksplit == 0 && (ksplit == 1 || c.waves >= 4) &&
             dot_lds_bytes(cols, tokens, c.waves, c.stages) * c.resident <= DOT_LDS_LIMIT)
-            return DotShape{c.waves, c.stages};
-    return DotShape{4, 2};
+            return DotShape{c.waves, c.stages, ksplit};
+    return DotShape{4, 2, ksplit <= 4 ? ksplit : 4};
 }
 
 int q4_dot_launch(const Q4DotLaunch &launch, const DotShape &shape, hipStream_t stream) {
     Q4DotLaunch L = launch;
     if (L.total_wgs < 1 || L.tokens < 1 || L.tokens > 4 || !q4_dot_takes(L.cols)) return -1;
     if (dot_lds_bytes(L.cols, L.tokens, shape.waves, shape.stages) > DOT_LDS_LIMIT) return -1;
+    if (shape.ksplit < 1 || shape.waves % shape.ksplit) return -1;
     static const int debug_env = env_int("SALT_MI355_DOT_DEBUG", 0);
     L.debug = debug_env;
-    const int md = L.cols <= 4096 ? 16 : 32;
+    L.ksplit = shape.ksplit;
+    // groups of a strip that one wave walks: its registers hold 32 (MD = 16) or 64 (MD = 32)
+    const int steps = dot_steps(L.cols >> 6);
+    const int md = ((steps + shape.ksplit - 1) / shape.ksplit) * STAGE_GROUPS <= 32 ? 16 : 32;
 #define DOT_CASE(TT, WW, SS) \
     if (L.tokens == TT && shape.waves == WW && shape.stages == SS) \
         return md == 16 ? launch_shape<TT, WW, SS, 16>(L, stream) : launch_shape<TT, WW, SS, 32>(L, stream)
