@@ -275,6 +275,35 @@ def sweep_record(lib, sweep, ms, steps, warmup):
     }
 
 
+def nvfp4_class_t_leg(gpu, synth, lib, stream, events, w, per, packed_bytes, x, st, R, Cc, G):
+    y = gpu.DeviceBuffer(G * R * 4)
+    turn = [0]
+
+    def single(s):
+        g = turn[0] % G
+        turn[0] += 1
+        if lib.salt_mi355_nvfp4_matvec_t_dev(w.at(g * per), w.at(g * per + packed_bytes), 2688.0, 64.0, R, Cc, 1, x.ptr,
+                                             y.ptr, st.ptr, s) != 0:
+            raise RuntimeError(lib.salt_mi355_last_error().decode())
+
+    ms_1 = timed(lib, stream, events, single, 5, 100)
+    jobs = (gpu.Fp4Job * G)()
+    for g in range(G):
+        jobs[g] = gpu.Fp4Job(w.at(g * per), w.at(g * per + packed_bytes), 2688.0, x.ptr, y.at(g * R * 4), R)
+
+    def multi(s):
+        if lib.salt_mi355_nvfp4_jobs_t_dev(jobs, G, Cc, 1, 64.0, st.ptr, s) != 0:
+            raise RuntimeError(lib.salt_mi355_last_error().decode())
+
+    ms_16 = timed(lib, stream, events, multi, 3, 20)
+    gbps = G * synth.nvfp4_bytes(R, Cc, 1) / (ms_16 * 1e-3) / 1e9
+    return {"nvfp4_8192_class_t_matvec_us": round(ms_1 * 1e3, 2),
+            "nvfp4_8192_class_t_gbps": round(synth.nvfp4_bytes(R, Cc, 1) / (ms_1 * 1e-3) / 1e9, 1),
+            "nvfp4_8192_x16_class_t_one_launch_gbps": round(gbps, 1),
+            "nvfp4_8192_x16_class_t_hbm_frac": round(gbps / HBM_PEAK_GBS, 4),
+            "nvfp4_class_t_kernel": lib.salt_mi355_last_kernel().decode()}
+
+
 def run_only(args, gpu, synth, lib, stream, events):
     """One leg on its own, for profiler runs: the kernels of that leg are the only matvec kernels in the trace."""
     if args.only == "copy":
@@ -283,6 +312,18 @@ def run_only(args, gpu, synth, lib, stream, events):
         sweep = Q4Sweep(gpu, synth, tokens=4 if "b4" in args.only else 1, exact=args.only.endswith("exact"))
         ms = timed(lib, stream, events, sweep.step, args.warmup, args.steps)
         return sweep_record(lib, sweep, ms, args.steps, args.warmup)
+    if args.only == "nvfp4-t":
+        R = Cc = 8192
+        packed, fscales = synth.nvfp4_tensor(R, Cc, 40)
+        G = 16
+        per = packed.nbytes + fscales.nbytes
+        w = gpu.DeviceBuffer(per * G)
+        for g in range(G):
+            w.upload(packed, g * per)
+            w.upload(fscales, g * per + packed.nbytes)
+        x = gpu.DeviceBuffer.from_host(synth.activations(Cc, 1, 41))
+        st = gpu.DeviceBuffer(4, fill=0)
+        return nvfp4_class_t_leg(gpu, synth, lib, stream, events, w, per, packed.nbytes, x, st, R, Cc, G)
     sys.exit("unknown leg: " + args.only)
 
 
@@ -450,6 +491,10 @@ def main():
 
         ms_sw = timed(lib, stream, events, fp4_sweep_step, 2, 10)
         extra["nvfp4_8192_x16_one_launch_gbps"] = round(G * synth.nvfp4_bytes(R, Cc, 1) / (ms_sw * 1e-3) / 1e9, 1)
+        # the tolerance-class kernel (exact code products per block, activation quantised inside the launch):
+        # one matrix per launch, and the sixteen instances as one launch
+        fp4_t = nvfp4_class_t_leg(gpu, synth, lib, stream, events, w, per, packed.nbytes, x, st, R, Cc, G)
+        extra.update(fp4_t)
         del xq, ys16
         # NVFP4 8192 x 8192, batch 256, on the matrix cores (tolerance class); activation pass included
         B = 256

@@ -188,6 +188,25 @@ int salt_mi355_nvfp4_matvec_qdq_dev(const void *packed, const void *scales,
                                     int R, int C, const float *x, float *y,
                                     int *status_dev, int chains, void *stream);
 
+/* Tolerance-class reference matvec: the memory-bound kernel.  Every token is
+ * quantised as salt_nvfp4_quantize_input_reference does (nvfp4.c:82-130, the
+ * same codes and block scales) inside the launch, and ys[token][row]
+ * approximates the reference matvec (nvfp4.c:228-256): per 16-column block the
+ * sum of code products is exact, the block's two factors are applied once and
+ * the blocks are added in fp32 in a different order than the reference's 32
+ * chains.  Bound per output: |y - y_ref| <= 2^-20 * sum_c |w_c x_c|.  xs:
+ * [B][C] raw fp32 activations, 16-byte aligned; ys: [B][R].  *status_dev (device
+ * int, cleared by the caller) becomes -1 when a token of a job holds a
+ * non-finite value; that job then publishes nothing.  C a multiple of 64 from
+ * 512 to 8192 takes the streaming kernel, other multiples of 32 the bit-exact
+ * one-launch kernel.  The reference has no counterpart. */
+int salt_mi355_nvfp4_matvec_t_dev(const void *packed, const void *scales,
+                                  float stored_divisor, float input_global_scale,
+                                  int R, int C, int B, const float *xs, float *ys,
+                                  int *status_dev, void *stream);
+int salt_mi355_nvfp4_jobs_t_dev(const SaltMi355Fp4Job *jobs, int njobs, int C, int tokens,
+                                float input_global_scale, int *status_dev, void *stream);
+
 /* Prefill-sized NVFP4 matmul on the matrix cores (tolerance class): every
  * token is quantised and dequantised as salt_nvfp4_quantize_input_reference
  * does (nvfp4.c:82-130) and ys[token][row] approximates the reference matvec

@@ -229,6 +229,87 @@ int salt_mi355_nvfp4_matvec_qdq_dev(const void *packed, const void *scales, floa
     return 0;
 }
 
+// Tolerance-class reference matvec: jobs of `tokens` raw activation rows each, quantised inside the launch.
+int salt_mi355_nvfp4_jobs_t_dev(const SaltMi355Fp4Job *jobs, int njobs, int C, int tokens, float input_global_scale,
+                                int *status_dev, void *stream_handle) {
+    hipStream_t stream = (hipStream_t)stream_handle;
+    if (!g_state.ready) { set_error("nvfp4 t: library not initialised"); return -1; }
+    if (!g_state.fp8_is_ocp) { set_error("nvfp4: this device's fp8 converter is not OCP E4M3FN"); return -1; }
+    if (!jobs || njobs < 1 || tokens < 1 || !status_dev || !isfinite(input_global_scale) || input_global_scale <= 0.0f ||
+        C < 32 || (C & 31) || C > FP4_FUSED_MAX_COLS) {
+        set_error("nvfp4 t: bad arguments (C a multiple of 32 up to %d, a status word)", FP4_FUSED_MAX_COLS);
+        return -1;
+    }
+    bool streamable = fp4_dot_takes(C);
+    for (int j = 0; j < njobs; ++j) {
+        const SaltMi355Fp4Job &f = jobs[j];
+        if (!f.packed || !f.scales || !f.xs || !f.ys || f.rows < 1 || !isfinite(f.stored_divisor) ||
+            f.stored_divisor == 0.0f || ((uintptr_t)f.packed & 3) || ((uintptr_t)f.scales & 1) || ((uintptr_t)f.xs & 15) ||
+            ((uintptr_t)f.ys & 3)) {
+            set_error("nvfp4 t: job %d is malformed (packed 4-byte, activations 16-byte aligned, non-zero finite divisor)", j);
+            return -1;
+        }
+    }
+    if (!streamable) {
+        // column counts the streaming kernel does not take run on the bit-exact one-launch kernel, token by token
+        for (int j = 0; j < njobs; ++j)
+            for (int t = 0; t < tokens; ++t)
+                if (salt_mi355_nvfp4_matvec_qdq_dev(jobs[j].packed, jobs[j].scales, jobs[j].stored_divisor, input_global_scale,
+                                                    jobs[j].rows, C, jobs[j].xs + (size_t)t * C,
+                                                    jobs[j].ys + (size_t)t * jobs[j].rows, status_dev, 0, stream_handle) != 0)
+                    return -1;
+        return 0;
+    }
+    std::vector<Fp4Job> table((size_t)njobs);
+    for (int first = 0; first < tokens; first += 4) {
+        const int group = tokens - first < 4 ? tokens - first : 4;
+        long long blocks = 0;
+        for (int j = 0; j < njobs; ++j) blocks += (jobs[j].rows + DOT_BLOCK_ROWS - 1) / DOT_BLOCK_ROWS;
+        const DotShape shape = fp4_dot_shape(C, group, blocks);
+        const int rows_per_wg = shape.waves / shape.ksplit * DOT_BLOCK_ROWS;
+        Fp4DotLaunch launch;
+        memset(&launch, 0, sizeof launch);
+        int wgs = 0;
+        bool uniform = true;
+        for (int j = 0; j < njobs; ++j) {
+            Fp4Job &f = table[(size_t)j];
+            f.packed = (const uint8_t *)jobs[j].packed;
+            f.scales = (const uint8_t *)jobs[j].scales;
+            f.x = jobs[j].xs + (size_t)first * C;
+            f.y = jobs[j].ys + (size_t)first * jobs[j].rows;
+            f.weight_global_scale = 1.0f / jobs[j].stored_divisor;
+            f.rows = jobs[j].rows;
+            f.tile0 = wgs;
+            f.x_stride = C;
+            wgs += (jobs[j].rows + rows_per_wg - 1) / rows_per_wg;
+            uniform = uniform && jobs[j].rows == jobs[0].rows;
+        }
+        launch.njobs = njobs; launch.cols = C; launch.tokens = group; launch.total_wgs = wgs;
+        launch.wgs_per_job = uniform ? wgs / njobs : 0;
+        launch.input_global_scale = input_global_scale;
+        launch.status = status_dev;
+        State::TableSlot *slot = nullptr;
+        if (njobs == 1) {
+            launch.one = table[0];
+        } else {
+            slot = table_acquire(table.data(), table.size() * sizeof(Fp4Job), stream);
+            if (!slot) return -1;
+            launch.table = (const Fp4Job *)slot->device;
+        }
+        const int rc = fp4_dot_launch(launch, shape, stream);
+        table_release(slot, stream);
+        if (rc != 0) { set_error("nvfp4 t: kernel launch failed: %s", hipGetErrorString(hipGetLastError())); return -1; }
+    }
+    return 0;
+}
+
+int salt_mi355_nvfp4_matvec_t_dev(const void *packed, const void *scales, float stored_divisor, float input_global_scale,
+                                  int R, int C, int B, const float *xs, float *ys, int *status_dev, void *stream) {
+    SaltMi355Fp4Job job;
+    job.packed = packed; job.scales = scales; job.stored_divisor = stored_divisor; job.xs = xs; job.ys = ys; job.rows = R;
+    return salt_mi355_nvfp4_jobs_t_dev(&job, 1, C, B, input_global_scale, status_dev, stream);
+}
+
 int salt_mi355_bf16_matvec_dev(const void *weights, int R, int C, int B, const float *xs, const float *bias, float *ys,
                                 void *stream) {
     if (!g_state.ready) { set_error("bf16 matvec: library not initialised"); return -1; }

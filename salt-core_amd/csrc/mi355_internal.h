@@ -178,6 +178,24 @@ struct Fp4Launch {
 constexpr int FP4_FUSED_MAX_COLS = 8192;
 
 int fp4_launch(const Fp4Launch &launch, int chains_per_lane, hipStream_t stream);
+
+// The reference matvec (activation quantised inside the launch) on the tolerance-class streaming kernel
+// (nvfp4_dot.hip).  tile0 of a job = index of its first workgroup; job.x is the raw activation.
+struct Fp4DotLaunch {
+    Fp4Job one;
+    const Fp4Job *table;
+    int njobs;
+    int cols;
+    int tokens;               // 1..4
+    int total_wgs;
+    int ksplit;               // filled by fp4_dot_launch from the shape
+    int wgs_per_job;          // > 0 when every job of the table has this many workgroups
+    float input_global_scale;
+    int *status;              // cleared by the caller; becomes -1 when an activation is not finite
+};
+bool fp4_dot_takes(int cols);
+DotShape fp4_dot_shape(int cols, int tokens, long long total_blocks);
+int fp4_dot_launch(const Fp4DotLaunch &launch, const DotShape &shape, hipStream_t stream);
 // activation quantise/dequantise per 16-block; any of packed/scales/dequant/plane may be null.  plane receives
 // code value * block scale as bf16 (exact), the activation operand of the matrix-core matmul.
 int fp4_qdq_launch(const float *input, int cols, int tokens, float input_global_scale,

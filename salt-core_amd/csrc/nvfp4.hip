@@ -19,6 +19,7 @@
 // 16-element block with closed-form round-to-nearest-even encoders in place of
 // the reference's argmin scans (equality is proven on the host by the tests).
 #include "mi355_internal.h"
+#include "nvfp4_device.h"
 
 #include <stddef.h>
 
@@ -66,30 +67,6 @@ __device__ __forceinline__ Fp4Job find_job(const Fp4Launch &L, int tile) {
     job.tile0 = (int)(uint32_t)rec[5];
     job.x_stride = (int)(rec[5] >> 32);
     return job;
-}
-
-// Closed-form round-to-nearest-even E4M3FN encode of a finite, non-negative
-// value already clamped to 448.
-__device__ __forceinline__ uint32_t e4m3_encode_positive(float m) {
-    if (m < 0.015625f) return (uint32_t)__builtin_rintf(m * 512.0f);
-    uint32_t bits = __float_as_uint(m);
-    bits += 0x7FFFFu + ((bits >> 20) & 1u);
-    return (bits >> 20) - ((127u - 7u) << 3);
-}
-
-__device__ __forceinline__ uint32_t e2m1_encode(float v) {
-    const float m = __builtin_fabsf(v);
-    const uint32_t code = (uint32_t)(m > 0.25f) + (uint32_t)(m >= 0.75f) + (uint32_t)(m > 1.25f) +
-                          (uint32_t)(m >= 1.75f) + (uint32_t)(m > 2.5f) + (uint32_t)(m >= 3.5f) +
-                          (uint32_t)(m > 5.0f);
-    return code | ((__float_as_uint(v) >> 28) & 8u);
-}
-
-__device__ __forceinline__ float e2m1_decode(uint32_t code) {
-    const uint32_t m = code & 7u;
-    // 0, .5, 1, 1.5, 2, 3, 4, 6; magnitude zero is +0 whatever the sign bit
-    const float mag = m == 0 ? 0.0f : m == 1 ? 0.5f : (1.0f + 0.5f * (float)(m & 1u)) * (float)(1u << ((m >> 1) - 1u));
-    return (code & 8u) && m != 0 ? -mag : mag;
 }
 
 // Quantise and dequantise one 16-element block (reference nvfp4.c:82-130).

@@ -32,71 +32,15 @@
 // costs a quarter of the stream's rate: 64 scattered pieces per load.  Loads that return to registers are kept out
 // of the loop on purpose: on this device they do not complete in issue order with direct-to-LDS loads, so a partial
 // s_waitcnt vmcnt(n) cannot tell which of the two kinds has landed.)
-#include "mi355_internal.h"
+#include "dot_common.h"
 
-#ifndef DOT_SWIZZLE_LOW
-#define DOT_SWIZZLE_LOW 0
-#endif
-
-#include <stddef.h>
 #include <stdio.h>
-#include <stdlib.h>
-
-#include <type_traits>
-#include <utility>
 
 namespace mi355 {
 namespace {
 
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef const u32x4 __attribute__((address_space(1))) *global_u128_ptr;
-typedef __attribute__((address_space(3))) void *lds_void_ptr;
-typedef const uint64_t __attribute__((address_space(4))) *uniform_u64_ptr;
-
-constexpr int BLOCK_ROWS = DOT_BLOCK_ROWS;   // rows per block = N of the matrix instruction
-constexpr int STAGE_BYTES = 8192;            // 2 strips x 32 rows x 128 bytes
-constexpr int STAGE_GROUPS = 4;              // scale groups per strip and step
-constexpr int STEP_LDS = STAGE_BYTES;
-constexpr int LOADS_PER_STEP = 8;            // weight pieces
 constexpr int ZERO_BYTES = 1024 + 256;       // what lanes without a digit plane read instead
 constexpr int GROUP_IMAGE = 256;             // bytes of digits per group: 4 quarters x 4 planes x 16
-#ifndef DOT_STREAMING
-#define DOT_STREAMING 2
-#endif
-constexpr int STREAMING = DOT_STREAMING;     // 2 = non-temporal: every weight byte is read once
-
-__device__ __forceinline__ int swizzle(int piece) { return DOT_SWIZZLE_LOW ? (piece & 7) : ((piece >> 1) & 7); }
-
-// steps per strip: half of the row's groups, in whole steps
-__host__ __device__ __forceinline__ int dot_steps(int ngrp) { return ((ngrp + 1) / 2 + STAGE_GROUPS - 1) / STAGE_GROUPS; }
-
-// f(integral_constant<int, 0>), f(<1>), ... until one returns false; true when all ran
-template <int... I, class F>
-__device__ __forceinline__ bool static_steps(std::integer_sequence<int, I...>, F &&f) {
-    return (f(std::integral_constant<int, I>{}) && ...);
-}
-
-// A lane's scales (or biases) of one block: MD dwords = 2 * MD groups of its strip, in registers.
-template <int MD> struct MetaRegs { u32x4 q[MD / 4]; };
-
-// Written in assembly so that the compiler neither moves the load nor waits for it on its own: the one wait that
-// covers it names the registers (wait_meta).
-__device__ __forceinline__ u32x4 load_meta16(const uint8_t *address) {
-    u32x4 value;
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(value) : "v"(address) : "memory");
-    return value;
-}
-__device__ __forceinline__ void wait_meta(u32x4 &value) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(value) : : "memory"); }
-
-template <int N>
-__device__ __forceinline__ void wait_vm() {
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
 
 __device__ __forceinline__ Q4Job dot_find_job(const Q4DotLaunch &L, int wg) {
     if (L.table == nullptr) return L.one;
@@ -516,11 +460,6 @@ int launch_shape(const Q4DotLaunch &L, hipStream_t stream) {
     note_kernel("q4_dot_kernel<%d,%d,%d,%d>", T, WAVES, STAGES, MD);
     hipLaunchKernelGGL((q4_dot_kernel<T, WAVES, STAGES, MD>), dim3(L.total_wgs), dim3(WAVES * 64), lds, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
-}
-
-int env_int(const char *name, int fallback) {
-    const char *e = getenv(name);
-    return e ? atoi(e) : fallback;
 }
 
 // (waves per workgroup, steps of LDS per wave); `resident` workgroups share a compute unit's LDS

@@ -99,6 +99,8 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_nvfp4_matvec_dev, i, vp, vp, f, i, i, i, vp, vp, i, vp)
     _sig(lib.salt_mi355_nvfp4_jobs_dev, i, C.POINTER(Fp4Job), i, i, i, i, vp)
     _sig(lib.salt_mi355_nvfp4_matvec_qdq_dev, i, vp, vp, f, f, i, i, vp, vp, vp, i, vp)
+    _sig(lib.salt_mi355_nvfp4_matvec_t_dev, i, vp, vp, f, f, i, i, i, vp, vp, vp, vp)
+    _sig(lib.salt_mi355_nvfp4_jobs_t_dev, i, C.POINTER(Fp4Job), i, i, i, f, vp, vp)
     _sig(lib.salt_mi355_nvfp4_matmul_workspace_bytes, sz, i, i, i)
     _sig(lib.salt_mi355_nvfp4_matmul_dev, i, vp, vp, f, f, i, i, i, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_bf16_matvec_dev, i, vp, i, i, i, vp, vp, vp, vp)
@@ -237,6 +239,22 @@ def nvfp4_matvec(packed: np.ndarray, scales: np.ndarray, divisor: float, R: int,
         src = dq
     check(lib.salt_mi355_nvfp4_matvec_dev(dw.ptr, ds.ptr, divisor, R, C_, B, src.ptr, dy.ptr, chains, stream),
           "nvfp4_matvec_dev")
+    check(lib.salt_mi355_stream_sync(stream), "sync")
+    return int(st.to_host(np.int32)[0]), dy.to_host(np.float32).reshape(B, R)
+
+
+def nvfp4_matvec_t(packed: np.ndarray, scales: np.ndarray, divisor: float, R: int, C_: int, xs: np.ndarray,
+                   input_global_scale: float = 64.0):
+    """The reference matvec on the tolerance-class kernel (salt_mi355_nvfp4_matvec_t_dev).  Returns (status, ys[B, R]);
+    ys stays 0xFF-filled for a rejected job."""
+    lib = init()
+    xs = np.ascontiguousarray(xs, np.float32).reshape(-1, C_)
+    B = xs.shape[0]
+    dw, ds, dx = DeviceBuffer.from_host(packed), DeviceBuffer.from_host(scales), DeviceBuffer.from_host(xs)
+    dy, st = DeviceBuffer(B * R * 4, fill=0xFF), DeviceBuffer(4, fill=0)
+    stream = lib.salt_mi355_stream()
+    check(lib.salt_mi355_nvfp4_matvec_t_dev(dw.ptr, ds.ptr, divisor, input_global_scale, R, C_, B, dx.ptr, dy.ptr, st.ptr,
+                                            stream), "nvfp4_matvec_t_dev")
     check(lib.salt_mi355_stream_sync(stream), "sync")
     return int(st.to_host(np.int32)[0]), dy.to_host(np.float32).reshape(B, R)
 

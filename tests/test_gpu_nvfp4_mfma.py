@@ -53,6 +53,27 @@ def test_matmul_within_stated_tolerance(pkg, oracle, R, Cc, B, g):
     assert np.isfinite(got).all() and ratio <= 1.0, ratio
 
 
+def test_cfg4_8192x8192_batch256_sampled_rows(pkg, oracle):
+    """BASELINE configs[4] at batch 256 and full size (128 tiles x 4 K-splits plus the split sum): 32 rows x 256
+    tokens against the checker."""
+    R = Cc = 8192
+    B = 256
+    print("nvfp4 mfma 8192 x 8192 x 256", flush=True)
+    packed, scales = synth.nvfp4_tensor(R, Cc, 40)
+    xs = synth.activations(Cc, B, 42)
+    status, got = pkg.lib.nvfp4_matmul(packed, scales, 2688.0, 64.0, R, Cc, xs)
+    assert status == 0 and np.isfinite(got).all()
+    rows = np.arange(5, R, 256)
+    sub_packed = np.ascontiguousarray(packed.reshape(R, Cc // 2)[rows]).reshape(-1)
+    sub_scales = np.ascontiguousarray(scales.reshape(R, Cc // 16)[rows]).reshape(-1)
+    want, mags = reference(oracle, sub_packed, sub_scales, 2688.0, 64.0, len(rows), Cc, xs)
+    bound = 2.0 ** -20 * mags + 1e-30
+    err = np.abs(got[:, rows].astype(np.float64) - want)
+    ratio = float((err / bound).max())
+    print("max err / bound", ratio, flush=True)
+    assert ratio <= 1.0, ratio
+
+
 def test_non_finite_activation_publishes_nothing(pkg):
     R, Cc, B = 128, 128, 9
     packed, scales = synth.nvfp4_tensor(R, Cc, 3)
