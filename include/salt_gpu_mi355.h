@@ -321,6 +321,20 @@ int salt_mi355_moe_decode_step_dev(const void *pool, size_t expert_stride,
                                    const float *x, int *selected, float *weights,
                                    float *expert_out, float *out,
                                    void *workspace, void *stream);
+/* Tolerance-class form of the layer-step: router top-k, selection and weights
+ * are bit-identical to the reference; the three projections of every selected
+ * expert run on the kernel of salt_mi355_q4_matvec_t_dev (its bound applies to
+ * each projection against its own input), gelu_tanh and the ordered weighted
+ * sum are the reference's.  Stated tolerance of the composition (tests):
+ * |expert_out - ref| <= 2^-15 * max_d |ref[expert]| + 1e-6, the same for out.
+ * Same arguments and workspace as salt_mi355_moe_decode_step_dev; more than
+ * 256 experts or widths outside 512..4096 take the bit-exact plan. */
+int salt_mi355_moe_decode_step_t_dev(const void *pool, size_t expert_stride,
+                                     int hidden, int routed, int n_experts, int topk,
+                                     const float *logits, const float *per_expert_scale,
+                                     const float *x, int *selected, float *weights,
+                                     float *expert_out, float *out,
+                                     void *workspace, void *stream);
 /* The same layer-step for callers that cannot allocate device memory or pass a
  * workspace (code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc): the workspace is a static array inside the library, one

@@ -387,6 +387,8 @@ int salt_mi355_q4_jobs_t_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int t
         State::TableSlot *slot = nullptr;
         if (njobs == 1) {
             launch.one = table[0];
+        } else if (njobs <= Q4_INLINE_JOBS) {
+            memcpy(launch.inline_jobs, table.data(), (size_t)njobs * sizeof(Q4Job));
         } else {
             slot = table_acquire(table.data(), table.size() * sizeof(Q4Job), stream);
             if (!slot) return -1;

@@ -603,6 +603,35 @@ int salt_mi355_moe_decode_step_dev(const void *pool, size_t expert_stride, int h
     return 0;
 }
 
+// Tolerance-class form of the step: the projections run on the streaming kernel; geometries it does not serve take
+// the bit-exact plan (whose result is inside any tolerance).
+int salt_mi355_moe_decode_step_t_dev(const void *pool, size_t expert_stride, int hidden, int routed, int n_experts,
+                                     int topk, const float *logits, const float *per_expert_scale, const float *x,
+                                     int *selected, float *weights, float *expert_out, float *out, void *workspace,
+                                     void *stream) {
+    if (!g_state.ready) { set_error("moe step t: library not initialised"); return -1; }
+    if (!pool || !logits || !per_expert_scale || !x || !selected || !weights || !out || !workspace ||
+        ((uintptr_t)pool & 3) || (expert_stride & 15) || ((uintptr_t)workspace & 255)) {
+        set_error("moe step t: bad arguments (pool 4-byte aligned, expert stride a multiple of 16, workspace 256-byte aligned)");
+        return -1;
+    }
+    const MoeGeometry g = {hidden, routed, n_experts, topk};
+    const size_t n = (size_t)hidden * (size_t)routed;
+    if (hidden < 64 || (hidden & 63) || routed < 64 || (routed & 63) || n_experts < 1 || topk < 1 || topk > n_experts ||
+        expert_stride < 3 * (n / 2 + 4 * (n / 64))) {
+        set_error("moe step t: hidden and routed must be multiples of 64 and the stride must cover a slot");
+        return -1;
+    }
+    MoeWorkspace ws;
+    moe_workspace_carve(g, workspace, &ws);
+    if (moe_decode_step_t_launch(g, (const uint8_t *)pool, expert_stride, logits, per_expert_scale, x, selected, weights,
+                                 expert_out, out, ws, (hipStream_t)stream) == 0)
+        return 0;
+    (void)hipGetLastError();
+    return salt_mi355_moe_decode_step_dev(pool, expert_stride, hidden, routed, n_experts, topk, logits, per_expert_scale,
+                                          x, selected, weights, expert_out, out, workspace, stream);
+}
+
 // ---------------------------------------------------------------- the same step without a workspace argument
 
 }  // extern "C"

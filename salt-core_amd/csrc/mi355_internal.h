@@ -102,11 +102,19 @@ struct Q4DotLaunch {
     int ksplit;               // filled by q4_dot_launch from the shape
     int wgs_per_job;          // > 0 when every job of the table has this many workgroups (workgroup -> job by division)
     int debug;
+    MoeFuse moe;              // only read by q4_dot_moe_gate_up_launch / q4_dot_moe_down_launch
+    // Up to Q4_INLINE_JOBS job records inside the kernel arguments (table == nullptr, njobs > 1): a decode-sized
+    // batch then needs no table upload.  Must stay the last member.
+    Q4Job inline_jobs[Q4_INLINE_JOBS];
 };
 bool q4_dot_takes(int cols);
 int q4_dot_tokens_per_pass(int cols);      // 0: the column count does not fit at all
 DotShape q4_dot_shape(int cols, int tokens, long long total_blocks);
 int q4_dot_launch(const Q4DotLaunch &launch, const DotShape &shape, hipStream_t stream);
+// The MoE decode step's two matvec launches on the streaming kernel (router top-k in the prologue of the first,
+// gelu_tanh(gate) * up in the prologue of the second); -1: the geometry is not served.
+int q4_dot_moe_gate_up_launch(const MoeFuse &moe, hipStream_t stream);
+int q4_dot_moe_down_launch(const MoeFuse &moe, hipStream_t stream);
 
 // ---------------------------------------------------------------- affine Q4 on MFMA (tolerance class)
 
@@ -293,6 +301,13 @@ int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t exp
                            const float *logits, const float *per_expert_scale, const float *x,
                            int *selected, float *weights, float *expert_out, float *out,
                            const MoeWorkspace &ws, float code_scale, hipStream_t stream);
+
+// tolerance class (q4_dot.hip); -1 when the geometry is not served (more than 256 experts, widths the streaming
+// kernel does not take)
+int moe_decode_step_t_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_stride,
+                             const float *logits, const float *per_expert_scale, const float *x,
+                             int *selected, float *weights, float *expert_out, float *out,
+                             const MoeWorkspace &ws, hipStream_t stream);
 
 int moe_activate_launch(const float *gate, const float *up, float *act, size_t n, hipStream_t stream);
 int moe_reduce_launch(const float *expert_out, const float *weights, int topk, int hidden, float *out,

@@ -207,4 +207,20 @@ int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t exp
     return out ? moe_reduce_launch(eo, weights, g.topk, g.hidden, out, nullptr, stream) : 0;
 }
 
+// The same step on the tolerance-class matvec kernel: router top-k (bit-exact, in the prologue of the gate/up
+// launch), gate and up, gelu_tanh(gate) * up (in the prologue of the down launch), down, ordered weighted sum.
+int moe_decode_step_t_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_stride, const float *logits,
+                             const float *per_expert_scale, const float *x, int *selected, float *weights,
+                             float *expert_out, float *out, const MoeWorkspace &ws, hipStream_t stream) {
+    MoeFuse m;
+    memset(&m, 0, sizeof m);
+    m.logits = logits; m.per_expert_scale = per_expert_scale; m.pool = pool; m.expert_stride = expert_stride;
+    m.x = x; m.gate = ws.gate; m.up = ws.up; m.expert_out = expert_out ? expert_out : ws.expert_out;
+    m.selected = selected; m.weights = weights; m.status = ws.status;
+    m.n_experts = g.n_experts; m.topk = g.topk; m.hidden = g.hidden; m.routed = g.routed;
+    if (q4_dot_moe_gate_up_launch(m, stream) != 0) return -1;
+    if (q4_dot_moe_down_launch(m, stream) != 0) return -1;
+    return out ? moe_reduce_launch(m.expert_out, weights, g.topk, g.hidden, out, ws.status, stream) : 0;
+}
+
 }  // namespace mi355

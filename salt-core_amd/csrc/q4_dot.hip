@@ -33,8 +33,11 @@
 // of the loop on purpose: on this device they do not complete in issue order with direct-to-LDS loads, so a partial
 // s_waitcnt vmcnt(n) cannot tell which of the two kinds has landed.)
 #include "dot_common.h"
+#include "device_math.h"
+#include "router_device.h"
 
 #include <stdio.h>
+#include <string.h>
 
 namespace mi355 {
 namespace {
@@ -43,8 +46,13 @@ constexpr int ZERO_BYTES = 1024 + 256;       // what lanes without a digit plane
 constexpr int GROUP_IMAGE = 256;             // bytes of digits per group: 4 quarters x 4 planes x 16
 
 __device__ __forceinline__ Q4Job dot_find_job(const Q4DotLaunch &L, int wg) {
-    if (L.table == nullptr) return L.one;
-    const uniform_u64_ptr words = (uniform_u64_ptr)(uintptr_t)L.table;
+    if (L.table == nullptr && L.njobs <= 1) return L.one;
+    // 7 words per record, in a device table or inside the kernel arguments (the launch record is the kernel's only
+    // argument, so the inline records sit at their offset in the kernarg segment)
+    const uniform_u64_ptr words =
+        L.table ? (uniform_u64_ptr)(uintptr_t)L.table
+                : (uniform_u64_ptr)((const char __attribute__((address_space(4))) *)__builtin_amdgcn_kernarg_segment_ptr() +
+                                    offsetof(Q4DotLaunch, inline_jobs));
     int lo = 0, hi = L.njobs - 1;
     if (L.wgs_per_job > 0) {               // every job has the same number of workgroups: no search
         lo = wg / L.wgs_per_job;
@@ -71,9 +79,16 @@ __device__ __forceinline__ Q4Job dot_find_job(const Q4DotLaunch &L, int wg) {
 // T tokens per pass (1..4), WAVES waves per workgroup, STAGES steps of LDS per wave (one being consumed, the others
 // in flight), MD dwords of scales per lane (two groups each: 16 serves rows of up to 4096 columns, 32 up to 8192).
 // A workgroup owns WAVES consecutive blocks of 32 rows of one job, one per wave.
-template <int T, int WAVES, int STAGES, int MD>
+//
+// PRO selects a prologue of the MoE decode step (0: none, the jobs come from the launch): 1 = router top-k, the
+// workgroup derives its gate or up job from the selection (one workgroup past the jobs publishes selection, weights
+// and status); 2 = the down projection of one selected expert, whose activation gelu_tanh(gate) * up is computed
+// while the digit planes are built.
+template <int T, int WAVES, int STAGES, int MD, int PRO = 0>
 __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L) {
     static_assert(T >= 1 && T <= 4 && STAGES >= 2 && STAGES <= 4 && (MD == 16 || MD == 32), "tokens per pass, steps per wave");
+    static_assert(PRO == 0 || (T == 1 && sizeof(RouterShared) <= (size_t)WAVES * STAGES * STEP_LDS),
+                  "the MoE prologues serve one token; the router borrows the weight staging memory");
     constexpr int WAVE_LDS = STAGES * STEP_LDS;
     constexpr int AHEAD = STAGES - 1;                // steps in flight behind the one being consumed
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -82,7 +97,44 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const Q4Job job = dot_find_job(L, blockIdx.x);
+    Q4Job job;
+    const float *act_gate = nullptr, *act_up = nullptr;       // PRO == 2: the activation is gelu_tanh(gate) * up
+    if (PRO == 0) {
+        job = dot_find_job(L, blockIdx.x);
+    } else {
+        const MoeFuse &m = L.moe;
+        const size_t n = (size_t)m.hidden * (size_t)m.routed;
+        const size_t vals_bytes = n / 2, meta_bytes = (n / 64) * 2, proj_bytes = vals_bytes + 2 * meta_bytes;
+        const int wgs_per_job = L.wgs_per_job;
+        const int slot = (int)blockIdx.x / wgs_per_job;
+        if (PRO == 1) {
+            // The expert, and with it the weight pointers, is known only after the router has run; everything else
+            // is known now, so that the activation's digit planes can be built while the logits are on their way.
+            const int place = slot >> 1, proj = slot & 1;                  // slot = 2 * place + (0 gate | 1 up)
+            job.vals = nullptr;
+            job.x = m.x;
+            job.y = (proj ? m.up : m.gate) + (size_t)place * m.routed;
+            job.rows = m.routed;
+            job.x_stride = m.hidden;
+            job.y_stride = m.routed;
+        } else {
+            if (*(const int __attribute__((address_space(4))) *)(uintptr_t)m.status != 0) return;
+            const int place = slot;
+            const int expert = ((const int __attribute__((address_space(4))) *)(uintptr_t)m.selected)[place];
+            act_gate = m.gate + (size_t)place * m.routed;
+            act_up = m.up + (size_t)place * m.routed;
+            job.vals = m.pool + (size_t)expert * m.expert_stride + 2 * proj_bytes;
+            job.x = nullptr;
+            job.y = m.expert_out + (size_t)place * m.hidden;
+            job.rows = m.hidden;
+            job.x_stride = m.routed;
+            job.y_stride = m.hidden;
+        }
+        job.tile0 = slot * wgs_per_job;
+        job.scales = job.vals + vals_bytes;
+        job.biases = job.scales + meta_bytes;
+    }
+    const bool publisher = PRO == 1 && (int)blockIdx.x == L.total_wgs;     // one workgroup past the jobs
 
     const int C = L.cols;
     const int ngrp = C >> 6;
@@ -140,8 +192,8 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
     uint32_t rd_off[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s) rd_off[s] = (uint32_t)my_piece * 128u + (uint32_t)(s ^ swizzle(my_piece)) * 16u;
-    const bool no_bias = job.biases == nullptr;      // the load still happens (the waits count it); its result is dropped
-    const uint8_t *const bias_src = no_bias ? job.scales : job.biases;
+    // a job without biases: the load still happens (the waits count it, it reads the scales); its result is dropped
+    const bool no_bias = PRO == 0 && job.biases == nullptr;
     // digit planes: row m = l % 32 of the M side is (token m / 8, strip (m / 4) % 2, plane m % 4); it carries digits
     // only in the lanes of its own strip (l / 32)
     const int m_tok = n >> 3, m_strip = (n >> 2) & 1, m_plane = n & 3;
@@ -165,12 +217,12 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
             // pieces past the window are not fetched (and never read): the address repeats the last real one
             const int piece = 8 * q < meta_groups ? q : (meta_groups - 1) / 8;
             scales_r.q[q] = load_meta16(job.scales + at + 16 * piece);
-            biases_r.q[q] = load_meta16(bias_src + at + 16 * piece);
+            biases_r.q[q] = load_meta16((no_bias ? job.scales : job.biases) + at + 16 * piece);
         }
     };
     // Step st into ring slot `slot`: eight weight pieces.
-    const uint8_t *const block_vals = job.vals + (size_t)row_base * row_bytes;
     auto issue_step = [&](int st, int slot) {
+        const uint8_t *const block_vals = job.vals + (size_t)row_base * row_bytes;
         uint8_t *const stage = my_lds + slot * STEP_LDS;
         const uint32_t advance = (uint32_t)st * (STAGE_GROUPS * 32);
         if (rows_here == BLOCK_ROWS && st < whole_steps) {
@@ -323,7 +375,11 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
             const int t = (item >> 4) / (2 * SG);
             const bool valid = g < ngrp;               // slots past the row's end hold zero digits
             float xv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (valid) {
+            if (valid && PRO == 2) {
+                const size_t at = (size_t)g * 64 + 4 * q16;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) xv[k] = det_gelu_tanh(act_gate[at + k]) * act_up[at + k];
+            } else if (valid) {
                 const float *src = job.x + (size_t)t * job.x_stride + (size_t)g * 64 + 4 * q16;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) xv[k] = src[k];
@@ -382,13 +438,40 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
     // step of every row on the same memory channels, and waves that all began at step 0 would queue there.
     const int first_step = total_steps > 0 ? (int)(((unsigned)blockIdx.x * WAVES + wave) % (unsigned)total_steps) : 0;
     auto step_of = [&](int g) { const int st = g + first_step; return step_lo + (st < total_steps ? st : st - total_steps); };
+    if (PRO == 1) {
+        const MoeFuse &m = L.moe;
+        // first touch of the router's inputs now: they arrive while the digit planes are built
+        float warm = 0.0f;
+        if (tid < m.n_experts) warm = m.logits[tid] + m.per_expert_scale[tid];
+        if (!publisher) build_image();
+        asm volatile("" ::"v"(warm));
+        const int slot = (int)blockIdx.x / L.wgs_per_job;
+        int expert;
+        if (publisher) {
+            // the workgroup that publishes selection, weights and status runs the whole router (ordered sums and all)
+            RouterShared &sh = *reinterpret_cast<RouterShared *>(lds);     // the weight staging memory, idle here
+            router_topk_block(m.logits, m.per_expert_scale, m.n_experts, m.topk, true, true, sh);
+            const int bad = sh.bad;
+            if (tid == 0) *m.status = bad ? -1 : 0;
+            if (tid < m.topk && !bad) { m.selected[tid] = sh.out_sel[tid]; m.weights[tid] = sh.out_w[tid]; }
+            return;
+        }
+        // every other wave finds its expert on its own: with finite inputs the router cannot fail later
+        expert = router_select_wave(m.logits, m.per_expert_scale, m.n_experts, m.topk, slot >> 1);
+        if (expert < 0) return;                                            // uniform: every wave sees the same inputs
+        const size_t n_weights = (size_t)m.hidden * (size_t)m.routed;
+        const size_t vals_bytes = n_weights / 2, meta_bytes = (n_weights / 64) * 2;
+        job.vals = m.pool + (size_t)expert * m.expert_stride + (size_t)(slot & 1) * (vals_bytes + 2 * meta_bytes);
+        job.scales = job.vals + vals_bytes;
+        job.biases = job.scales + meta_bytes;
+    }
     if (has_rows) {
         issue_meta();
 #pragma unroll
         for (int g = 0; g < STAGES; ++g)
             if (g < total_steps) issue_step(step_of(g), g);
     }
-    if (!(L.debug & 2)) build_image();
+    if (PRO != 1 && !(L.debug & 2)) build_image();
     __syncthreads();
     if (has_rows) {
 #pragma unroll
@@ -447,18 +530,20 @@ size_t dot_lds_bytes(int cols, int tokens, int waves, int stages) {
     return (size_t)waves * stages * STEP_LDS + ZERO_BYTES + (size_t)tokens * 2 * sg * (GROUP_IMAGE + 8);
 }
 
-template <int T, int WAVES, int STAGES, int MD>
+template <int T, int WAVES, int STAGES, int MD, int PRO = 0>
 int launch_shape(const Q4DotLaunch &L, hipStream_t stream) {
     const size_t lds = dot_lds_bytes(L.cols, T, WAVES, STAGES);
     static size_t raised = 0;                 // per instantiation: the largest dynamic LDS size asked for so far
     if (lds > raised) {
-        if (hipFuncSetAttribute((const void *)q4_dot_kernel<T, WAVES, STAGES, MD>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess)
+        if (hipFuncSetAttribute((const void *)q4_dot_kernel<T, WAVES, STAGES, MD, PRO>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
             return -1;
         raised = lds;
     }
-    note_kernel("q4_dot_kernel<%d,%d,%d,%d>", T, WAVES, STAGES, MD);
-    hipLaunchKernelGGL((q4_dot_kernel<T, WAVES, STAGES, MD>), dim3(L.total_wgs), dim3(WAVES * 64), lds, stream, L);
+    note_kernel("q4_dot_kernel<%d,%d,%d,%d,%d>", T, WAVES, STAGES, MD, PRO);
+    // the router prologue has one more workgroup: the one that publishes its outputs
+    hipLaunchKernelGGL((q4_dot_kernel<T, WAVES, STAGES, MD, PRO>), dim3(L.total_wgs + (PRO == 1 ? 1 : 0)), dim3(WAVES * 64),
+                       lds, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -516,6 +601,49 @@ int q4_dot_launch(const Q4DotLaunch &launch, const DotShape &shape, hipStream_t 
 #undef DOT_CASES
 #undef DOT_CASE
     return -1;
+}
+
+// The two matvec launches of the MoE decode step on the streaming kernel: four waves per workgroup, the rows cut
+// along their columns so that every compute unit gets work.  Geometries the prologues do not serve return -1 (the
+// caller then takes the bit-exact plan).
+static bool moe_dot_geometry_ok(const MoeFuse &m) {
+    return m.n_experts >= 1 && m.n_experts <= 256 && m.topk >= 1 && m.topk <= m.n_experts && m.topk <= ROUTER_MAX_TOPK &&
+           q4_dot_takes(m.hidden) && q4_dot_takes(m.routed) && m.hidden <= 4096 && m.routed <= 4096;
+}
+
+static int moe_dot_ksplit(long long blocks, int cols) {
+    const int nstage = dot_steps(cols >> 6);
+    int ksplit = 1;
+    while (ksplit < 4 && blocks * ksplit < 1024 && nstage >= 2 * ksplit) ksplit *= 2;
+    return ksplit;
+}
+
+int q4_dot_moe_gate_up_launch(const MoeFuse &m, hipStream_t stream) {
+    if (!moe_dot_geometry_ok(m) || dot_lds_bytes(m.hidden, 1, 4, 2) > DOT_LDS_LIMIT) return -1;
+    Q4DotLaunch L;
+    memset(&L, 0, sizeof L);
+    L.moe = m;
+    L.cols = m.hidden; L.tokens = 1; L.njobs = 2 * m.topk;
+    const int blocks = (m.routed + DOT_BLOCK_ROWS - 1) / DOT_BLOCK_ROWS;
+    L.ksplit = moe_dot_ksplit((long long)blocks * 2 * m.topk, m.hidden);
+    L.wgs_per_job = (blocks + 4 / L.ksplit - 1) / (4 / L.ksplit);
+    L.total_wgs = 2 * m.topk * L.wgs_per_job;
+    static const int debug_env = env_int("SALT_MI355_DOT_DEBUG", 0);
+    L.debug = debug_env;
+    return launch_shape<1, 4, 2, 16, 1>(L, stream);
+}
+
+int q4_dot_moe_down_launch(const MoeFuse &m, hipStream_t stream) {
+    if (!moe_dot_geometry_ok(m) || dot_lds_bytes(m.routed, 1, 4, 2) > DOT_LDS_LIMIT) return -1;
+    Q4DotLaunch L;
+    memset(&L, 0, sizeof L);
+    L.moe = m;
+    L.cols = m.routed; L.tokens = 1; L.njobs = m.topk;
+    const int blocks = (m.hidden + DOT_BLOCK_ROWS - 1) / DOT_BLOCK_ROWS;
+    L.ksplit = moe_dot_ksplit((long long)blocks * m.topk, m.routed);
+    L.wgs_per_job = (blocks + 4 / L.ksplit - 1) / (4 / L.ksplit);
+    L.total_wgs = m.topk * L.wgs_per_job;
+    return launch_shape<1, 4, 2, 16, 2>(L, stream);
 }
 
 }  // namespace mi355

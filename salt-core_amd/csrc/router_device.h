@@ -141,4 +141,68 @@ __device__ __forceinline__ void router_topk_block(const float *__restrict__ logi
     __syncthreads();
 }
 
+// The same selection for one wave on its own, without LDS or barriers: which expert stands at position `place` of
+// the chosen experts in ascending-id order (the order in which the reference's callers run them,
+// gemma4_text.c:7923-7930).  Returns -1 when a logit or a per-expert scale is not finite (the reference rejects the
+// call).  n_experts <= 256, every lane of the wave active.
+//
+// "Rank below topk" is a selection of the topk largest logits with ties going to the smaller index.  The wave finds
+// the topk-th largest value by a radix search over order-preserving integer keys (32 steps of compare + popcount),
+// takes everything above it and the lowest-indexed of the values equal to it.
+constexpr int ROUTER_WAVE_MAX_EXPERTS = 256;
+
+__device__ __forceinline__ int router_select_wave(const float *__restrict__ logits,
+                                                  const float *__restrict__ per_expert_scale, int n_experts, int topk,
+                                                  int place) {
+    const int lane = threadIdx.x & 63;
+    uint32_t key[4];
+    bool finite = true;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int e = q * 64 + lane;
+        key[q] = 0u;                                                     // below every real key
+        if (e < n_experts) {
+            const float v = logits[e] + 0.0f;                            // -0 becomes +0: they compare equal
+            const float sc = per_expert_scale[e];
+            finite = finite && (__builtin_fabsf(v) < __builtin_inff()) && (__builtin_fabsf(sc) < __builtin_inff());
+            const uint32_t bits = __float_as_uint(v);
+            key[q] = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+        }
+    }
+    if (__ballot(!finite) != 0ull) return -1;
+    // the largest threshold that at least topk keys reach
+    uint32_t threshold = 0u;
+    for (int bit = 31; bit >= 0; --bit) {
+        const uint32_t candidate = threshold | (1u << bit);
+        int reach = 0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) reach += __popcll(__ballot(key[q] >= candidate));
+        if (reach >= topk) threshold = candidate;
+    }
+    int above = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) above += __popcll(__ballot(key[q] > threshold));
+    const int ties_wanted = topk - above;                                // of the keys equal to the threshold
+    const uint64_t below_me = (1ull << lane) - 1ull;
+    bool chosen[4];
+    int ties_before = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint64_t equal = __ballot(key[q] == threshold);
+        const int my_tie = ties_before + __popcll(equal & below_me);
+        chosen[q] = key[q] > threshold || (key[q] == threshold && my_tie < ties_wanted);
+        ties_before += __popcll(equal);
+    }
+    // position of every chosen expert in ascending-id order; the one at `place` answers
+    int expert = -1, before = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint64_t mask = __ballot(chosen[q]);
+        const uint64_t hit = __ballot(chosen[q] && before + __popcll(mask & below_me) == place);
+        if (hit != 0ull) expert = q * 64 + (int)__builtin_ctzll(hit);
+        before += __popcll(mask);
+    }
+    return expert;
+}
+
 }  // namespace mi355

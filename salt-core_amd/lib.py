@@ -111,6 +111,7 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_router_topk_dev, i, vp, vp, i, i, i, vp, vp, vp, vp)
     _sig(lib.salt_mi355_moe_workspace_bytes, sz, i, i, i, i)
     _sig(lib.salt_mi355_moe_decode_step_dev, i, vp, sz, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, vp, vp)
+    _sig(lib.salt_mi355_moe_decode_step_t_dev, i, vp, sz, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_moe_decode_step_static_dev, i, vp, sz, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, vp, vp)
     _sig(lib.salt_mi355_moe_prefill_workspace_bytes, sz, i, i, i, i, i)
     _sig(lib.salt_mi355_moe_prefill_dev, i, vp, sz, i, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, vp, vp)
@@ -389,9 +390,11 @@ class MoeLayer:
         self.x, self.out = DeviceBuffer(hidden * 4), DeviceBuffer(hidden * 4)
         self.sel, self.w = DeviceBuffer(topk * 4), DeviceBuffer(topk * 4)
         self.eo = DeviceBuffer(topk * hidden * 4)
+        self.tolerance_class = False    # True: salt_mi355_moe_decode_step_t_dev
 
     def enqueue(self, stream):
-        return self.lib.salt_mi355_moe_decode_step_dev(
+        fn = self.lib.salt_mi355_moe_decode_step_t_dev if self.tolerance_class else self.lib.salt_mi355_moe_decode_step_dev
+        return fn(
             self.pool.at(self.header), self.stride, self.H, self.F, self.E, self.K, self.logits.ptr, self.scale.ptr, self.x.ptr,
             self.sel.ptr, self.w.ptr, self.eo.ptr, self.out.ptr, self.ws.ptr, stream)
 
