@@ -222,6 +222,24 @@ int salt_mi355_nvfp4_matmul_dev(const void *packed, const void *scales,
                                 int R, int C, int B, const float *xs, float *ys,
                                 int *status_dev, void *workspace, void *stream);
 
+/* ---- the formats themselves, device-resident ----------------------------- */
+
+/* reference salt_q4_decode (src/kernels.c:188-208): out[k] for n flat elements,
+ * the scale and bias of group k / 64, two roundings per element; any byte
+ * alignment of vals / scales / biases, biases may be NULL.  Bit-exact. */
+int salt_mi355_q4_decode_dev(const void *vals, const void *scales, const void *biases,
+                             size_t n, float *out, void *stream);
+/* reference salt_nvfp4_dequantize_weights_reference (src/nvfp4.c:132-155):
+ * out[R*C] = e2m1(code) * (e4m3(scale) * (1 / stored_divisor)).  Bit-exact. */
+int salt_mi355_nvfp4_dequant_weights_dev(const void *packed, const void *scales,
+                                         float stored_divisor, int R, int C,
+                                         float *out, void *stream);
+/* reference salt_router (src/router.c:22-57), the fixture router: scores are
+ * hashes of (state, layer, expert); idx[topk] in selection order, w[topk] the
+ * unbiased scores.  n_experts <= 1024.  Bit-exact (indices and weight bits). */
+int salt_mi355_router_fixture_dev(int n_experts, int topk, uint64_t state, int layer,
+                                  double locality, int *idx, float *w, void *stream);
+
 /* ---- bf16 and 8-bit affine matvecs, device-resident --------------------- */
 
 /* reference salt_bf16_matvec (src/kernels.c:139-174), the arithmetic behind

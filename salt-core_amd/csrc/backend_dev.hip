@@ -695,6 +695,43 @@ int salt_mi355_moe_decode_step_static_dev(const void *pool, size_t expert_stride
     return 0;
 }
 
+int salt_mi355_q4_decode_dev(const void *vals, const void *scales, const void *biases, size_t n, float *out, void *stream) {
+    if (!g_state.ready) { set_error("q4 decode: library not initialised"); return -1; }
+    if (!vals || !scales || !out || ((uintptr_t)out & 3)) { set_error("q4 decode: bad arguments"); return -1; }
+    if (q4_decode_launch((const uint8_t *)vals, (const uint8_t *)scales, (const uint8_t *)biases, n, out, (hipStream_t)stream) != 0) {
+        set_error("q4 decode: launch failed");
+        return -1;
+    }
+    return 0;
+}
+
+int salt_mi355_nvfp4_dequant_weights_dev(const void *packed, const void *scales, float stored_divisor, int R, int C,
+                                         float *out, void *stream) {
+    if (!g_state.ready) { set_error("nvfp4 dequant: library not initialised"); return -1; }
+    if (!g_state.fp8_is_ocp) { set_error("nvfp4: this device's fp8 converter is not OCP E4M3FN"); return -1; }
+    if (!packed || !scales || !out || R < 1 || C < 16 || (C & 15) || !isfinite(stored_divisor) || stored_divisor == 0.0f ||
+        ((uintptr_t)out & 3)) {
+        set_error("nvfp4 dequant: bad arguments (C a multiple of 16, non-zero finite divisor)");
+        return -1;
+    }
+    if (nvfp4_dequant_launch((const uint8_t *)packed, (const uint8_t *)scales, 1.0f / stored_divisor, R, C, out,
+                             (hipStream_t)stream) != 0) {
+        set_error("nvfp4 dequant: launch failed");
+        return -1;
+    }
+    return 0;
+}
+
+int salt_mi355_router_fixture_dev(int n_experts, int topk, uint64_t state, int layer, double locality, int *idx, float *w,
+                                  void *stream) {
+    if (!g_state.ready) { set_error("fixture router: library not initialised"); return -1; }
+    if (!idx || !w || router_fixture_launch(n_experts, topk, state, layer, locality, idx, w, (hipStream_t)stream) != 0) {
+        set_error("fixture router: bad arguments (1 <= topk <= n_experts <= 1024)");
+        return -1;
+    }
+    return 0;
+}
+
 int salt_mi355_moe_activate_dev(const float *gate, const float *up, float *act, size_t n, void *stream) {
     if (!g_state.ready || !gate || !up || !act || n < 1) { set_error("moe activate: bad arguments"); return -1; }
     return moe_activate_launch(gate, up, act, n, (hipStream_t)stream);

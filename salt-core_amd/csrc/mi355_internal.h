@@ -325,6 +325,15 @@ int moe_prefill_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_
 // Zero `words` 32-bit words at dst with a kernel on `stream` (safe under graph capture, unlike a memset node).
 int clear_words_launch(void *dst, size_t words, hipStream_t stream);
 
+// ---------------------------------------------------------------- formats (formats.hip)
+
+int q4_decode_launch(const uint8_t *vals, const uint8_t *scales, const uint8_t *biases, size_t n, float *out,
+                     hipStream_t stream);
+int nvfp4_dequant_launch(const uint8_t *packed, const uint8_t *scales, float weight_global_scale, int R, int C, float *out,
+                         hipStream_t stream);
+int router_fixture_launch(int n_experts, int topk, uint64_t state, int layer, double locality, int *idx, float *w,
+                          hipStream_t stream);
+
 // ---------------------------------------------------------------- probes
 
 // Decodes all 256 byte values through the fp8 and fp4 converters (device

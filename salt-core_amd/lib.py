@@ -103,6 +103,9 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_nvfp4_jobs_t_dev, i, C.POINTER(Fp4Job), i, i, i, f, vp, vp)
     _sig(lib.salt_mi355_nvfp4_matmul_workspace_bytes, sz, i, i, i)
     _sig(lib.salt_mi355_nvfp4_matmul_dev, i, vp, vp, f, f, i, i, i, vp, vp, vp, vp, vp)
+    _sig(lib.salt_mi355_q4_decode_dev, i, vp, vp, vp, sz, vp, vp)
+    _sig(lib.salt_mi355_nvfp4_dequant_weights_dev, i, vp, vp, f, i, i, vp, vp)
+    _sig(lib.salt_mi355_router_fixture_dev, i, i, i, C.c_uint64, i, C.c_double, vp, vp, vp)
     _sig(lib.salt_mi355_bf16_matvec_dev, i, vp, i, i, i, vp, vp, vp, vp)
     _sig(lib.salt_mi355_q8_matvec_dev, i, vp, vp, vp, i, i, i, vp, vp, vp)
     _sig(lib.salt_mi355_cells_dev, i, C.POINTER(Cell), i, vp, vp)
