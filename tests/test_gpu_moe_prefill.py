@@ -5,11 +5,13 @@ against the reference's grouping (src/moe_group.c:138-184) as recorded in the
 golden fixtures and as recomputed here.  Values run on the matrix-core matmul
 and carry a stated tolerance against the bit-exact CPU checker:
 
-    |error[token][d]| <= 2^-16 * max_d |y[token][d]| + 1e-6
+    |error[token][d]| <= 2^-18 * M[token][d] + 1e-6,
+    M[token][d] = sum over the token's experts k of |w_k| * sum_f |Wd_k[d][f] * h_k[f]|
 
-(the gate/up projections are accurate to a few 2^-20 of their term magnitudes;
-gelu and the down projection propagate that, and cancellation inside one
-output is covered by comparing with the token's largest component)."""
+per output, where h_k = gelu_tanh(gate_k) * up_k is the expert's activation and Wd_k its dequantised down projection
+(the sum of the magnitudes of the terms that make up the output; test_against_cpu_checker computes it in float64).
+At the full BASELINE geometry the fixtures hold outputs only; there the bound is per token,
+2^-18 * max_d |y[token][d]| + 1e-6."""
 import ctypes as C
 
 import numpy as np
@@ -29,9 +31,35 @@ def expected_grouping(sel, E):
     return np.bincount(flat, minlength=E).astype(np.int32), order
 
 
-def check_values(got, want):
-    scale = np.abs(want).max(axis=1, keepdims=True).astype(np.float64)
-    bound = 2.0 ** -16 * scale + 1e-6
+def dequantised(pool, e, p, H, F):
+    """Expert e's projection p (0 gate, 1 up, 2 down) as float64 [rows][cols]."""
+    proj, n = synth.expert_proj_bytes(H, F), H * F
+    at = (e * 3 + p) * proj
+    vals = pool[at:at + n // 2].view(np.uint32)
+    sc = synth.bf16_bits_to_f32(pool[at + n // 2:at + n // 2 + n // 32].view(np.uint16)).astype(np.float64)
+    bi = synth.bf16_bits_to_f32(pool[at + n // 2 + n // 32:at + proj].view(np.uint16)).astype(np.float64)
+    q = ((vals[:, None] >> (4 * np.arange(8, dtype=np.uint32))) & 15).reshape(-1).astype(np.float64)
+    w = q * np.repeat(sc, 64) + np.repeat(bi, 64)
+    return w.reshape((F, H) if p < 2 else (H, F))
+
+
+def term_magnitudes(pool, sel, w, xs, H, F):
+    """M[token][d] of the module docstring, in float64."""
+    T, K = sel.shape
+    M = np.zeros((T, H))
+    x64 = xs.astype(np.float64)
+    for e in np.unique(sel):
+        tok, rank = np.nonzero(sel == e)
+        gate, up, down = (dequantised(pool, int(e), p, H, F) for p in range(3))
+        g = x64[tok] @ gate.T
+        h = 0.5 * g * (1.0 + np.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3))) * (x64[tok] @ up.T)
+        M[tok] += np.abs(w[tok, rank].astype(np.float64))[:, None] * (np.abs(h) @ np.abs(down).T)
+    return M
+
+
+def check_values(got, want, magnitudes=None):
+    scale = np.abs(want).max(axis=1, keepdims=True).astype(np.float64) if magnitudes is None else magnitudes
+    bound = 2.0 ** -18 * scale + 1e-6
     err = np.abs(got.astype(np.float64) - want.astype(np.float64))
     ratio = float((err / bound).max())
     print("max err / bound", ratio, flush=True)
@@ -71,7 +99,7 @@ def test_against_cpu_checker(pkg, oracle, T, E, K, H, F):
     assert status == 0
     want_rows, want_pairs = expected_grouping(sel, E)
     assert np.array_equal(rows, want_rows) and np.array_equal(pairs, want_pairs)
-    check_values(ys, want)
+    check_values(ys, want, term_magnitudes(pool, sel, w, xs, H, F))
     # a second call with fewer tokens on the same workspace
     status, ys2, rows2, _ = layer.run(sel[: T // 2 + 1], w[: T // 2 + 1], xs[: T // 2 + 1])
     assert status == 0 and rows2.sum() == (T // 2 + 1) * K
