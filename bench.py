@@ -191,6 +191,29 @@ def cpu_other_configs(synth, pool, cores: int, budget_s: float = 3.0):
             fn()
         return unit_count * reps / (time.perf_counter() - t0), reps
 
+    # BASELINE configs[0] (one 4096 x 4096 matvec) and the batch-4 sweep with the reference's own salt_q4_matvec (its
+    # x86 batch path decodes the weights once per token, so four tokens are four calls)
+    if ref is not None:
+        v0, s0, b0 = synth.q4_tensor(4096, 4096, 60)
+        x0, y0 = synth.activations(4096, 1, 61)[0], np.zeros(4096, np.float32)
+        calls_per_s, reps = rate(lambda: ref.salt_q4_matvec(ptr(v0), ptr(s0), ptr(b0), 4096, 4096, ptr(x0), ptr(y0)), 1,
+                                 budget_s)
+        out["q4_4096_matvec_us"] = {"value": round(1e6 / calls_per_s, 1), "kind": "reference", "cores": cores,
+                                    "sample": f"{reps} calls"}
+        sweep_cases = []
+        for seed, (R, Cc) in enumerate(SWEEP):
+            vals, scales, biases = synth.q4_tensor(R, Cc, 100 + seed)
+            sweep_cases.append((R, Cc, vals, scales, biases, synth.activations(Cc, 4, 200 + seed), np.zeros((4, R), np.float32)))
+
+        def batch4_pass():
+            for R, Cc, vals, scales, biases, xs4, ys4 in sweep_cases:
+                for t in range(4):
+                    ref.salt_q4_matvec(ptr(vals), ptr(scales), ptr(biases), R, Cc, ptr(xs4[t]), ptr(ys4[t]))
+
+        nbytes4 = sum(synth.q4_bytes(R, Cc, 4) for R, Cc in SWEEP)
+        bytes_per_s, reps = rate(batch4_pass, nbytes4, budget_s)
+        out["q4_sweep_batch4_gbps"] = {"value": round(bytes_per_s / 1e9, 3), "kind": "reference", "cores": cores,
+                                       "sample": f"{reps} passes of the 3-shape sweep at batch 4 (one call per token)"}
     # MoE decode layer-step (port of the reference's step, experts run on `cores` threads)
     E, K, H, F = 128, 8, 2816, 704
     g = ExpertGeometry(H, F)
@@ -275,6 +298,37 @@ def sweep_record(lib, sweep, ms, steps, warmup):
     }
 
 
+def moe_leg(gpu, synth, lib, stream, events, pool, tolerance_class):
+    """MoE decode layer-step, E = 128 top-8, d_model 2816, d_ff 704.  Two layer instances (857 MB of experts) and 32
+    logit vectors per layer taken in turn, so that the selection changes from step to step and the 256 MB last-level
+    cache cannot hold the experts a step reads."""
+    E, K, H, F = 128, 8, 2816, 704
+    layers = [gpu.MoeLayer(pool, E, H, F, K) for _ in range(2)]
+    logit_sets = []
+    for i, layer in enumerate(layers):
+        layer.tolerance_class = tolerance_class
+        logit_sets.append([gpu.DeviceBuffer.from_host(synth.router_logits(E, 900 + 100 * i + k)) for k in range(32)])
+        layer.scale.upload(np.ones(E, np.float32))
+        layer.x.upload(synth.activations(H, 1, 950 + i)[0])
+    turn = [0]
+
+    def moe_step(st):
+        for layer, sets in zip(layers, logit_sets):
+            layer.logits = sets[turn[0] % len(sets)]
+            if layer.enqueue(st) != 0:
+                raise RuntimeError(lib.salt_mi355_last_error().decode())
+        turn[0] += 1
+
+    ms_moe = timed(lib, stream, events, moe_step, 5, 100) / len(layers)
+    step_bytes = synth.moe_step_bytes(H, F, E, K)
+    tag = "moe_decode_step_class_t" if tolerance_class else "moe_decode_step"
+    out = {tag + "_us": round(ms_moe * 1e3, 2),
+           tag + "_gbps": round(step_bytes / (ms_moe * 1e-3) / 1e9, 1),
+           tag + "_hbm_frac": round(step_bytes / (ms_moe * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    out["moe_layer_tokens_per_s_class_t" if tolerance_class else "moe_layer_tokens_per_s"] = round(1e3 / ms_moe, 1)
+    return out
+
+
 def nvfp4_class_t_leg(gpu, synth, lib, stream, events, w, per, packed_bytes, x, st, R, Cc, G):
     y = gpu.DeviceBuffer(G * R * 4)
     turn = [0]
@@ -312,6 +366,9 @@ def run_only(args, gpu, synth, lib, stream, events):
         sweep = Q4Sweep(gpu, synth, tokens=4 if "b4" in args.only else 1, exact=args.only.endswith("exact"))
         ms = timed(lib, stream, events, sweep.step, args.warmup, args.steps)
         return sweep_record(lib, sweep, ms, args.steps, args.warmup)
+    if args.only in ("moe", "moe-t"):
+        pool = synth.expert_pool(128, 2816, 704, 7)
+        return moe_leg(gpu, synth, lib, stream, events, pool, args.only == "moe-t")
     if args.only == "nvfp4-t":
         R = Cc = 8192
         packed, fscales = synth.nvfp4_tensor(R, Cc, 40)
@@ -377,33 +434,11 @@ def main():
             ms_w = timed(lib, stream, events, warm.step, 5, max(20, args.steps))
             extra[name] = round(warm.bytes_per_step / (ms_w * 1e-3) / 1e9, 1)
             del warm
-        # MoE decode layer-step, E = 128 top-8, d_model 2816, d_ff 704.  Two layer instances (857 MB of experts) and 32
-        # logit vectors per layer taken in turn, so that the selection changes from step to step and the 256 MB
-        # last-level cache cannot hold the experts a step reads.
+        # MoE decode layer-step, E = 128 top-8, d_model 2816, d_ff 704: bit-exact plan and tolerance-class plan
         E, K, H, F = 128, 8, 2816, 704
         pool = synth.expert_pool(E, H, F, 7)
-        layers = [gpu.MoeLayer(pool, E, H, F, K) for _ in range(2)]
-        logit_sets = []
-        for i, layer in enumerate(layers):
-            logit_sets.append([gpu.DeviceBuffer.from_host(synth.router_logits(E, 900 + 100 * i + k)) for k in range(32)])
-            layer.scale.upload(np.ones(E, np.float32))
-            layer.x.upload(synth.activations(H, 1, 950 + i)[0])
-        turn = [0]
-
-        def moe_step(st):
-            for layer, sets in zip(layers, logit_sets):
-                layer.logits = sets[turn[0] % len(sets)]
-                if layer.enqueue(st) != 0:
-                    raise RuntimeError(lib.salt_mi355_last_error().decode())
-            turn[0] += 1
-
-        ms_moe = timed(lib, stream, events, moe_step, 5, 100) / len(layers)
-        step_bytes = synth.moe_step_bytes(H, F, E, K)
-        extra["moe_decode_step_us"] = round(ms_moe * 1e3, 2)
-        extra["moe_layer_tokens_per_s"] = round(1e3 / ms_moe, 1)
-        extra["moe_decode_step_gbps"] = round(step_bytes / (ms_moe * 1e-3) / 1e9, 1)
-        extra["moe_decode_step_hbm_frac"] = round(step_bytes / (ms_moe * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
-        del layers, logit_sets
+        extra.update(moe_leg(gpu, synth, lib, stream, events, pool, False))
+        extra.update(moe_leg(gpu, synth, lib, stream, events, pool, True))
         # the whole feed-forward block of a decoder layer for one token: pre-norms, dense FFN (2112 wide), router input,
         # 8-bit gate, top-8 of 128, routed experts, parallel combine -- bit-exact, device-resident.  32 residuals taken
         # in turn: the routing, hence the experts read, changes from block to block.
@@ -455,6 +490,17 @@ def main():
         ms_q0 = timed(lib, stream, events, q4_single_step, 2, 10) / G
         extra["q4_4096_matvec_us"] = round(ms_q0 * 1e3, 2)
         extra["q4_4096_matvec_gbps"] = round(synth.q4_bytes(R, Cc, 1) / (ms_q0 * 1e-3) / 1e9, 1)
+
+        def q4_single_step_t(s):
+            for g in range(G):
+                at = g * per
+                if lib.salt_mi355_q4_matvec_t_dev(w0.at(at), w0.at(at + vals.nbytes), w0.at(at + vals.nbytes + scales.nbytes),
+                                                  R, Cc, 1, x0.ptr, y0.ptr, s) != 0:
+                    raise RuntimeError(lib.salt_mi355_last_error().decode())
+
+        ms_q0t = timed(lib, stream, events, q4_single_step_t, 2, 10) / G
+        extra["q4_4096_class_t_matvec_us"] = round(ms_q0t * 1e3, 2)
+        extra["q4_4096_class_t_matvec_gbps"] = round(synth.q4_bytes(R, Cc, 1) / (ms_q0t * 1e-3) / 1e9, 1)
         del w0, x0, y0
         # NVFP4 8192 x 8192, batch 1, reference semantics (activation Q/DQ inside the rows' launch), 16 instances
         R = Cc = 8192
