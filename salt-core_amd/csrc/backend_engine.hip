@@ -81,15 +81,32 @@ struct Seat {                         // one expert-cache seat
 
 struct Pending { const void *staged; void *host; size_t nbytes; };
 
+// Expert residency (include/salt/gpu_residency.h:63-89).  The ledger on the engine's side owns the protocol (which
+// seat, which staging buffer, which ticket); what the backend keeps is what it needs to answer it:
+//  * a staging buffer is "in flight" from populate until the copy out of it is known to be complete; it remembers the
+//    ticket and the seat it feeds, and carries the one event that marks the end of its copy;
+//  * a seat remembers the staging buffer that is filling it (or none);
+//  * copies are spread over several streams ("lanes", staging buffer b uses lane b % lanes), so that independent fills
+//    overlap on the copy engines instead of queueing behind each other.
 struct Residency {
-    int ready = 0, poisoned = 0;
+    static constexpr uint32_t kNone = 0xffffffffu;
+    static constexpr int kLanes = 4;
+    struct StagingBuffer {
+        hipEvent_t copied = nullptr;  // recorded behind the copy out of this buffer
+        uint64_t ticket = 0;          // 0: idle
+        uint32_t seat = kNone;
+    };
+    int live = 0;                     // create succeeded and destroy has not run
+    int broken = 0;                   // a copy stream failed: every later call is refused until destroy
     SaltGpuResidencyPlan plan = {};
-    uint8_t *arena = nullptr, *staging = nullptr;
-    hipStream_t stream = nullptr;
-    std::vector<hipEvent_t> events;
-    std::vector<uint64_t> slot_ticket, staging_ticket;
-    std::vector<uint32_t> slot_staging;
+    uint8_t *arena = nullptr, *pinned = nullptr;
+    hipStream_t lanes[kLanes] = {};
+    std::vector<StagingBuffer> buffers;
+    std::vector<uint32_t> seat_buffer; // per seat: the staging buffer that is filling it, or kNone
     int published = 0;                // the permanent spans are populated and resolvable
+
+    uint8_t *staging_at(uint32_t b) const { return pinned + (size_t)b * plan.staging_bytes; }
+    hipStream_t lane_of(uint32_t b) const { return lanes[b % kLanes]; }
 };
 
 struct Engine {
@@ -589,7 +606,7 @@ int salt_gpu_init(void) {
 
 int salt_gpu_free(void) {
     Engine &e = g_engine;
-    if (e.residency.ready) { set_error("salt_gpu_free: the residency arena is still live"); return -1; }
+    if (e.residency.live || e.residency.broken) { set_error("salt_gpu_free: the residency arena is still live"); return -1; }
     int failed = 0;
     if (g_state.ready) {
         failed |= salt_gpu_sync();
@@ -1253,7 +1270,7 @@ int salt_gpu_selected_resource_bind_resident(int slot, uint64_t logical_id, cons
     if (ready_or_fail("selected_resource_bind_resident") != 0 || seat_checks(slot, logical_id) != 0) return -1;
     Engine &e = g_engine;
     const Residency &res = e.residency;
-    if (!payload || nbytes < 1 || !device_address || !res.ready ||
+    if (!payload || nbytes < 1 || !device_address || !res.live || res.broken ||
         device_address < (uintptr_t)res.arena || nbytes > res.plan.device_budget_bytes ||
         device_address - (uintptr_t)res.arena > res.plan.device_budget_bytes - nbytes) {
         set_error("bind_resident: the device address is not inside the residency arena");
@@ -1671,112 +1688,128 @@ int salt_gpu_exact_cells(const SaltGpuExactCell *cells, int count) {
 
 // ================================================================ residency operations
 
+// Gives back everything create took.  Used by destroy and by every failure inside create, so that a half-built
+// arena never lingers.
+static int residency_release(Residency &r) {
+    int failed = 0;
+    for (Residency::StagingBuffer &b : r.buffers)
+        if (b.copied) failed |= hip_ok(hipEventDestroy(b.copied), "residency: destroy event");
+    for (hipStream_t &lane : r.lanes)
+        if (lane) failed |= hip_ok(hipStreamDestroy(lane), "residency: destroy copy stream");
+    if (r.pinned) failed |= hip_ok(hipHostFree(r.pinned), "residency: free staging");
+    if (r.arena) failed |= hip_ok(hipFree(r.arena), "residency: free arena");
+    r = Residency();
+    return failed;
+}
+
 static int res_create(void *, const SaltGpuResidencyPlan *plan) {
     Residency &r = g_engine.residency;
-    if (!g_state.ready || r.ready || !plan || plan->slot_count < 1 || plan->staging_count < 1 || plan->slot_bytes < 1 ||
-        plan->staging_bytes < plan->slot_bytes || plan->device_budget_bytes < 1 ||
-        plan->slot_base_offset > plan->device_budget_bytes ||
-        (uint64_t)plan->slot_count * plan->slot_bytes > plan->device_budget_bytes - plan->slot_base_offset) {
-        set_error("residency create: invalid plan or arena already live");
-        return -1;
-    }
+    if (!g_state.ready) { set_error("residency: the backend is not initialised"); return -1; }
+    if (r.live || r.broken) { set_error("residency: an arena exists already (destroy it first)"); return -1; }
+    if (!plan) { set_error("residency: no plan"); return -1; }
+    const uint64_t seats_bytes = (uint64_t)plan->slot_count * plan->slot_bytes;
+    const bool shaped = plan->slot_count >= 1 && plan->staging_count >= 1 && plan->slot_bytes >= 1 &&
+                        plan->staging_bytes >= plan->slot_bytes && plan->device_budget_bytes >= 1;
+    const bool fits = shaped && plan->slot_base_offset <= plan->device_budget_bytes &&
+                      seats_bytes <= plan->device_budget_bytes - plan->slot_base_offset;
+    if (!fits) { set_error("residency: the plan's seats do not fit its device budget"); return -1; }
     r = Residency();
     r.plan = *plan;
-    if (hip_ok(hipMalloc((void **)&r.arena, plan->device_budget_bytes), "hipMalloc residency arena") != 0 ||
-        hip_ok(hipHostMalloc((void **)&r.staging, plan->staging_bytes * plan->staging_count, hipHostMallocDefault),
-               "hipHostMalloc residency staging") != 0 ||
-        hip_ok(hipStreamCreateWithFlags(&r.stream, hipStreamNonBlocking), "hipStreamCreate residency") != 0) {
-        if (r.arena) (void)hipFree(r.arena);
-        if (r.staging) (void)hipHostFree(r.staging);
-        r = Residency();
+    int ok = hip_ok(hipMalloc((void **)&r.arena, plan->device_budget_bytes), "residency: arena in HBM") == 0 &&
+             hip_ok(hipHostMalloc((void **)&r.pinned, (size_t)plan->staging_bytes * plan->staging_count, hipHostMallocDefault),
+                    "residency: pinned staging") == 0;
+    for (int l = 0; ok && l < Residency::kLanes; ++l)
+        ok = hip_ok(hipStreamCreateWithFlags(&r.lanes[l], hipStreamNonBlocking), "residency: copy stream") == 0;
+    if (ok) r.buffers.assign(plan->staging_count, Residency::StagingBuffer());
+    for (size_t b = 0; ok && b < r.buffers.size(); ++b)
+        ok = hip_ok(hipEventCreateWithFlags(&r.buffers[b].copied, hipEventDisableTiming), "residency: copy event") == 0;
+    if (!ok) {
+        char keep[sizeof g_state.last_error];
+        memcpy(keep, g_state.last_error, sizeof keep);
+        (void)residency_release(r);
+        memcpy(g_state.last_error, keep, sizeof keep);
         return -1;
     }
-    r.events.assign(plan->slot_count, nullptr);
-    for (hipEvent_t &ev : r.events)
-        if (hip_ok(hipEventCreateWithFlags(&ev, hipEventDisableTiming), "hipEventCreate residency") != 0) {
-            r.poisoned = 1;
-            return -1;
-        }
-    r.slot_ticket.assign(plan->slot_count, 0);
-    r.staging_ticket.assign(plan->staging_count, 0);
-    r.slot_staging.assign(plan->slot_count, UINT32_MAX);
-    r.ready = 1;
+    r.seat_buffer.assign(plan->slot_count, Residency::kNone);
+    r.live = 1;
     return 0;
 }
 
 static int res_staging(void *, uint32_t staging_slot, void **address, size_t *capacity) {
     Residency &r = g_engine.residency;
-    if (!r.ready || r.poisoned || !address || !capacity || staging_slot >= r.plan.staging_count) return -1;
-    *address = r.staging + (size_t)staging_slot * r.plan.staging_bytes;
+    if (!r.live || r.broken || !address || !capacity || staging_slot >= r.buffers.size()) return -1;
+    *address = r.staging_at(staging_slot);
     *capacity = (size_t)r.plan.staging_bytes;
     return 0;
 }
 
+// The staging buffer holds the seat's bytes (the engine's read callback filled it): start the copy into the seat.
 static int res_populate(void *, uint32_t slot, uint64_t device_offset, uint32_t staging_slot, size_t nbytes,
                         uint64_t ticket) {
     Residency &r = g_engine.residency;
-    if (!r.ready || r.poisoned || ticket == 0 || nbytes == 0 || slot >= r.plan.slot_count ||
-        staging_slot >= r.plan.staging_count || nbytes > r.plan.slot_bytes || r.slot_ticket[slot] != 0 ||
-        r.staging_ticket[staging_slot] != 0 ||
-        device_offset != r.plan.slot_base_offset + (uint64_t)slot * r.plan.slot_bytes)
+    if (!r.live || r.broken || ticket == 0 || nbytes == 0 || nbytes > r.plan.slot_bytes) return -1;
+    if (slot >= r.seat_buffer.size() || staging_slot >= r.buffers.size()) return -1;
+    if (device_offset != r.plan.slot_base_offset + (uint64_t)slot * r.plan.slot_bytes) return -1;   // a seat's own place
+    Residency::StagingBuffer &buffer = r.buffers[staging_slot];
+    if (buffer.ticket != 0 || r.seat_buffer[slot] != Residency::kNone) return -1;    // either side is still busy
+    const hipStream_t lane = r.lane_of(staging_slot);
+    if (hip_ok(hipMemcpyAsync(r.arena + device_offset, r.staging_at(staging_slot), nbytes, hipMemcpyHostToDevice, lane),
+               "residency: seat copy") != 0)
         return -1;
-    if (hip_ok(hipMemcpyAsync(r.arena + device_offset, r.staging + (size_t)staging_slot * r.plan.staging_bytes, nbytes,
-                              hipMemcpyHostToDevice, r.stream), "residency populate") != 0)
-        return -1;
-    if (hip_ok(hipEventRecord(r.events[slot], r.stream), "residency event") != 0) {
-        if (hipStreamSynchronize(r.stream) != hipSuccess) r.poisoned = 1;
+    if (hip_ok(hipEventRecord(buffer.copied, lane), "residency: seat copy event") != 0) {
+        // the copy is queued but cannot be observed: wait it out so that the buffer may be reused, or give up
+        if (hipStreamSynchronize(lane) != hipSuccess) r.broken = 1;
         return -1;
     }
-    r.slot_ticket[slot] = ticket;
-    r.staging_ticket[staging_slot] = ticket;
-    r.slot_staging[slot] = staging_slot;
+    buffer.ticket = ticket;
+    buffer.seat = slot;
+    r.seat_buffer[slot] = staging_slot;
     return 0;
 }
 
 static int res_poll(void *, uint32_t slot, uint64_t ticket, int *complete) {
     Residency &r = g_engine.residency;
-    if (!r.ready || r.poisoned || !complete || ticket == 0 || slot >= r.plan.slot_count || r.slot_ticket[slot] != ticket)
-        return -1;
-    const hipError_t q = hipEventQuery(r.events[slot]);
-    if (q == hipErrorNotReady) { *complete = 0; return 0; }
-    if (q != hipSuccess) return hip_ok(q, "residency poll");
-    const uint32_t st = r.slot_staging[slot];
-    if (st >= r.plan.staging_count || r.staging_ticket[st] != ticket) return -1;
-    r.slot_ticket[slot] = 0; r.staging_ticket[st] = 0; r.slot_staging[slot] = UINT32_MAX;
+    if (!r.live || r.broken || !complete || ticket == 0 || slot >= r.seat_buffer.size()) return -1;
+    const uint32_t b = r.seat_buffer[slot];
+    if (b == Residency::kNone || r.buffers[b].ticket != ticket || r.buffers[b].seat != slot) return -1;
+    const hipError_t state = hipEventQuery(r.buffers[b].copied);
+    if (state == hipErrorNotReady) { *complete = 0; return 0; }
+    if (state != hipSuccess) return hip_ok(state, "residency: seat copy");
+    r.buffers[b].ticket = 0;
+    r.buffers[b].seat = Residency::kNone;
+    r.seat_buffer[slot] = Residency::kNone;
     *complete = 1;
     return 0;
 }
 
 static int res_resolve(void *, uint64_t device_offset, size_t nbytes, uintptr_t *address) {
     Residency &r = g_engine.residency;
-    if (!r.ready || r.poisoned || !address || nbytes == 0 || device_offset > r.plan.device_budget_bytes ||
-        nbytes > r.plan.device_budget_bytes - device_offset)
-        return -1;
+    if (!r.live || r.broken || !address || nbytes == 0) return -1;
+    if (device_offset > r.plan.device_budget_bytes || nbytes > r.plan.device_budget_bytes - device_offset) return -1;
     *address = (uintptr_t)(r.arena + device_offset);
     return 0;
 }
 
+// The seat is about to be given to another expert: a fill that is still running must end, and no kernel may still
+// read the old bytes.
 static int res_retire(void *, uint32_t slot, uint64_t) {
     Residency &r = g_engine.residency;
-    if (!r.ready || r.poisoned || slot >= r.plan.slot_count) return -1;
-    const uint64_t ticket = r.slot_ticket[slot];
-    const uint32_t st = r.slot_staging[slot];
-    if (ticket != 0) {
-        if (hip_ok(hipEventSynchronize(r.events[slot]), "residency retire") != 0) return -1;
-        if (st >= r.plan.staging_count || r.staging_ticket[st] != ticket) return -1;
-        r.staging_ticket[st] = 0;
-    } else if (st != UINT32_MAX) {
-        return -1;
+    if (!r.live || r.broken || slot >= r.seat_buffer.size()) return -1;
+    const uint32_t b = r.seat_buffer[slot];
+    if (b != Residency::kNone) {
+        if (b >= r.buffers.size() || r.buffers[b].seat != slot) return -1;
+        if (hip_ok(hipEventSynchronize(r.buffers[b].copied), "residency: retire waits for the fill") != 0) return -1;
+        r.buffers[b].ticket = 0;
+        r.buffers[b].seat = Residency::kNone;
+        r.seat_buffer[slot] = Residency::kNone;
     }
-    // kernels of the compute stream may still be reading the seat
     if (salt_gpu_sync() != 0 || drain_device() != 0) return -1;
-    r.slot_ticket[slot] = 0; r.slot_staging[slot] = UINT32_MAX;
     return 0;
 }
 
 static int res_destroy(void *) {
     Residency &r = g_engine.residency;
-    if (!r.ready && !r.poisoned) return -1;
+    if (!r.live && !r.broken) return -1;
     int failed = drain_device();
     for (Seat &s : g_engine.seats)
         if (s.active && s.resident) { g_engine.logical_seat[(size_t)s.logical_id] = -1; s = Seat(); }
@@ -1787,11 +1820,7 @@ static int res_destroy(void *) {
     }
     g_engine.pool_layout_bytes = g_engine.pool_layout_max_span = 0;
     g_engine.pool_span_count = 0;
-    for (hipEvent_t ev : r.events) if (ev) failed |= hip_ok(hipEventDestroy(ev), "hipEventDestroy");
-    if (r.stream) failed |= hip_ok(hipStreamDestroy(r.stream), "hipStreamDestroy");
-    if (r.staging) failed |= hip_ok(hipHostFree(r.staging), "hipHostFree");
-    if (r.arena) failed |= hip_ok(hipFree(r.arena), "hipFree");
-    r = Residency();
+    failed |= residency_release(r);
     return failed ? -1 : 0;
 }
 
@@ -1859,7 +1888,7 @@ static int res_permanent_copy(void *, uint32_t span_index, uint64_t device_offse
                               uint64_t ticket) {
     Engine &e = g_engine;
     Residency &r = e.residency;
-    if (!r.ready || r.poisoned || r.published || ticket == 0 || nbytes == 0 || span_index >= e.pool_span_count ||
+    if (!r.live || r.broken || r.published || ticket == 0 || nbytes == 0 || span_index >= e.pool_span_count ||
         span_index >= e.regions.size() || staging_slot >= r.plan.staging_count || nbytes > r.plan.staging_bytes)
         return -1;
     Region &g = e.regions[span_index];
@@ -1868,10 +1897,12 @@ static int res_permanent_copy(void *, uint32_t span_index, uint64_t device_offse
         set_error("permanent copy: chunks of a span arrive in order and stay inside the permanent part of the arena");
         return -1;
     }
-    if (hip_ok(hipMemcpyAsync(r.arena + device_offset, r.staging + (size_t)staging_slot * r.plan.staging_bytes, nbytes,
-                              hipMemcpyHostToDevice, r.stream), "permanent span copy") != 0)
+    const hipStream_t lane = r.lane_of(staging_slot);
+    if (r.buffers[staging_slot].ticket != 0) return -1;      // a seat fill still reads this buffer
+    if (hip_ok(hipMemcpyAsync(r.arena + device_offset, r.staging_at(staging_slot), nbytes, hipMemcpyHostToDevice, lane),
+               "permanent span copy") != 0)
         return -1;
-    if (hip_ok(hipStreamSynchronize(r.stream), "permanent span copy") != 0) { r.poisoned = 1; return -1; }
+    if (hip_ok(hipStreamSynchronize(lane), "permanent span copy") != 0) { r.broken = 1; return -1; }
     g.populated += nbytes;                                   // the staging slot is free again on return
     return 0;
 }
@@ -1879,7 +1910,7 @@ static int res_permanent_copy(void *, uint32_t span_index, uint64_t device_offse
 static int res_permanent_publish(void *) {
     Engine &e = g_engine;
     Residency &r = e.residency;
-    if (!r.ready || r.poisoned || r.published || e.pool_span_count == 0 || e.pool_span_count != e.regions.size()) return -1;
+    if (!r.live || r.broken || r.published || e.pool_span_count == 0 || e.pool_span_count != e.regions.size()) return -1;
     uint64_t total = 0;
     for (const Region &g : e.regions)
         if (g.populated != g.nbytes || g.arena_offset > r.plan.permanent_bytes ||

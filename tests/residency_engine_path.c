@@ -28,6 +28,9 @@
 #include "salt/salt.h"
 #include "gemma4.h"
 
+/* device-to-host copy helper of the backend library (include/salt_gpu_mi355.h) */
+int salt_mi355_dev_download(void *host_dst, const void *device_src, size_t nbytes);
+
 #include <fcntl.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -438,6 +441,66 @@ int main(int argc, char **argv) {
     salt_cache_free(&cache);
     CHECK(salt_gpu_residency_destroy(&model.residency) == 0);
     free(model.arena);
+
+    /* phase 3: the ledger driven the way a prefetcher would: a fill is begun on every staging buffer before the
+     * first is polled, so the engine's read of the next expert overlaps the copies of the previous ones (the cache's
+     * bind hook of phases 1 and 2, like the model's, waits for each fill before it begins the next). */
+    {
+        const uint32_t seats = 512, staging = 8;
+        const int layer = real_layers[0];
+        uint64_t tickets[512];
+        uint8_t *back = malloc(SLOT_BYTES);
+        memset(&model, 0, sizeof model);
+        CHECK(back && open_residency(&model, seats, staging, 0, &layout) == 0);
+        t0 = now_s();
+        for (uint32_t seat = 0; seat < seats; seat++) {
+            SaltGpuResidencySource source;
+            const int expert = (int)(seat % EXPERTS);
+            const uint64_t logical = (uint64_t)layer * EXPERTS + (uint64_t)expert;
+            const uint8_t *payload = salt_pool_expert_ptr(&pool, (size_t)layer * EXPERTS + (size_t)expert, SLOT_BYTES);
+            CHECK(payload != NULL);
+            if (seat >= staging) {                       /* the staging buffer about to be reused must be drained */
+                const uint32_t old = seat - staging;
+                int polled;
+                do polled = salt_gpu_residency_population_poll(&model.residency, old, (uint64_t)layer * EXPERTS + old % EXPERTS,
+                                                               old + 1u, tickets[old]);
+                while (polled == 0);
+                CHECK(polled == 1);
+            }
+            memset(&source, 0, sizeof source);
+            source.resource.kind = SALT_GPU_RESOURCE_EXPERT_LAYER;
+            source.resource.resource_id = (uint32_t)logical;
+            source.logical_resource_id = logical;
+            source.nbytes = SLOT_BYTES;
+            source.read = payload_read;
+            source.read_context = (void *)payload;
+            CHECK(salt_gpu_residency_population_begin(&model.residency, seat, seat + 1u, &source, seat % staging,
+                                                      &tickets[seat]) == 0);
+        }
+        for (uint32_t seat = seats - staging; seat < seats; seat++) {
+            int polled;
+            do polled = salt_gpu_residency_population_poll(&model.residency, seat, (uint64_t)layer * EXPERTS + seat % EXPERTS,
+                                                           seat + 1u, tickets[seat]);
+            while (polled == 0);
+            CHECK(polled == 1);
+        }
+        t1 = now_s();
+        printf("residency-engine-path: %u seats filled with %u fills in flight: %.1f GB/s\n", seats, staging,
+               (double)seats * SLOT_BYTES / 1e9 / (t1 - t0));
+        for (uint32_t seat = 0; seat < seats; seat += 37) {          /* the seats hold the experts' bytes */
+            SaltGpuResidencyBinding binding;
+            uintptr_t address = 0;
+            CHECK(salt_gpu_residency_acquire(&model.residency, seat, (uint64_t)layer * EXPERTS + seat % EXPERTS, seat + 1u,
+                                             &binding) == 1);
+            CHECK(salt_gpu_residency_resolve(&model.residency, &binding, &address) == 0);
+            CHECK(salt_mi355_dev_download(back, (const void *)address, SLOT_BYTES) == 0);
+            CHECK(memcmp(back, salt_pool_expert_ptr(&pool, (size_t)layer * EXPERTS + seat % EXPERTS, SLOT_BYTES), SLOT_BYTES) == 0);
+            CHECK(salt_gpu_residency_release(&model.residency, &binding) == 0);
+        }
+        CHECK(salt_gpu_residency_destroy(&model.residency) == 0);
+        free(model.arena);
+        free(back);
+    }
     CHECK(salt_gpu_shared_buffer_free(&b.in) == 0 && salt_gpu_shared_buffer_free(&b.out) == 0);
     CHECK(salt_gpu_shared_buffer_free(&b.gate) == 0 && salt_gpu_shared_buffer_free(&b.up) == 0);
     CHECK(salt_gpu_weight_resource_deactivate(SALT_GPU_RESOURCE_TRUNK, 0) == 0);
