@@ -1088,13 +1088,28 @@ int moe_chain(const SaltGpuMoeExpert *experts, int count, int hidden, int routed
     const size_t in_floats = (size_t)rows * hidden, mid_floats = (size_t)rows * routed;
     const size_t dev_bytes = align_up(in_floats * 4, 256) * 2 + align_up(mid_floats * 4, 256) * 3;
     if (staging_reserve(align_up(in_floats * 4, 256) * 2, dev_bytes) != 0) return -1;
-    const float *x_dev = upload_activations(inputs, in_floats);
+    // Activations that already sit in a shared buffer (pinned, with a device view: the selected chain's contract) skip
+    // the host copies through the staging memory: the device copies the inputs straight out of the buffer, and small
+    // results are written through the buffer's device view, so that nothing is left to publish.
+    const uint8_t *in_view = seats_only ? (const uint8_t *)shared_device_view(inputs, in_floats * 4) : nullptr;
+    uint8_t *out_view = seats_only ? (uint8_t *)shared_device_view(outputs, in_floats * 4) : nullptr;
+    const float *x_dev;
+    if (in_view) {
+        uint8_t *dev = device_take(in_floats * 4);
+        if (hip_ok(hipMemcpyAsync(dev, inputs, in_floats * 4, hipMemcpyHostToDevice, g_state.stream), "activation upload") != 0)
+            return -1;
+        x_dev = (const float *)dev;
+    } else {
+        x_dev = upload_activations(inputs, in_floats);
+    }
     if (!x_dev) return -1;
     float *gate_dev = (float *)device_take(mid_floats * 4), *up_dev = (float *)device_take(mid_floats * 4);
     float *act_dev = (float *)device_take(mid_floats * 4);
     uint8_t *out_dev = device_take(in_floats * 4), *out_pin = pinned_take(in_floats * 4);
-    const bool out_in_place = zero_copy(in_floats * 4);
-    if (out_in_place) out_dev = pinned_device_view(out_pin);
+    const bool out_direct = out_view != nullptr && zero_copy(in_floats * 4);
+    const bool out_in_place = out_direct || zero_copy(in_floats * 4);
+    if (out_direct) out_dev = out_view;
+    else if (out_in_place) out_dev = pinned_device_view(out_pin);
     std::vector<HostJob> jobs;
     size_t row = 0;
     for (int i = 0; i < count; ++i) {
@@ -1125,7 +1140,7 @@ int moe_chain(const SaltGpuMoeExpert *experts, int count, int hidden, int routed
             (void)salt_gpu_sync();
             return -1;
         }
-        e.pending.push_back({out_pin, outputs, in_floats * 4});
+        if (!out_direct) e.pending.push_back({out_pin, outputs, in_floats * 4});
         std::vector<OutputCopy> copies;
         if (!out_in_place) copies.push_back(OutputCopy{out_dev, out_pin, in_floats * 4});
         count_batch(experts[0].gate_vals, any_legacy);
@@ -1142,7 +1157,7 @@ int moe_chain(const SaltGpuMoeExpert *experts, int count, int hidden, int routed
         row += (size_t)g;
     }
     if (run_q4_jobs(jobs, routed, &none) != 0) { (void)salt_gpu_sync(); return -1; }
-    e.pending.push_back({out_pin, outputs, in_floats * 4});
+    if (!out_direct) e.pending.push_back({out_pin, outputs, in_floats * 4});
     std::vector<OutputCopy> copies;
     if (!out_in_place) copies.push_back(OutputCopy{out_dev, out_pin, in_floats * 4});
     count_batch(experts[0].gate_vals, any_legacy);
