@@ -362,7 +362,7 @@ int salt_mi355_q4_jobs_t_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int t
         long long blocks = 0;
         for (int j = 0; j < njobs; ++j) blocks += (jobs[j].rows + DOT_BLOCK_ROWS - 1) / DOT_BLOCK_ROWS;
         const DotShape shape = q4_dot_shape(C, group, blocks);
-        const int rows_per_wg = shape.waves / shape.ksplit * DOT_BLOCK_ROWS;
+        const int rows_per_wg = shape.waves / shape.ksplit * shape.blocks_per_wave * DOT_BLOCK_ROWS;
         int wgs = 0;
         bool uniform = true;
         for (int j = 0; j < njobs; ++j) {

@@ -89,8 +89,9 @@ constexpr int DOT_MAX_COLS = 8192;         // callers send everything else to th
 constexpr int DOT_LDS_LIMIT = 160 * 1024;
 
 // How a launch is cut: waves per workgroup, steps of LDS per wave, parts a row is cut into along its columns
-// (ksplit waves share one block of 32 rows; a workgroup owns waves / ksplit blocks).
-struct DotShape { int waves, stages, ksplit; };
+// (ksplit waves share one block of 32 rows), consecutive blocks a wave walks back to back (1 or 2).  A workgroup owns
+// waves / ksplit * blocks_per_wave blocks.
+struct DotShape { int waves, stages, ksplit, blocks_per_wave; };
 
 struct Q4DotLaunch {
     Q4Job one;                // used when table == nullptr; tile0 = index of the job's first workgroup

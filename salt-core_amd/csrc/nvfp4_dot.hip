@@ -373,9 +373,9 @@ DotShape fp4_dot_shape(int cols, int tokens, long long total_blocks) {
     while ((nstage + ksplit - 1) / ksplit * STAGE_GROUPS > 32) ksplit *= 2;
     while (ksplit > 1 && ksplit > nstage) ksplit /= 2;
     // the activation codes are small: two workgroups of four waves fit every supported column count
-    if (ksplit <= 4 && 2 * fp4_dot_lds_bytes(cols, tokens, 4, 2) <= DOT_LDS_LIMIT) return DotShape{4, 2, ksplit};
-    if (fp4_dot_lds_bytes(cols, tokens, 8, 2) <= DOT_LDS_LIMIT) return DotShape{8, 2, ksplit};
-    return DotShape{4, 2, ksplit <= 4 ? ksplit : 4};
+    if (ksplit <= 4 && 2 * fp4_dot_lds_bytes(cols, tokens, 4, 2) <= DOT_LDS_LIMIT) return DotShape{4, 2, ksplit, 1};
+    if (fp4_dot_lds_bytes(cols, tokens, 8, 2) <= DOT_LDS_LIMIT) return DotShape{8, 2, ksplit, 1};
+    return DotShape{4, 2, ksplit <= 4 ? ksplit : 4, 1};
 }
 
 int fp4_dot_launch(const Fp4DotLaunch &launch, const DotShape &shape, hipStream_t stream) {

@@ -84,8 +84,13 @@ __device__ __forceinline__ Q4Job dot_find_job(const Q4DotLaunch &L, int wg) {
 // workgroup derives its gate or up job from the selection (one workgroup past the jobs publishes selection, weights
 // and status); 2 = the down projection of one selected expert, whose activation gelu_tanh(gate) * up is computed
 // while the digit planes are built.
-template <int T, int WAVES, int STAGES, int MD, int PRO = 0>
+//
+// NB = 2 gives every wave two consecutive blocks of 32 rows, walked back to back as one stream of steps (the second
+// block's first loads go out while the first block's last steps are consumed): launches with many blocks, rows not
+// cut, MD = 16.  Both blocks' scales and biases are fetched before the stream starts.
+template <int T, int WAVES, int STAGES, int MD, int PRO = 0, int NB = 1>
 __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L) {
+    static_assert(NB == 1 || (NB == 2 && MD == 16 && PRO == 0), "two blocks per wave: plain jobs, short rows");
     static_assert(T >= 1 && T <= 4 && STAGES >= 2 && STAGES <= 4 && (MD == 16 || MD == 32), "tokens per pass, steps per wave");
     static_assert(PRO == 0 || (T == 1 && sizeof(RouterShared) <= (size_t)WAVES * STAGES * STEP_LDS),
                   "the MoE prologues serve one token; the router borrows the weight staging memory");
@@ -164,11 +169,19 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
     uint8_t *const img_lds = zero_lds + ZERO_BYTES;                        // [T][2 * SG][GROUP_IMAGE]
     float *const xm_lds = (float *)(img_lds + (size_t)T * 2 * SG * GROUP_IMAGE);   // [T][2 * SG] (power of two, sum)
 
-    // the wave's block and its stream of steps
-    const int row_base = (((int)blockIdx.x - job.tile0) * blocks_per_wg + my_block) * BLOCK_ROWS;
-    const bool has_rows = my_block < blocks_per_wg && row_base < job.rows;   // a wave without rows still helps with the activations
-    const int rows_here = !has_rows ? 1 : (job.rows - row_base < BLOCK_ROWS ? job.rows - row_base : BLOCK_ROWS);
-    const int total_steps = has_rows ? step_hi - step_lo : 0;
+    // the wave's blocks and its stream of steps
+    const int row_base0 = (((int)blockIdx.x - job.tile0) * blocks_per_wg + my_block) * (NB * BLOCK_ROWS);
+    auto row_base_of = [&](int b) { return row_base0 + b * BLOCK_ROWS; };
+    auto rows_of = [&](int b) {                       // 1..32; a block past the job's rows is never walked
+        const int left = job.rows - row_base_of(b);
+        return left < 1 ? 1 : (left < BLOCK_ROWS ? left : BLOCK_ROWS);
+    };
+    int live_blocks = 0;                             // a wave without rows still helps with the activations
+#pragma unroll
+    for (int b = 0; b < NB; ++b) live_blocks += my_block < blocks_per_wg && row_base_of(b) < job.rows;
+    const bool has_rows = live_blocks > 0;
+    const int steps_per_block = step_hi - step_lo;
+    const int total_steps = live_blocks * steps_per_block;
 
     // ---------------------------------------------------------------- per-lane geometry
     // weights: load k of a step covers strip k / 4, rows 8 (k % 4) .. + 7 of the block; lane i lands in slot 64 k + i,
@@ -206,23 +219,25 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
 
     // ---------------------------------------------------------------- loads
     // The block's scales and biases: lane (n, h) fetches 2 * MD groups of row n, 16 bytes at a time.
-    typedef uint32_t MetaVec __attribute__((ext_vector_type(MD)));
-    MetaRegs<MD> scales_r, biases_r;
+    typedef uint32_t MetaVec __attribute__((ext_vector_type(MD * NB)));
+    MetaRegs<MD> scales_r[NB], biases_r[NB];
     MetaVec scales_v, biases_v;                      // the same registers as one indexable vector, valid after the wait
-    auto issue_meta = [&]() {
+    auto issue_meta = [&](int b) {
+        const int rows_here = rows_of(b);
         const int row = n < rows_here ? n : rows_here - 1;
-        const size_t at = ((size_t)(row_base + row) * ngrp + (h ? window1 : window0)) * 2;
+        const size_t at = ((size_t)(row_base_of(b) + row) * ngrp + (h ? window1 : window0)) * 2;
 #pragma unroll
         for (int q = 0; q < MD / 4; ++q) {
             // pieces past the window are not fetched (and never read): the address repeats the last real one
             const int piece = 8 * q < meta_groups ? q : (meta_groups - 1) / 8;
-            scales_r.q[q] = load_meta16(job.scales + at + 16 * piece);
-            biases_r.q[q] = load_meta16((no_bias ? job.scales : job.biases) + at + 16 * piece);
+            scales_r[b].q[q] = load_meta16(job.scales + at + 16 * piece);
+            biases_r[b].q[q] = load_meta16((no_bias ? job.scales : job.biases) + at + 16 * piece);
         }
     };
-    // Step st into ring slot `slot`: eight weight pieces.
-    auto issue_step = [&](int st, int slot) {
-        const uint8_t *const block_vals = job.vals + (size_t)row_base * row_bytes;
+    // Step st of the wave's block b into ring slot `slot`: eight weight pieces.
+    auto issue_step = [&](int b, int st, int slot) {
+        const int rows_here = rows_of(b);
+        const uint8_t *const block_vals = job.vals + (size_t)row_base_of(b) * row_bytes;
         uint8_t *const stage = my_lds + slot * STEP_LDS;
         const uint32_t advance = (uint32_t)st * (STAGE_GROUPS * 32);
         if (rows_here == BLOCK_ROWS && st < whole_steps) {
@@ -261,7 +276,7 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
             w.raw[u][4] = w1.x; w.raw[u][5] = w1.y; w.raw[u][6] = w1.z; w.raw[u][7] = w1.w;
         }
     };
-    auto consume = [&](int st, const StepWeights &w) {
+    auto consume = [&](int b, int st, const StepWeights &w) {
         const uint8_t *a_ptr = a_base + (uint32_t)st * a_step;
         // the step's four scales and four biases: two dwords each out of the lane's registers, at a wave-uniform
         // index for either strip (groups past the row's end have zero digits; they take whatever the clamped index
@@ -272,8 +287,8 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
             auto pick = [&](const MetaVec &m, int dword) -> uint32_t { return m[dword]; };
             const int last = MD - 2;
             const int at0 = 2 * (st - step_lo) + (shift0 >> 1), at1 = 2 * (st - step_lo) + (shift1 >> 1);
-            const int i0 = at0 < last ? at0 : last;
-            const int i1 = at1 < last ? at1 : last;
+            const int i0 = b * MD + (at0 < last ? at0 : last);
+            const int i1 = b * MD + (at1 < last ? at1 : last);
             uint32_t s_lo = pick(scales_v, i0), s_hi = pick(scales_v, i0 + 1);
             uint32_t b_lo = pick(biases_v, i0), b_hi = pick(biases_v, i0 + 1);
             if (i1 != i0) {                        // uniform
@@ -337,7 +352,9 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
 
     // The two strips of a row meet; with the row cut into parts, every wave leaves its sums in its own (now idle)
     // LDS and the first wave of the block adds them in part order.
-    auto finish_block = [&]() {
+    auto finish_block = [&](int b) {
+        const int row_base = row_base_of(b), rows_here = rows_of(b);
+        const bool block_has_rows = my_block < blocks_per_wg && row_base < job.rows;
         float sum[T];
 #pragma unroll
         for (int t = 0; t < T; ++t) sum[t] = acc[t] + __shfl_xor(acc[t], 32, 64);
@@ -357,10 +374,12 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
                 sum[t] = total;
             }
         }
-        if (has_rows && lane < rows_here) {
+        if (block_has_rows && lane < rows_here) {
 #pragma unroll
             for (int t = 0; t < T; ++t) job.y[(size_t)t * job.y_stride + row_base + lane] = sum[t];
         }
+#pragma unroll
+        for (int t = 0; t < T; ++t) acc[t] = 0.0f;
     };
 
     // ---------------------------------------------------------------- activations -> digit planes (all waves)
@@ -436,8 +455,13 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
     // only loads that return to registers, are waited for with everything that is in flight at that moment, once.
     // Blocks start their walk over the row at different steps: rows whose length is a power of two put the same
     // step of every row on the same memory channels, and waves that all began at step 0 would queue there.
-    const int first_step = total_steps > 0 ? (int)(((unsigned)blockIdx.x * WAVES + wave) % (unsigned)total_steps) : 0;
-    auto step_of = [&](int g) { const int st = g + first_step; return step_lo + (st < total_steps ? st : st - total_steps); };
+    const int first_step = steps_per_block > 0 ? (int)(((unsigned)blockIdx.x * WAVES + wave) % (unsigned)steps_per_block) : 0;
+    // step g of the stream: block g / steps_per_block, and inside the block the walk that starts at first_step
+    auto block_of = [&](int g) { return NB == 1 ? 0 : g / steps_per_block; };
+    auto step_of = [&](int g) {
+        const int st = (NB == 1 ? g : g - block_of(g) * steps_per_block) + first_step;
+        return step_lo + (st < steps_per_block ? st : st - steps_per_block);
+    };
     if (PRO == 1) {
         const MoeFuse &m = L.moe;
         // first touch of the router's inputs now: they arrive while the digit planes are built
@@ -466,22 +490,27 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
         job.biases = job.scales + meta_bytes;
     }
     if (has_rows) {
-        issue_meta();
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+            if (b < live_blocks) issue_meta(b);
 #pragma unroll
         for (int g = 0; g < STAGES; ++g)
-            if (g < total_steps) issue_step(step_of(g), g);
+            if (g < total_steps) issue_step(block_of(g), step_of(g), g);
     }
     if (PRO != 1 && !(L.debug & 2)) build_image();
     __syncthreads();
     if (has_rows) {
 #pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
     for (int q = 0; q < MD / 4; ++q) {
-        wait_meta(scales_r.q[q]);
-        wait_meta(biases_r.q[q]);
+        if (b >= live_blocks) { scales_r[b].q[q] = u32x4{0u, 0u, 0u, 0u}; biases_r[b].q[q] = u32x4{0u, 0u, 0u, 0u}; }
+        wait_meta(scales_r[b].q[q]);
+        wait_meta(biases_r[b].q[q]);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            scales_v[4 * q + e] = scales_r.q[q][e];
-            biases_v[4 * q + e] = biases_r.q[q][e];
+            scales_v[b * MD + 4 * q + e] = scales_r[b].q[q][e];
+            biases_v[b * MD + 4 * q + e] = biases_r[b].q[q][e];
         }
     }
     if ((shift0 | shift1) & 1) {
@@ -489,8 +518,8 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
         // one group (16 bits), so that a step's four again fill two whole registers
         const bool odd = ((h ? shift1 : shift0) & 1) != 0;
 #pragma unroll
-        for (int i = 0; i < MD; ++i) {
-            const uint32_t s_next = i + 1 < MD ? scales_v[i + 1] : 0u, b_next = i + 1 < MD ? biases_v[i + 1] : 0u;
+        for (int i = 0; i < MD * NB; ++i) {
+            const uint32_t s_next = (i + 1) % MD ? scales_v[i + 1] : 0u, b_next = (i + 1) % MD ? biases_v[i + 1] : 0u;
             const uint32_t s_moved = __builtin_amdgcn_alignbit(s_next, scales_v[i], 16);
             const uint32_t b_moved = __builtin_amdgcn_alignbit(b_next, biases_v[i], 16);
             scales_v[i] = odd ? s_moved : scales_v[i];
@@ -515,14 +544,16 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
             fetch(r, w);
             // the reads have returned before the slot is written again
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            if (!(L.debug & 4) && g + STAGES < total_steps) issue_step(step_of(g + STAGES), r);
-            if (!(L.debug & 8)) consume(step_of(g), w);
+            if (!(L.debug & 4) && g + STAGES < total_steps) issue_step(block_of(g + STAGES), step_of(g + STAGES), r);
+            if (!(L.debug & 8)) consume(block_of(g), step_of(g), w);
+            // the last step of a block that is not the wave's last: its rows are complete
+            if (NB > 1 && (g + 1) % steps_per_block == 0 && g + 1 < total_steps) finish_block(block_of(g));
             return true;
         });
         if (!more) break;
     }
     }   // has_rows
-    finish_block();
+    finish_block(live_blocks > 0 ? live_blocks - 1 : 0);
 }
 
 size_t dot_lds_bytes(int cols, int tokens, int waves, int stages) {
@@ -530,20 +561,20 @@ size_t dot_lds_bytes(int cols, int tokens, int waves, int stages) {
     return (size_t)waves * stages * STEP_LDS + ZERO_BYTES + (size_t)tokens * 2 * sg * (GROUP_IMAGE + 8);
 }
 
-template <int T, int WAVES, int STAGES, int MD, int PRO = 0>
+template <int T, int WAVES, int STAGES, int MD, int PRO = 0, int NB = 1>
 int launch_shape(const Q4DotLaunch &L, hipStream_t stream) {
     const size_t lds = dot_lds_bytes(L.cols, T, WAVES, STAGES);
     static size_t raised = 0;                 // per instantiation: the largest dynamic LDS size asked for so far
     if (lds > raised) {
-        if (hipFuncSetAttribute((const void *)q4_dot_kernel<T, WAVES, STAGES, MD, PRO>,
+        if (hipFuncSetAttribute((const void *)q4_dot_kernel<T, WAVES, STAGES, MD, PRO, NB>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
             return -1;
         raised = lds;
     }
-    note_kernel("q4_dot_kernel<%d,%d,%d,%d,%d>", T, WAVES, STAGES, MD, PRO);
+    note_kernel("q4_dot_kernel<%d,%d,%d,%d,%d,%d>", T, WAVES, STAGES, MD, PRO, NB);
     // the router prologue has one more workgroup: the one that publishes its outputs
-    hipLaunchKernelGGL((q4_dot_kernel<T, WAVES, STAGES, MD, PRO>), dim3(L.total_wgs + (PRO == 1 ? 1 : 0)), dim3(WAVES * 64),
-                       lds, stream, L);
+    hipLaunchKernelGGL((q4_dot_kernel<T, WAVES, STAGES, MD, PRO, NB>), dim3(L.total_wgs + (PRO == 1 ? 1 : 0)),
+                       dim3(WAVES * 64), lds, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -576,9 +607,15 @@ DotShape q4_dot_shape(int cols, int tokens, long long total_blocks) {
     for (const Candidate &c : CANDIDATES)
         if ((want_waves == 0 || want_waves == c.waves) && (want_stages == 0 || want_stages == c.stages) &&
             c.waves % ksplit == 0 && (ksplit == 1 || c.waves >= 4) &&
-            dot_lds_bytes(cols, tokens, c.waves, c.stages) * c.resident <= DOT_LDS_LIMIT)
-            return DotShape{c.waves, c.stages, ksplit};
-    return DotShape{4, 2, ksplit <= 4 ? ksplit : 4};
+            dot_lds_bytes(cols, tokens, c.waves, c.stages) * c.resident <= DOT_LDS_LIMIT) {
+            // Two blocks per wave (a stream twice as long) where the launch has plenty of blocks, the rows are not
+            // cut and a lane's registers hold both blocks' scales (rows of up to 4096 columns; four or six waves).
+            static const int want_nb = env_int("SALT_MI355_DOT_BLOCKS", 0);
+            const bool can = ksplit == 1 && nstage * STAGE_GROUPS <= 32 && (c.waves == 4 || c.waves == 6) && c.stages == 2;
+            const int nb = can && (want_nb == 2 || (want_nb == 0 && total_blocks >= 2048)) ? 2 : 1;
+            return DotShape{c.waves, c.stages, ksplit, nb};
+        }
+    return DotShape{4, 2, ksplit <= 4 ? ksplit : 4, 1};
 }
 
 int q4_dot_launch(const Q4DotLaunch &launch, const DotShape &shape, hipStream_t stream) {
@@ -592,6 +629,14 @@ int q4_dot_launch(const Q4DotLaunch &launch, const DotShape &shape, hipStream_t 
     // groups of a strip that one wave walks: its registers hold 32 (MD = 16) or 64 (MD = 32)
     const int steps = dot_steps(L.cols >> 6);
     const int md = ((steps + shape.ksplit - 1) / shape.ksplit) * STAGE_GROUPS <= 32 ? 16 : 32;
+    if (shape.blocks_per_wave == 2) {
+        if (md != 16 || shape.ksplit != 1 || shape.stages != 2) return -1;
+#define DOT_NB2(TT, WW) if (L.tokens == TT && shape.waves == WW) return launch_shape<TT, WW, 2, 16, 0, 2>(L, stream)
+        DOT_NB2(1, 4); DOT_NB2(2, 4); DOT_NB2(3, 4); DOT_NB2(4, 4);
+        DOT_NB2(1, 6); DOT_NB2(2, 6); DOT_NB2(3, 6); DOT_NB2(4, 6);
+#undef DOT_NB2
+        return -1;
+    }
 #define DOT_CASE(TT, WW, SS) \
     if (L.tokens == TT && shape.waves == WW && shape.stages == SS) \
         return md == 16 ? launch_shape<TT, WW, SS, 16>(L, stream) : launch_shape<TT, WW, SS, 32>(L, stream)
