@@ -362,7 +362,8 @@ int salt_mi355_q4_jobs_t_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int t
         long long blocks = 0;
         for (int j = 0; j < njobs; ++j) blocks += (jobs[j].rows + DOT_BLOCK_ROWS - 1) / DOT_BLOCK_ROWS;
         const DotShape shape = q4_dot_shape(C, group, blocks);
-        const int rows_per_wg = shape.waves / shape.ksplit * shape.blocks_per_wave * DOT_BLOCK_ROWS;
+        const int waves16 = q4_dot16_waves(C, group, blocks);
+        const int rows_per_wg = waves16 ? waves16 * 16 : shape.waves / shape.ksplit * shape.blocks_per_wave * DOT_BLOCK_ROWS;
         int wgs = 0;
         bool uniform = true;
         for (int j = 0; j < njobs; ++j) {
@@ -394,7 +395,7 @@ int salt_mi355_q4_jobs_t_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int t
             if (!slot) return -1;
             launch.table = (const Q4Job *)slot->device;
         }
-        const int rc = q4_dot_launch(launch, shape, stream);
+        const int rc = waves16 ? q4_dot16_launch(launch, waves16, stream) : q4_dot_launch(launch, shape, stream);
         table_release(slot, stream);
         if (rc != 0) { set_error("q4 t: kernel launch failed: %s", hipGetErrorString(hipGetLastError())); return -1; }
     }

@@ -112,6 +112,10 @@ bool q4_dot_takes(int cols);
 int q4_dot_tokens_per_pass(int cols);      // 0: the column count does not fit at all
 DotShape q4_dot_shape(int cols, int tokens, long long total_blocks);
 int q4_dot_launch(const Q4DotLaunch &launch, const DotShape &shape, hipStream_t stream);
+// The same arithmetic on blocks of sixteen rows (q4_dot16.hip): one or two tokens, launches with many blocks.
+// q4_dot16_waves: waves per workgroup to use (a workgroup owns that many blocks of 16 rows), or 0 = use the 32-row kernel.
+int q4_dot16_waves(int cols, int tokens, long long total_blocks32);
+int q4_dot16_launch(const Q4DotLaunch &launch, int waves, hipStream_t stream);
 // The MoE decode step's two matvec launches on the streaming kernel (router top-k in the prologue of the first,
 // gelu_tanh(gate) * up in the prologue of the second); -1: the geometry is not served.
 int q4_dot_moe_gate_up_launch(const MoeFuse &moe, hipStream_t stream);
