@@ -1,4 +1,4 @@
-// Affine-Q4 decode matvec, tolerance class, for launches with many blocks and one or two tokens: the arithmetic and
+// Affine-Q4 decode matvec, tolerance class, for launches with many blocks (one to four tokens): the arithmetic and
 // the bound of q4_dot.hip on blocks of sixteen rows.
 //
 // Why a second shape: a step of q4_dot.hip (32 rows, 8 KiB) keeps a wave busy for about as long as two steps take to
@@ -54,10 +54,13 @@ __device__ __forceinline__ Q4Job dot16_find_job(const Q4DotLaunch &L, int wg) {
     return job;
 }
 
-// T tokens (1 or 2), WAVES waves of 16 rows per workgroup, MD dwords of scales per lane.  Two steps of LDS per wave.
+// T tokens (1..4), WAVES waves of 16 rows per workgroup, MD dwords of scales per lane.  Two steps of LDS per wave.
+// The M side of one matrix instruction holds two tokens; three or four tokens take a second pair of instructions per
+// group on the same weight registers.
 template <int T, int WAVES, int MD>
 __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch L) {
-    static_assert((T == 1 || T == 2) && (MD == 16 || MD == 32), "tokens per pass, scale registers");
+    static_assert(T >= 1 && T <= 4 && (MD == 16 || MD == 32), "tokens per pass, scale registers");
+    constexpr int SETS = (T + 1) / 2;                // pairs of tokens
     constexpr int STAGES = 2;
     constexpr int WAVE_LDS = STAGES * STEP16_BYTES;
     constexpr int THREADS = WAVES * 64;
@@ -112,20 +115,27 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch 
 #pragma unroll
     for (int u = 0; u < STAGE_GROUPS; ++u)
         rd_off[u] = (uint32_t)my_piece * 128u + (uint32_t)((2 * u + (kq & 1)) ^ swizzle(my_piece)) * 16u;
-    // results: lane (n, mq) holds row n's plane sums of strip mq % 2, token mq / 2
+    // results: lane (n, mq) holds row n's plane sums of strip mq % 2, token mq / 2 of each pair of tokens
     const int mq = kq;
     const int my_strip = mq & 1, my_token = mq >> 1;
-    const bool has_result = my_token < T;
     const bool no_bias = job.biases == nullptr;
     // digit planes: row m = l % 16 of the M side is (token m / 8, strip (m / 4) % 2, plane m % 4); it carries digits in
     // the two k-slices of its own strip
     const int m_tok = n >> 3, m_strip = (n >> 2) & 1, m_plane = n & 3;
-    const bool has_digits = m_tok < T && m_strip == (kq >> 1);
-    const uint8_t *const a_base = has_digits
-        ? img_lds + ((size_t)(m_tok * 2 * SG + m_strip * SG) * 16 + 2 * (kq & 1) * 4 + m_plane) * 16
-        : zero_lds + 64;
-    const uint32_t a_step = has_digits ? STAGE_GROUPS * GROUP_IMAGE : 0u;
-    const float *const xm_ptr = xm_lds + 2 * (my_token * 2 * SG + my_strip * SG);
+    const uint8_t *a_base[SETS];
+    uint32_t a_step[SETS];
+    const float *xm_ptr[SETS];
+#pragma unroll
+    for (int s = 0; s < SETS; ++s) {
+        const bool has_digits = 2 * s + m_tok < T && m_strip == (kq >> 1);
+        a_base[s] = has_digits
+            ? img_lds + ((size_t)((2 * s + m_tok) * 2 * SG + m_strip * SG) * 16 + 2 * (kq & 1) * 4 + m_plane) * 16
+            : zero_lds + 64;
+        a_step[s] = has_digits ? STAGE_GROUPS * GROUP_IMAGE : 0u;
+        // a lane without a token (three tokens: the second pair's upper lanes) reads token 0's factors and stores nothing
+        const int tok = 2 * s + my_token < T ? 2 * s + my_token : 0;
+        xm_ptr[s] = xm_lds + 2 * (tok * 2 * SG + my_strip * SG);
+    }
 
     // ---------------------------------------------------------------- loads
     typedef uint32_t MetaVec __attribute__((ext_vector_type(MD)));
@@ -163,7 +173,9 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch 
     };
 
     // ---------------------------------------------------------------- arithmetic of one step
-    float acc = 0.0f;
+    float acc[SETS];
+#pragma unroll
+    for (int s = 0; s < SETS; ++s) acc[s] = 0.0f;
     struct StepWeights { u32x4 group[STAGE_GROUPS]; };
     auto fetch = [&](int slot, StepWeights &w) {
         const uint8_t *stage = my_lds + slot * STEP16_BYTES;
@@ -171,7 +183,6 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch 
         for (int u = 0; u < STAGE_GROUPS; ++u) w.group[u] = *(const u32x4 *)(stage + rd_off[u]);
     };
     auto consume = [&](int st, const StepWeights &w) {
-        const uint8_t *a_ptr = a_base + (uint32_t)st * a_step;
         // the step's four scales and four biases of the lane's result strip (register indexing, wave-uniform index
         // per strip)
         float scale[STAGE_GROUPS], bias[STAGE_GROUPS];
@@ -189,36 +200,45 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch 
             scale[2] = __uint_as_float(s_hi << 16); scale[3] = __uint_as_float(s_hi & 0xffff0000u);
             bias[0] = __uint_as_float(b_lo << 16); bias[1] = __uint_as_float(b_lo & 0xffff0000u);
             bias[2] = __uint_as_float(b_hi << 16); bias[3] = __uint_as_float(b_hi & 0xffff0000u);
+            if (no_bias) { bias[0] = bias[1] = bias[2] = bias[3] = 0.0f; }
         }
-        const f32x4 xm_a = *(const f32x4 *)(xm_ptr + 2 * (st * STAGE_GROUPS));
-        const f32x4 xm_b = *(const f32x4 *)(xm_ptr + 2 * (st * STAGE_GROUPS) + 4);
-        const float xm[8] = {xm_a.x, xm_a.y, xm_a.z, xm_a.w, xm_b.x, xm_b.y, xm_b.z, xm_b.w};
-        v4i d[STAGE_GROUPS];
+        // unpacked codes of the step: the operands of both instructions of every group, shared by the token pairs
+        v4i b[STAGE_GROUPS][2];
 #pragma unroll
-        for (int u = 0; u < STAGE_GROUPS; ++u) d[u] = v4i{0, 0, 0, 0};
+        for (int u = 0; u < STAGE_GROUPS; ++u)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            v4i a[STAGE_GROUPS];
+            for (int j = 0; j < 2; ++j) {
+                const uint32_t lo = j ? w.group[u].z : w.group[u].x, hi = j ? w.group[u].w : w.group[u].y;
+                b[u][j].x = (int)(lo & 0x0f0f0f0fu);
+                b[u][j].y = (int)((lo >> 4) & 0x0f0f0f0fu);
+                b[u][j].z = (int)(hi & 0x0f0f0f0fu);
+                b[u][j].w = (int)((hi >> 4) & 0x0f0f0f0fu);
+            }
 #pragma unroll
-            for (int u = 0; u < STAGE_GROUPS; ++u) a[u] = *(const v4i *)(a_ptr + u * GROUP_IMAGE + j * 64);
+        for (int s = 0; s < SETS; ++s) {
+            const uint8_t *a_ptr = a_base[s] + (uint32_t)st * a_step[s];
+            const f32x4 xm_a = *(const f32x4 *)(xm_ptr[s] + 2 * (st * STAGE_GROUPS));
+            const f32x4 xm_b = *(const f32x4 *)(xm_ptr[s] + 2 * (st * STAGE_GROUPS) + 4);
+            const float xm[8] = {xm_a.x, xm_a.y, xm_a.z, xm_a.w, xm_b.x, xm_b.y, xm_b.z, xm_b.w};
+            v4i d[STAGE_GROUPS];
+#pragma unroll
+            for (int u = 0; u < STAGE_GROUPS; ++u) d[u] = v4i{0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                v4i a[STAGE_GROUPS];
+#pragma unroll
+                for (int u = 0; u < STAGE_GROUPS; ++u) a[u] = *(const v4i *)(a_ptr + u * GROUP_IMAGE + j * 64);
+#pragma unroll
+                for (int u = 0; u < STAGE_GROUPS; ++u) d[u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[u], b[u][j], d[u], 0, 0, 0);
+            }
 #pragma unroll
             for (int u = 0; u < STAGE_GROUPS; ++u) {
-                const uint32_t lo = j ? w.group[u].z : w.group[u].x, hi = j ? w.group[u].w : w.group[u].y;
-                v4i b;
-                b.x = (int)(lo & 0x0f0f0f0fu);
-                b.y = (int)((lo >> 4) & 0x0f0f0f0fu);
-                b.z = (int)(hi & 0x0f0f0f0fu);
-                b.w = (int)((hi >> 4) & 0x0f0f0f0fu);
-                d[u] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[u], b, d[u], 0, 0, 0);
+                const int lo = d[u].x + (d[u].y << 8);
+                const int hi = d[u].z + (d[u].w << 8);
+                const float f = __builtin_fmaf((float)hi, 65536.0f, (float)lo);
+                acc[s] = __builtin_fmaf(scale[u] * xm[2 * u], f, acc[s]);
+                acc[s] = __builtin_fmaf(bias[u], xm[2 * u + 1], acc[s]);
             }
-        }
-#pragma unroll
-        for (int u = 0; u < STAGE_GROUPS; ++u) {
-            const int lo = d[u].x + (d[u].y << 8);
-            const int hi = d[u].z + (d[u].w << 8);
-            const float f = __builtin_fmaf((float)hi, 65536.0f, (float)lo);
-            acc = __builtin_fmaf(scale[u] * xm[2 * u], f, acc);
-            acc = __builtin_fmaf(no_bias ? 0.0f : bias[u], xm[2 * u + 1], acc);
         }
     };
 
@@ -273,9 +293,12 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch 
         if (!more) break;
     }
     // the two strips of a row meet: lanes (n, 2t) and (n, 2t + 1)
-    const float other = __shfl_xor(acc, 16, 64);
-    if (has_result && my_strip == 0 && n < rows_here)
-        job.y[(size_t)my_token * job.y_stride + row_base + n] = acc + other;
+#pragma unroll
+    for (int s = 0; s < SETS; ++s) {
+        const float other = __shfl_xor(acc[s], 16, 64);
+        const int token = 2 * s + my_token;
+        if (token < T && my_strip == 0 && n < rows_here) job.y[(size_t)token * job.y_stride + row_base + n] = acc[s] + other;
+    }
 }
 
 size_t dot16_lds_bytes(int cols, int tokens, int waves) {
@@ -304,7 +327,7 @@ int launch16(const Q4DotLaunch &L, hipStream_t stream) {
 // two workgroups per compute unit where the digit planes leave room, else one of twelve waves.
 int q4_dot16_waves(int cols, int tokens, long long total_blocks32) {
     static const int want = env_int("SALT_MI355_DOT16", -1);           // 0 forbids the shape, 8 / 12 force it
-    if (want == 0 || tokens > 2 || !q4_dot_takes(cols)) return 0;
+    if (want == 0 || tokens > 4 || !q4_dot_takes(cols)) return 0;
     if (want != 8 && want != 12 && total_blocks32 < 2048) return 0;     // few blocks: the 32-row kernel cuts rows instead
     if ((want == -1 || want == 8) && 2 * dot16_lds_bytes(cols, tokens, 8) <= DOT_LDS_LIMIT) return 8;
     if ((want == -1 || want == 12) && dot16_lds_bytes(cols, tokens, 12) <= DOT_LDS_LIMIT) return 12;
@@ -312,11 +335,13 @@ int q4_dot16_waves(int cols, int tokens, long long total_blocks32) {
 }
 
 int q4_dot16_launch(const Q4DotLaunch &L, int waves, hipStream_t stream) {
-    if (L.total_wgs < 1 || L.tokens < 1 || L.tokens > 2 || !q4_dot_takes(L.cols)) return -1;
+    if (L.total_wgs < 1 || L.tokens < 1 || L.tokens > 4 || !q4_dot_takes(L.cols)) return -1;
+    if (dot16_lds_bytes(L.cols, L.tokens, waves) > DOT_LDS_LIMIT) return -1;
     const int md = dot_steps(L.cols >> 6) * STAGE_GROUPS <= 32 ? 16 : 32;
 #define DOT16_CASE(TT, WW) \
     if (L.tokens == TT && waves == WW) return md == 16 ? launch16<TT, WW, 16>(L, stream) : launch16<TT, WW, 32>(L, stream)
-    DOT16_CASE(1, 8); DOT16_CASE(2, 8); DOT16_CASE(1, 12); DOT16_CASE(2, 12);
+    DOT16_CASE(1, 8); DOT16_CASE(2, 8); DOT16_CASE(3, 8); DOT16_CASE(4, 8);
+    DOT16_CASE(1, 12); DOT16_CASE(2, 12); DOT16_CASE(3, 12); DOT16_CASE(4, 12);
 #undef DOT16_CASE
     return -1;
 }
