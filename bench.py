@@ -45,6 +45,7 @@ INSTANCE_BYTES = 640e6                                      # distinct weight by
 # runs scaled by a copy of known size; taken from the profile summary named beside it, for the default instance
 # counts only.  bench.py does not measure it: it reports it with its source.
 TRAFFIC_FROM_PROFILE = {
+    "q4_dot16_kernel": (650_800_000, "profiles/q4_dot_kernel_decode_sweep_b1.md"),
     "q4_dot_kernel": (657_200_000, "profiles/q4_dot_kernel_decode_sweep_b1.md"),
     "q4_tile_kernel": (661_320_000, "profiles/q4_tile_kernel_decode_sweep_b1.md"),
 }
