@@ -150,6 +150,30 @@ def test_many_jobs_one_launch(pkg, oracle):
         check(got, reference(oracle, vals, scales, biases, R, Cc, xs), vals, scales, biases, R, Cc, xs)
 
 
+@pytest.mark.parametrize("R,Cc,njobs,tokens", [(2816, 2816, 24, 1), (2816, 2816, 24, 3), (8192, 8192, 8, 1), (1424, 704, 48, 2)])
+def test_launches_with_many_blocks_take_the_sixteen_row_shape(pkg, oracle, R, Cc, njobs, tokens):
+    """From 2048 blocks of 32 rows on, a launch runs on q4_dot16_kernel (16 rows per wave).  Three weight tensors are
+    shared by the jobs; every job has its own activations and outputs."""
+    lib = pkg.lib.init()
+    tensors = [synth.q4_tensor(R, Cc, 500 + k) for k in range(3)]
+    dev = [tuple(pkg.lib.DeviceBuffer.from_host(a) for a in t) for t in tensors]
+    xs = [synth.activations(Cc, tokens, 600 + j) for j in range(njobs)]
+    dxs = [pkg.lib.DeviceBuffer.from_host(x) for x in xs]
+    dys = [pkg.lib.DeviceBuffer(tokens * R * 4, fill=0xFF) for _ in range(njobs)]
+    jobs = (pkg.lib.Q4Job * njobs)()
+    for j in range(njobs):
+        dv, ds, db = dev[j % 3]
+        jobs[j] = pkg.lib.Q4Job(dv.ptr, ds.ptr, db.ptr, dxs[j].ptr, dys[j].ptr, R)
+    stream = lib.salt_mi355_stream()
+    pkg.lib.check(lib.salt_mi355_q4_jobs_t_dev(jobs, njobs, Cc, tokens, stream), "q4_jobs_t_dev")
+    pkg.lib.check(lib.salt_mi355_stream_sync(stream), "sync")
+    assert lib.salt_mi355_last_kernel().decode().startswith("q4_dot16_kernel"), lib.salt_mi355_last_kernel()
+    for j in range(0, njobs, 5):
+        vals, scales, biases = tensors[j % 3]
+        got = dys[j].to_host(np.float32).reshape(tokens, R)
+        check(got, reference(oracle, vals, scales, biases, R, Cc, xs[j]), vals, scales, biases, R, Cc, xs[j])
+
+
 def test_rejections(pkg):
     lib = pkg.lib.init()
     buf = pkg.lib.DeviceBuffer(1 << 16)
