@@ -102,7 +102,6 @@ struct Q4DotLaunch {
     int total_wgs;
     int ksplit;               // filled by q4_dot_launch from the shape
     int wgs_per_job;          // > 0 when every job of the table has this many workgroups (workgroup -> job by division)
-    int debug;
     MoeFuse moe;              // only read by q4_dot_moe_gate_up_launch / q4_dot_moe_down_launch
     // Up to Q4_INLINE_JOBS job records inside the kernel arguments (table == nullptr, njobs > 1): a decode-sized
     // batch then needs no table upload.  Must stay the last member.

@@ -93,7 +93,6 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
     static_assert(PRO == 0 || (T == 1 && sizeof(RouterShared) <= (size_t)WAVES * STAGES * STEP_LDS),
                   "the MoE prologues serve one token; the router borrows the weight staging memory");
     constexpr int WAVE_LDS = STAGES * STEP_LDS;
-    constexpr int AHEAD = STAGES - 1;                // steps in flight behind the one being consumed
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int THREADS = WAVES * 64;
 
@@ -444,7 +443,7 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
         for (int g = 0; g < STAGES; ++g)
             if (g < total_steps) issue_step(block_of(g), step_of(g), g);
     }
-    if (PRO != 1 && !(L.debug & 2)) build_image();
+    if (PRO != 1) build_image();
     __syncthreads();
     if (has_rows) {
 #pragma unroll
@@ -479,10 +478,9 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
             constexpr int r = decltype(step_in_turn)::value;       // ring slot of step base + r
             const int g = base + r;
             if (g >= total_steps) return false;
-            if (!(L.debug & 4)) {
+            {
                 const int behind = total_steps - 1 - g < STAGES - 1 ? total_steps - 1 - g : STAGES - 1;
-                if (L.debug & 1) wait_vm<0>();
-                else if (behind == 0) wait_vm<0>();
+                if (behind == 0) wait_vm<0>();
                 else if (behind == 1) wait_vm<LOADS_PER_STEP>();
                 else if (behind == 2) wait_vm<2 * LOADS_PER_STEP>();
                 else wait_vm<3 * LOADS_PER_STEP>();
@@ -491,8 +489,8 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
             fetch(r, w);
             // the reads have returned before the slot is written again
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            if (!(L.debug & 4) && g + STAGES < total_steps) issue_step(block_of(g + STAGES), step_of(g + STAGES), r);
-            if (!(L.debug & 8)) consume(block_of(g), step_of(g), w);
+            if (g + STAGES < total_steps) issue_step(block_of(g + STAGES), step_of(g + STAGES), r);
+            consume(block_of(g), step_of(g), w);
             // the last step of a block that is not the wave's last: its rows are complete
             if (NB > 1 && (g + 1) % steps_per_block == 0 && g + 1 < total_steps) finish_block(block_of(g));
             return true;
@@ -570,8 +568,6 @@ int q4_dot_launch(const Q4DotLaunch &launch, const DotShape &shape, hipStream_t 
     if (L.total_wgs < 1 || L.tokens < 1 || L.tokens > 4 || !q4_dot_takes(L.cols)) return -1;
     if (dot_lds_bytes(L.cols, L.tokens, shape.waves, shape.stages) > DOT_LDS_LIMIT) return -1;
     if (shape.ksplit < 1 || shape.waves % shape.ksplit) return -1;
-    static const int debug_env = env_int("SALT_MI355_DOT_DEBUG", 0);
-    L.debug = debug_env;
     L.ksplit = shape.ksplit;
     // groups of a strip that one wave walks: its registers hold 32 (MD = 16) or 64 (MD = 32)
     const int steps = dot_steps(L.cols >> 6);
@@ -620,8 +616,6 @@ int q4_dot_moe_gate_up_launch(const MoeFuse &m, hipStream_t stream) {
     L.ksplit = moe_dot_ksplit((long long)blocks * 2 * m.topk, m.hidden);
     L.wgs_per_job = (blocks + 4 / L.ksplit - 1) / (4 / L.ksplit);
     L.total_wgs = 2 * m.topk * L.wgs_per_job;
-    static const int debug_env = env_int("SALT_MI355_DOT_DEBUG", 0);
-    L.debug = debug_env;
     return launch_shape<1, 4, 2, 16, 1>(L, stream);
 }
 
