@@ -36,6 +36,7 @@ struct MoeFuse {
     size_t expert_stride;
     const float *x;               // [hidden]
     float *gate, *up;             // [topk][routed]
+    float *act;                   // [topk][routed]: gelu_tanh(gate) * up (the two-launch plan of moe_dot16.hip)
     float *expert_out;            // [topk][hidden]
     int *selected;                // [topk], ascending expert id
     float *weights;               // [topk]
@@ -117,6 +118,9 @@ int q4_dot16_waves(int cols, int tokens, long long total_blocks32);
 int q4_dot16_launch(const Q4DotLaunch &launch, int waves, hipStream_t stream);
 // The MoE decode step's two matvec launches on the streaming kernel (router top-k in the prologue of the first,
 // gelu_tanh(gate) * up in the prologue of the second); -1: the geometry is not served.
+// The whole step in two launches (moe_dot16.hip): gate + up + activation, then down + ordered weighted sum; `out`
+// receives the layer output, moe.expert_out (optional) the expert outputs.  -1: the geometry is not served.
+int moe16_step_launch(const MoeFuse &moe, float *out, hipStream_t stream);
 int q4_dot_moe_gate_up_launch(const MoeFuse &moe, hipStream_t stream);
 int q4_dot_moe_down_launch(const MoeFuse &moe, hipStream_t stream);
 

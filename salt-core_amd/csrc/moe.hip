@@ -218,6 +218,14 @@ int moe_decode_step_t_launch(const MoeGeometry &g, const uint8_t *pool, size_t e
     m.x = x; m.gate = ws.gate; m.up = ws.up; m.expert_out = expert_out ? expert_out : ws.expert_out;
     m.selected = selected; m.weights = weights; m.status = ws.status;
     m.n_experts = g.n_experts; m.topk = g.topk; m.hidden = g.hidden; m.routed = g.routed;
+    m.act = ws.act;
+    // two launches when the caller wants the layer output (the weighted sum rides in the down launch)
+    if (out) {
+        MoeFuse two = m;
+        two.expert_out = expert_out;              // optional there
+        if (moe16_step_launch(two, out, stream) == 0) return 0;
+        (void)hipGetLastError();
+    }
     if (q4_dot_moe_gate_up_launch(m, stream) != 0) return -1;
     if (q4_dot_moe_down_launch(m, stream) != 0) return -1;
     return out ? moe_reduce_launch(m.expert_out, weights, g.topk, g.hidden, out, ws.status, stream) : 0;
