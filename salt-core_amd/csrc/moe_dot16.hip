@@ -48,9 +48,15 @@ __global__ __launch_bounds__(2 * PARTS * 64) void moe16_gate_up_kernel(const Moe
     float *const xm_lds = (float *)(img_lds + (size_t)2 * SG * GROUP_IMAGE);
 
     const int place = (int)blockIdx.x / blocks_per_place, block = (int)blockIdx.x - place * blocks_per_place;
+    // The activation and the router's inputs are requested together, the activation first: when the logits have
+    // arrived, so has the activation, and the weight loads that follow queue behind neither.
+    const ImageItems items(1, stream.ngrp);
+    Q4ImageBuilder<THREADS> image;
+    image.request_early(tid, items, [&](int) { return m.x; });
     // every wave finds its expert on its own (with finite inputs the router cannot fail later) and sends for its
     // scales and first weights at once: they are on their way while the digit planes are built
     const int expert = router_select_wave(m.logits, m.per_expert_scale, m.n_experts, m.topk, place);
+    image.settle(expert, items);
     if (expert < 0) return;                          // uniform: every wave sees the same inputs; no barrier passed yet
     const size_t n_weights = (size_t)m.hidden * (size_t)m.routed;
     const size_t vals_bytes = n_weights / 2, meta_bytes = (n_weights / 64) * 2, proj_bytes = vals_bytes + 2 * meta_bytes;
@@ -60,9 +66,9 @@ __global__ __launch_bounds__(2 * PARTS * 64) void moe16_gate_up_kernel(const Moe
     stream.bind(vals, vals + vals_bytes, vals + vals_bytes + meta_bytes, m.routed, row_base,
                 part * stream.nstage / PARTS, (part + 1) * stream.nstage / PARTS);
     stream.start();
-    build_q4_image<1, THREADS>(tid, stream.ngrp, SG, zero_lds, img_lds, xm_lds, [&](int, size_t column, float (&xv)[4]) {
+    image.build(tid, items, SG, zero_lds, img_lds, xm_lds, [&](int, size_t column, float (&xv)[8]) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) xv[k] = m.x[column + k];
+        for (int k = 0; k < 8; ++k) xv[k] = m.x[column + k];
     });
     __syncthreads();                                 // the digit planes are in place
 
@@ -92,7 +98,16 @@ __global__ __launch_bounds__(MOE16_MAX_TOPK * 64) void moe16_down_sum_kernel(con
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    if (*(const int __attribute__((address_space(4))) *)(uintptr_t)m.status != 0) return;      // the router rejected its input
+    // what the first launch left: status, selection and routing weights, fetched in one go as wave-uniform values
+    typedef const int __attribute__((address_space(4))) *uniform_int_ptr;
+    typedef const float __attribute__((address_space(4))) *uniform_float_ptr;
+    const bool has_expert = wave < m.topk;
+    const int status = *(uniform_int_ptr)(uintptr_t)m.status;
+    const int expert = ((uniform_int_ptr)(uintptr_t)m.selected)[has_expert ? wave : 0];
+    float routing[WAVES];
+#pragma unroll
+    for (int e = 0; e < WAVES; ++e) routing[e] = ((uniform_float_ptr)(uintptr_t)m.weights)[e < m.topk ? e : 0];
+    if (status != 0) return;                         // the router rejected its input
 
     Dot16Stream<MD> stream;
     stream.setup(lane, m.routed, lds + (size_t)wave * WAVE16_LDS);
@@ -101,23 +116,19 @@ __global__ __launch_bounds__(MOE16_MAX_TOPK * 64) void moe16_down_sum_kernel(con
     uint8_t *const img_lds = zero_lds + ZERO_BYTES;                        // [expert of the selection][2 * SG][GROUP_IMAGE]
     float *const xm_lds = (float *)(img_lds + (size_t)WAVES * 2 * SG * GROUP_IMAGE);
 
-    const bool has_expert = wave < m.topk;
     const int row_base = (int)blockIdx.x * ROWS16;
     const size_t n_weights = (size_t)m.hidden * (size_t)m.routed;
     const size_t vals_bytes = n_weights / 2, meta_bytes = (n_weights / 64) * 2, proj_bytes = vals_bytes + 2 * meta_bytes;
     if (has_expert) {
-        const int expert = ((const int __attribute__((address_space(4))) *)(uintptr_t)m.selected)[wave];
         const uint8_t *vals = m.pool + (size_t)expert * m.expert_stride + 2 * proj_bytes;
         stream.bind(vals, vals + vals_bytes, vals + vals_bytes + meta_bytes, m.hidden, row_base, 0, stream.nstage);
         stream.start();
     }
     // the activations of all selected experts become digit planes: expert e of the selection is "token" e
     const int topk = m.topk;
-    build_q4_image<WAVES, THREADS>(tid, stream.ngrp, SG, zero_lds, img_lds, xm_lds, [&](int e, size_t column, float (&xv)[4]) {
-        if (e < topk) {
+    build_q4_image<0, THREADS>(tid, stream.ngrp, SG, zero_lds, img_lds, xm_lds, topk, [&](int e, size_t column, float (&xv)[8]) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) xv[k] = m.act[(size_t)e * m.routed + column + k];
-        }
+        for (int k = 0; k < 8; ++k) xv[k] = m.act[(size_t)e * m.routed + column + k];
     });
     __syncthreads();
 
@@ -137,9 +148,12 @@ __global__ __launch_bounds__(MOE16_MAX_TOPK * 64) void moe16_down_sum_kernel(con
         // reference gemma4_text.c:8301-8304: out = 0; out += o_i * w_i in ascending expert order, product and sum
         // rounded separately
         float total = 0.0f;
-        for (int e = 0; e < topk; ++e) {
-            const float term = ((const float *)(lds + (size_t)e * WAVE16_LDS))[lane] * m.weights[e];
-            total = total + term;
+#pragma unroll
+        for (int e = 0; e < WAVES; ++e) {
+            if (e < topk) {
+                const float term = ((const float *)(lds + (size_t)e * WAVE16_LDS))[lane] * routing[e];
+                total = total + term;
+            }
         }
         out[row_base + lane] = total;
     }
@@ -162,6 +176,26 @@ int raise_lds(Kernel kernel, size_t lds, size_t &raised) {
     return 0;
 }
 
+template <int PARTS, int MD>
+int launch_gate_up(const MoeFuse &m, int blocks, size_t lds, hipStream_t stream) {
+    static size_t raised = 0;
+    if (raise_lds(moe16_gate_up_kernel<PARTS, MD>, lds, raised) != 0) return -1;
+    hipLaunchKernelGGL((moe16_gate_up_kernel<PARTS, MD>), dim3(m.topk * blocks + 1), dim3(2 * PARTS * 64), lds, stream, m, blocks);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+template <int MD>
+int launch_down_sum(const MoeFuse &m, float *out, size_t lds, hipStream_t stream) {
+    static size_t raised = 0;
+    if (raise_lds(moe16_down_sum_kernel<MD>, lds, raised) != 0) return -1;
+    hipLaunchKernelGGL((moe16_down_sum_kernel<MD>), dim3((m.hidden + ROWS16 - 1) / ROWS16), dim3(MOE16_MAX_TOPK * 64), lds,
+                       stream, m, out);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// dwords of scales a lane keeps for a wave that walks `steps` steps of a strip: two groups per dword
+int meta_dwords(int steps) { return steps <= 2 ? 4 : steps <= 4 ? 8 : 16; }
+
 }  // namespace
 
 // -1: the geometry is not served (the caller takes another plan).
@@ -172,25 +206,25 @@ int moe16_step_launch(const MoeFuse &m, float *out, hipStream_t stream) {
     const int steps_hidden = dot_steps(m.hidden >> 6), steps_routed = dot_steps(m.routed >> 6);
     // three parts per matrix where the row has at least three steps, else one
     const int parts = steps_hidden >= 3 ? 3 : 1;
-    if ((steps_hidden + parts - 1) / parts * STAGE_GROUPS > 32 || steps_routed * STAGE_GROUPS > 32) return -1;   // MD = 16
+    const int steps_a = (steps_hidden + parts - 1) / parts;
+    if (steps_a > 8 || steps_routed > 8) return -1;   // a lane's registers hold the scales of at most 32 groups
     if (m.n_experts > 2 * parts * 64) return -1;      // the publishing workgroup runs the router with one thread per expert
     const size_t lds_a = moe16_gate_up_lds(m.hidden, 2 * parts), lds_b = moe16_down_lds(m.routed);
     if (lds_a > DOT_LDS_LIMIT || lds_b > DOT_LDS_LIMIT) return -1;
     const int blocks = (m.routed + ROWS16 - 1) / ROWS16;
-    static size_t raised_a3 = 0, raised_a1 = 0, raised_b = 0;
-    if (parts == 3) {
-        if (raise_lds(moe16_gate_up_kernel<3, 16>, lds_a, raised_a3) != 0) return -1;
-        hipLaunchKernelGGL((moe16_gate_up_kernel<3, 16>), dim3(m.topk * blocks + 1), dim3(6 * 64), lds_a, stream, m, blocks);
-    } else {
-        if (raise_lds(moe16_gate_up_kernel<1, 16>, lds_a, raised_a1) != 0) return -1;
-        hipLaunchKernelGGL((moe16_gate_up_kernel<1, 16>), dim3(m.topk * blocks + 1), dim3(2 * 64), lds_a, stream, m, blocks);
-    }
-    if (hipGetLastError() != hipSuccess) return -1;
-    if (raise_lds(moe16_down_sum_kernel<16>, lds_b, raised_b) != 0) return -1;
-    hipLaunchKernelGGL((moe16_down_sum_kernel<16>), dim3((m.hidden + ROWS16 - 1) / ROWS16), dim3(MOE16_MAX_TOPK * 64), lds_b,
-                       stream, m, out);
-    note_kernel("moe16_gate_up_kernel<%d,16> + moe16_down_sum_kernel<16>", parts);
-    return hipGetLastError() == hipSuccess ? 0 : -1;
+    const int md_a = meta_dwords(steps_a), md_b = meta_dwords(steps_routed);
+    int rc;
+    if (parts == 3)
+        rc = md_a == 4 ? launch_gate_up<3, 4>(m, blocks, lds_a, stream)
+           : md_a == 8 ? launch_gate_up<3, 8>(m, blocks, lds_a, stream) : launch_gate_up<3, 16>(m, blocks, lds_a, stream);
+    else
+        rc = md_a == 4 ? launch_gate_up<1, 4>(m, blocks, lds_a, stream)
+           : md_a == 8 ? launch_gate_up<1, 8>(m, blocks, lds_a, stream) : launch_gate_up<1, 16>(m, blocks, lds_a, stream);
+    if (rc != 0) return -1;
+    rc = md_b == 4 ? launch_down_sum<4>(m, out, lds_b, stream)
+       : md_b == 8 ? launch_down_sum<8>(m, out, lds_b, stream) : launch_down_sum<16>(m, out, lds_b, stream);
+    note_kernel("moe16_gate_up_kernel<%d,%d> + moe16_down_sum_kernel<%d>", parts, md_a, md_b);
+    return rc;
 }
 
 }  // namespace mi355

@@ -381,14 +381,14 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
 
     // ---------------------------------------------------------------- activations -> digit planes (all waves)
     auto build_image = [&]() {
-        build_q4_image<T, THREADS>(tid, ngrp, SG, zero_lds, img_lds, xm_lds, [&](int t, size_t column, float (&xv)[4]) {
+        build_q4_image<T, THREADS>(tid, ngrp, SG, zero_lds, img_lds, xm_lds, T, [&](int t, size_t column, float (&xv)[8]) {
             if (PRO == 2) {
 #pragma unroll
-                for (int k = 0; k < 4; ++k) xv[k] = det_gelu_tanh(act_gate[column + k]) * act_up[column + k];
+                for (int k = 0; k < 8; ++k) xv[k] = det_gelu_tanh(act_gate[column + k]) * act_up[column + k];
             } else {
                 const float *src = job.x + (size_t)t * job.x_stride + column;
 #pragma unroll
-                for (int k = 0; k < 4; ++k) xv[k] = src[k];
+                for (int k = 0; k < 8; ++k) xv[k] = src[k];
             }
         });
     };

@@ -76,10 +76,10 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch 
     stream.bind(job.vals, job.scales, job.biases, job.rows, has_rows ? row_base : 0, 0, has_rows ? stream.nstage : 0);
     if (has_rows) stream.start();
 
-    build_q4_image<T, THREADS>(tid, stream.ngrp, SG, zero_lds, img_lds, xm_lds, [&](int t, size_t column, float (&xv)[4]) {
+    build_q4_image<T, THREADS>(tid, stream.ngrp, SG, zero_lds, img_lds, xm_lds, T, [&](int t, size_t column, float (&xv)[8]) {
         const float *src = job.x + (size_t)t * job.x_stride + column;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) xv[k] = src[k];
+        for (int k = 0; k < 8; ++k) xv[k] = src[k];
     });
     __syncthreads();
     if (!has_rows) return;                           // no barrier below

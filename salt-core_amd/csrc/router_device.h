@@ -147,18 +147,21 @@ __device__ __forceinline__ void router_topk_block(const float *__restrict__ logi
 // call).  n_experts <= 256, every lane of the wave active.
 //
 // "Rank below topk" is a selection of the topk largest logits with ties going to the smaller index.  The wave finds
-// the topk-th largest value by a radix search over order-preserving integer keys (32 steps of compare + popcount),
-// takes everything above it and the lowest-indexed of the values equal to it.
+// the topk-th largest value by a radix search over order-preserving integer keys (a compare and a population count
+// per bit, from the top; the search ends as soon as exactly topk keys reach the candidate, which for distinct logits
+// happens after the few bits in which the topk-th and the next value differ), takes everything above it and the
+// lowest-indexed of the values equal to it.  Q = registers of keys per lane = ceil(n_experts / 64).
 constexpr int ROUTER_WAVE_MAX_EXPERTS = 256;
 
-__device__ __forceinline__ int router_select_wave(const float *__restrict__ logits,
-                                                  const float *__restrict__ per_expert_scale, int n_experts, int topk,
-                                                  int place) {
+template <int Q>
+__device__ __forceinline__ int router_select_wave_keys(const float *__restrict__ logits,
+                                                       const float *__restrict__ per_expert_scale, int n_experts, int topk,
+                                                       int place) {
     const int lane = threadIdx.x & 63;
-    uint32_t key[4];
+    uint32_t key[Q];
     bool finite = true;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int q = 0; q < Q; ++q) {
         const int e = q * 64 + lane;
         key[q] = 0u;                                                     // below every real key
         if (e < n_experts) {
@@ -176,18 +179,19 @@ __device__ __forceinline__ int router_select_wave(const float *__restrict__ logi
         const uint32_t candidate = threshold | (1u << bit);
         int reach = 0;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) reach += __popcll(__ballot(key[q] >= candidate));
+        for (int q = 0; q < Q; ++q) reach += __popcll(__ballot(key[q] >= candidate));
         if (reach >= topk) threshold = candidate;
+        if (reach == topk) break;                                        // these topk keys are the selection
     }
     int above = 0;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) above += __popcll(__ballot(key[q] > threshold));
+    for (int q = 0; q < Q; ++q) above += __popcll(__ballot(key[q] > threshold));
     const int ties_wanted = topk - above;                                // of the keys equal to the threshold
     const uint64_t below_me = (1ull << lane) - 1ull;
-    bool chosen[4];
+    bool chosen[Q];
     int ties_before = 0;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int q = 0; q < Q; ++q) {
         const uint64_t equal = __ballot(key[q] == threshold);
         const int my_tie = ties_before + __popcll(equal & below_me);
         chosen[q] = key[q] > threshold || (key[q] == threshold && my_tie < ties_wanted);
@@ -196,13 +200,21 @@ __device__ __forceinline__ int router_select_wave(const float *__restrict__ logi
     // position of every chosen expert in ascending-id order; the one at `place` answers
     int expert = -1, before = 0;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int q = 0; q < Q; ++q) {
         const uint64_t mask = __ballot(chosen[q]);
         const uint64_t hit = __ballot(chosen[q] && before + __popcll(mask & below_me) == place);
         if (hit != 0ull) expert = q * 64 + (int)__builtin_ctzll(hit);
         before += __popcll(mask);
     }
     return expert;
+}
+
+__device__ __forceinline__ int router_select_wave(const float *__restrict__ logits,
+                                                  const float *__restrict__ per_expert_scale, int n_experts, int topk,
+                                                  int place) {
+    if (n_experts <= 64) return router_select_wave_keys<1>(logits, per_expert_scale, n_experts, topk, place);
+    if (n_experts <= 128) return router_select_wave_keys<2>(logits, per_expert_scale, n_experts, topk, place);
+    return router_select_wave_keys<4>(logits, per_expert_scale, n_experts, topk, place);
 }
 
 }  // namespace mi355
