@@ -123,7 +123,18 @@ int salt_mi355_q4_jobs_activated_dev(const SaltMi355Q4Job *jobs, int njobs, int 
  * reference: the rows that touch it).  C a multiple of 64, at least 512, and
  * dword-aligned values take the streaming kernel; anything else runs on the
  * bit-exact kernels.  The reference has no counterpart (north star: "otherwise
- * within a stated max-abs/relative fp32 tolerance"). */
+ * within a stated max-abs/relative fp32 tolerance").
+ *
+ * Which bits a result has depends on the LAUNCH, not only on the matrix and
+ * the activation: the column count, the number of tokens and the number of
+ * 32-row blocks summed over all jobs of the call choose the kernel shape (rows
+ * per wave, parts a row is cut into, tokens per pass) and with it the order of
+ * the fp32 additions over a row's groups.  The same job alone, among 23 others,
+ * or at batch 3 instead of 4 may differ in its last bits, always inside the
+ * bound; the reference's identities "batch == per token" and "tiles == whole"
+ * (tools/test/gemma4-bit-identity-test.c:88-144) hold for the bit-exact
+ * kernels only.  For one and the same call the result is reproducible bit
+ * for bit, run after run: no atomics, no dependence on workgroup order. */
 int salt_mi355_q4_matvec_t_dev(const void *vals, const void *scales, const void *biases,
                                int R, int C, int B, const float *xs, float *ys, void *stream);
 int salt_mi355_q4_jobs_t_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int tokens, void *stream);

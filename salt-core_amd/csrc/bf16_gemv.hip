@@ -172,30 +172,16 @@ __global__ __launch_bounds__(64) void bf16_generic_kernel(Bf16Launch L) {
     }
 }
 
-int env_shape() {
-    static int shape = -1;
-    if (shape < 0) {
-        const char *v = getenv("SALT_MI355_BF16_SHAPE");
-        shape = v ? atoi(v) : 0;
-    }
-    return shape;
-}
-
 template <int NB, int STAGES, int WAVES>
 void launch_tiles(const Bf16Launch &L, hipStream_t stream) {
     const int tiles = (L.rows + ROWS - 1) / ROWS;
     bf16_tile_kernel<NB, STAGES, WAVES><<<dim3((tiles + WAVES - 1) / WAVES), dim3(WAVES * 64), 0, stream>>>(L);
 }
 
+// two stages, four waves per workgroup: 64 KB of LDS, eight waves per compute unit (measured best of
+// {2,1} {3,1} {2,2} {2,4} stages x waves on the 262144 x 2816 head)
 template <int NB>
-void launch_shape(const Bf16Launch &L, hipStream_t stream) {
-    switch (env_shape()) {
-    case 1: launch_tiles<NB, 2, 1>(L, stream); break;
-    case 2: launch_tiles<NB, 3, 1>(L, stream); break;
-    case 3: launch_tiles<NB, 2, 2>(L, stream); break;
-    default: launch_tiles<NB, 2, 4>(L, stream); break;
-    }
-}
+void launch_shape(const Bf16Launch &L, hipStream_t stream) { launch_tiles<NB, 2, 4>(L, stream); }
 
 }  // namespace
 

@@ -67,10 +67,5 @@ __device__ __forceinline__ void wait_vm() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-inline int env_int(const char *name, int fallback) {
-    const char *e = getenv(name);
-    return e ? atoi(e) : fallback;
-}
-
 }  // namespace
 }  // namespace mi355

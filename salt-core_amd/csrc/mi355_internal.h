@@ -120,6 +120,7 @@ int q4_dot16_launch(const Q4DotLaunch &launch, int waves, hipStream_t stream);
 // gelu_tanh(gate) * up in the prologue of the second); -1: the geometry is not served.
 // The whole step in two launches (moe_dot16.hip): gate + up + activation, then down + ordered weighted sum; `out`
 // receives the layer output, moe.expert_out (optional) the expert outputs.  -1: the geometry is not served.
+constexpr int MOE16_NOT_SERVED = 1;
 int moe16_step_launch(const MoeFuse &moe, float *out, hipStream_t stream);
 int q4_dot_moe_gate_up_launch(const MoeFuse &moe, hipStream_t stream);
 int q4_dot_moe_down_launch(const MoeFuse &moe, hipStream_t stream);
@@ -312,10 +313,9 @@ int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t exp
 
 // tolerance class (q4_dot.hip); -1 when the geometry is not served (more than 256 experts, widths the streaming
 // kernel does not take)
-int moe_decode_step_t_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_stride,
-                             const float *logits, const float *per_expert_scale, const float *x,
-                             int *selected, float *weights, float *expert_out, float *out,
-                             const MoeWorkspace &ws, hipStream_t stream);
+int moe_decode_step_t_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_stride, const float *logits,
+                             const float *per_expert_scale, const float *x, int *selected, float *weights,
+                             float *expert_out, float *out, const MoeWorkspace &ws, hipStream_t stream);
 
 int moe_activate_launch(const float *gate, const float *up, float *act, size_t n, hipStream_t stream);
 int moe_reduce_launch(const float *expert_out, const float *weights, int topk, int hidden, float *out,

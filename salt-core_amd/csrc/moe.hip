@@ -207,8 +207,9 @@ int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t exp
     return out ? moe_reduce_launch(eo, weights, g.topk, g.hidden, out, nullptr, stream) : 0;
 }
 
-// The same step on the tolerance-class matvec kernel: router top-k (bit-exact, in the prologue of the gate/up
-// launch), gate and up, gelu_tanh(gate) * up (in the prologue of the down launch), down, ordered weighted sum.
+// The same step on the tolerance-class matvec kernels: router top-k (bit-exact), gate and up, gelu_tanh(gate) * up,
+// down, ordered weighted sum.  Two launches where moe_dot16.hip serves the geometry (the activation rides in the
+// first, the weighted sum in the second), else three launches on the 32-row kernel with the sum on its own.
 int moe_decode_step_t_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_stride, const float *logits,
                              const float *per_expert_scale, const float *x, int *selected, float *weights,
                              float *expert_out, float *out, const MoeWorkspace &ws, hipStream_t stream) {
@@ -219,12 +220,12 @@ int moe_decode_step_t_launch(const MoeGeometry &g, const uint8_t *pool, size_t e
     m.selected = selected; m.weights = weights; m.status = ws.status;
     m.n_experts = g.n_experts; m.topk = g.topk; m.hidden = g.hidden; m.routed = g.routed;
     m.act = ws.act;
-    // two launches when the caller wants the layer output (the weighted sum rides in the down launch)
     if (out) {
         MoeFuse two = m;
         two.expert_out = expert_out;              // optional there
-        if (moe16_step_launch(two, out, stream) == 0) return 0;
-        (void)hipGetLastError();
+        const int served = moe16_step_launch(two, out, stream);
+        if (served == 0) return 0;
+        if (served != MOE16_NOT_SERVED) return -1;    // a launch failed: nothing to fall back on
     }
     if (q4_dot_moe_gate_up_launch(m, stream) != 0) return -1;
     if (q4_dot_moe_down_launch(m, stream) != 0) return -1;

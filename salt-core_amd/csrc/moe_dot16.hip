@@ -198,19 +198,20 @@ int meta_dwords(int steps) { return steps <= 2 ? 4 : steps <= 4 ? 8 : 16; }
 
 }  // namespace
 
-// -1: the geometry is not served (the caller takes another plan).
+// 0: both launches are enqueued.  MOE16_NOT_SERVED: this geometry is not served, nothing was launched (the caller
+// takes another plan).  -1: a launch failed.
 int moe16_step_launch(const MoeFuse &m, float *out, hipStream_t stream) {
     if (m.n_experts < 1 || m.n_experts > ROUTER_WAVE_MAX_EXPERTS || m.topk < 1 || m.topk > MOE16_MAX_TOPK ||
         m.topk > m.n_experts || !q4_dot_takes(m.hidden) || !q4_dot_takes(m.routed) || !out || !m.act)
-        return -1;
+        return MOE16_NOT_SERVED;
     const int steps_hidden = dot_steps(m.hidden >> 6), steps_routed = dot_steps(m.routed >> 6);
     // three parts per matrix where the row has at least three steps, else one
     const int parts = steps_hidden >= 3 ? 3 : 1;
     const int steps_a = (steps_hidden + parts - 1) / parts;
-    if (steps_a > 8 || steps_routed > 8) return -1;   // a lane's registers hold the scales of at most 32 groups
-    if (m.n_experts > 2 * parts * 64) return -1;      // the publishing workgroup runs the router with one thread per expert
+    if (steps_a > 8 || steps_routed > 8) return MOE16_NOT_SERVED;   // a lane's registers hold the scales of at most 32 groups
+    if (m.n_experts > 2 * parts * 64) return MOE16_NOT_SERVED;      // the publishing workgroup runs the router with one thread per expert
     const size_t lds_a = moe16_gate_up_lds(m.hidden, 2 * parts), lds_b = moe16_down_lds(m.routed);
-    if (lds_a > DOT_LDS_LIMIT || lds_b > DOT_LDS_LIMIT) return -1;
+    if (lds_a > DOT_LDS_LIMIT || lds_b > DOT_LDS_LIMIT) return MOE16_NOT_SERVED;
     const int blocks = (m.routed + ROWS16 - 1) / ROWS16;
     const int md_a = meta_dwords(steps_a), md_b = meta_dwords(steps_routed);
     int rc;

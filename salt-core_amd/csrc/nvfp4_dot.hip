@@ -183,15 +183,15 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_dot_kernel(const Fp4DotLaunch 
         // either strip (blocks past the row's end meet zero codes; they take whatever the clamped index yields)
         uint32_t sc[4];
         {
-            const int last = MD - 4;
+            // past the registers' end (a step that straddles the row's end: its real blocks are in the last dwords,
+            // the rest meet zero codes) each index is held back on its own
             const int at0 = 4 * (st - step_lo) + shift0, at1 = 4 * (st - step_lo) + shift1;
-            const int i0 = at0 < last ? at0 : last, i1 = at1 < last ? at1 : last;
 #pragma unroll
-            for (int d = 0; d < 4; ++d) sc[d] = scales_v[i0 + d];
-            if (i1 != i0) {                        // uniform
+            for (int d = 0; d < 4; ++d) sc[d] = scales_v[at0 + d < MD - 1 ? at0 + d : MD - 1];
+            if (at1 != at0) {                      // uniform
 #pragma unroll
                 for (int d = 0; d < 4; ++d) {
-                    const uint32_t other = scales_v[i1 + d];
+                    const uint32_t other = scales_v[at1 + d < MD - 1 ? at1 + d : MD - 1];
                     sc[d] = h ? other : sc[d];
                 }
             }
@@ -363,13 +363,10 @@ int launch_shape(const Fp4DotLaunch &L, hipStream_t stream) {
 bool fp4_dot_takes(int cols) { return cols >= DOT_MIN_COLS && cols <= DOT_MAX_COLS && (cols & 63) == 0; }
 
 DotShape fp4_dot_shape(int cols, int tokens, long long total_blocks) {
-    static const int want_ksplit = env_int("SALT_MI355_DOT_KSPLIT", 0);
     const int nstage = dot_steps(cols >> 6);
     int ksplit = 1;
     while (ksplit < 8 && total_blocks * ksplit < 1024 && nstage >= 2 * ksplit) ksplit *= 2;
     // a lane's registers hold the block scales of at most 32 groups of its strip
-    while ((nstage + ksplit - 1) / ksplit * STAGE_GROUPS > 32) ksplit *= 2;
-    if (want_ksplit == 1 || want_ksplit == 2 || want_ksplit == 4 || want_ksplit == 8) ksplit = want_ksplit;
     while ((nstage + ksplit - 1) / ksplit * STAGE_GROUPS > 32) ksplit *= 2;
     while (ksplit > 1 && ksplit > nstage) ksplit /= 2;
     // the activation codes are small: two workgroups of four waves fit every supported column count

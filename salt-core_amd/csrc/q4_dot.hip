@@ -282,15 +282,16 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
         {
             // register indexing by a wave-uniform index
             auto pick = [&](const MetaVec &m, int dword) -> uint32_t { return m[dword]; };
-            const int last = MD - 2;
+            // A step's four groups are two dwords; past the registers' end (a step that straddles the row's end: its
+            // real groups are in the last dword, the rest meet zero digits) each index is held back on its own
             const int at0 = 2 * (st - step_lo) + (shift0 >> 1), at1 = 2 * (st - step_lo) + (shift1 >> 1);
-            const int i0 = b * MD + (at0 < last ? at0 : last);
-            const int i1 = b * MD + (at1 < last ? at1 : last);
-            uint32_t s_lo = pick(scales_v, i0), s_hi = pick(scales_v, i0 + 1);
-            uint32_t b_lo = pick(biases_v, i0), b_hi = pick(biases_v, i0 + 1);
-            if (i1 != i0) {                        // uniform
-                const uint32_t s_lo1 = pick(scales_v, i1), s_hi1 = pick(scales_v, i1 + 1);
-                const uint32_t b_lo1 = pick(biases_v, i1), b_hi1 = pick(biases_v, i1 + 1);
+            const int lo0 = b * MD + (at0 < MD - 1 ? at0 : MD - 1), hi0 = b * MD + (at0 + 1 < MD - 1 ? at0 + 1 : MD - 1);
+            const int lo1 = b * MD + (at1 < MD - 1 ? at1 : MD - 1), hi1 = b * MD + (at1 + 1 < MD - 1 ? at1 + 1 : MD - 1);
+            uint32_t s_lo = pick(scales_v, lo0), s_hi = pick(scales_v, hi0);
+            uint32_t b_lo = pick(biases_v, lo0), b_hi = pick(biases_v, hi0);
+            if (at1 != at0) {                      // uniform
+                const uint32_t s_lo1 = pick(scales_v, lo1), s_hi1 = pick(scales_v, hi1);
+                const uint32_t b_lo1 = pick(biases_v, lo1), b_hi1 = pick(biases_v, hi1);
                 s_lo = h ? s_lo1 : s_lo; s_hi = h ? s_hi1 : s_hi;
                 b_lo = h ? b_lo1 : b_lo; b_hi = h ? b_hi1 : b_hi;
             }
@@ -516,17 +517,19 @@ int launch_shape(const Q4DotLaunch &L, hipStream_t stream) {
             return -1;
         raised = lds;
     }
-    note_kernel("q4_dot_kernel<%d,%d,%d,%d,%d,%d>", T, WAVES, STAGES, MD, PRO, NB);
+    note_kernel("q4_dot_kernel<%d,%d,%d,%d,%d,%d> ksplit %d", T, WAVES, STAGES, MD, PRO, NB, L.ksplit);
     // the router prologue has one more workgroup: the one that publishes its outputs
     hipLaunchKernelGGL((q4_dot_kernel<T, WAVES, STAGES, MD, PRO, NB>), dim3(L.total_wgs + (PRO == 1 ? 1 : 0)),
                        dim3(WAVES * 64), lds, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
-// (waves per workgroup, steps of LDS per wave); `resident` workgroups share a compute unit's LDS
+// (waves per workgroup, steps of LDS per wave); `resident` workgroups share a compute unit's LDS.  Every entry is
+// the first fit for some (columns, tokens, blocks): {4,2,2} rows of up to 3584 columns; {3,2,2} wider rows that are
+// not cut; {8,2,1} rows cut in 2, 4 or 8; {7,2,1} 8192 columns uncut; {6,2,1} 8192 columns cut in 2; {4,3,1} 8192
+// columns cut in 4; {4,2,1} several tokens of 8192 columns.
 struct Candidate { int waves, stages, resident; };
-constexpr Candidate CANDIDATES[] = {{4, 2, 2}, {3, 2, 2}, {8, 2, 1}, {7, 2, 1}, {6, 2, 1}, {5, 3, 1}, {4, 4, 1}, {4, 3, 1},
-                                    {4, 2, 1}, {2, 2, 2}};
+constexpr Candidate CANDIDATES[] = {{4, 2, 2}, {3, 2, 2}, {8, 2, 1}, {7, 2, 1}, {6, 2, 1}, {4, 3, 1}, {4, 2, 1}};
 
 }  // namespace
 
@@ -540,24 +543,19 @@ int q4_dot_tokens_per_pass(int cols) {
 }
 
 DotShape q4_dot_shape(int cols, int tokens, long long total_blocks) {
-    static const int want_waves = env_int("SALT_MI355_DOT_WAVES", 0), want_stages = env_int("SALT_MI355_DOT_STAGES", 0);
-    static const int want_ksplit = env_int("SALT_MI355_DOT_KSPLIT", 0);
     const int nstage = dot_steps(cols >> 6);
     // Few blocks: cut the rows along their columns until the launch has about a thousand waves
     int ksplit = 1;
     while (ksplit < 8 && total_blocks * ksplit < 1024 && nstage >= 2 * ksplit) ksplit *= 2;
-    if (want_ksplit == 1 || want_ksplit == 2 || want_ksplit == 4 || want_ksplit == 8) ksplit = want_ksplit;
     while (ksplit > 1 && ksplit > nstage) ksplit /= 2;
     // in order of preference; the first that fits the LDS beside the digit planes is taken
     for (const Candidate &c : CANDIDATES)
-        if ((want_waves == 0 || want_waves == c.waves) && (want_stages == 0 || want_stages == c.stages) &&
-            c.waves % ksplit == 0 && (ksplit == 1 || c.waves >= 4) &&
+        if (c.waves % ksplit == 0 && (ksplit == 1 || c.waves >= 4) &&
             dot_lds_bytes(cols, tokens, c.waves, c.stages) * c.resident <= DOT_LDS_LIMIT) {
             // Two blocks per wave (a stream twice as long) where the launch has plenty of blocks, the rows are not
-            // cut and a lane's registers hold both blocks' scales (rows of up to 4096 columns; four or six waves).
-            static const int want_nb = env_int("SALT_MI355_DOT_BLOCKS", 0);
-            const bool can = ksplit == 1 && nstage * STAGE_GROUPS <= 32 && (c.waves == 4 || c.waves == 6) && c.stages == 2;
-            const int nb = can && (want_nb == 2 || (want_nb == 0 && total_blocks >= 2048)) ? 2 : 1;
+            // cut and a lane's registers hold both blocks' scales (rows of up to 4096 columns, four waves).
+            const bool can = ksplit == 1 && nstage * STAGE_GROUPS <= 32 && c.waves == 4 && c.stages == 2;
+            const int nb = can && total_blocks >= 2048 ? 2 : 1;
             return DotShape{c.waves, c.stages, ksplit, nb};
         }
     return DotShape{4, 2, ksplit <= 4 ? ksplit : 4, 1};
@@ -576,15 +574,14 @@ int q4_dot_launch(const Q4DotLaunch &launch, const DotShape &shape, hipStream_t 
         if (md != 16 || shape.ksplit != 1 || shape.stages != 2) return -1;
 #define DOT_NB2(TT, WW) if (L.tokens == TT && shape.waves == WW) return launch_shape<TT, WW, 2, 16, 0, 2>(L, stream)
         DOT_NB2(1, 4); DOT_NB2(2, 4); DOT_NB2(3, 4); DOT_NB2(4, 4);
-        DOT_NB2(1, 6); DOT_NB2(2, 6); DOT_NB2(3, 6); DOT_NB2(4, 6);
 #undef DOT_NB2
         return -1;
     }
 #define DOT_CASE(TT, WW, SS) \
     if (L.tokens == TT && shape.waves == WW && shape.stages == SS) \
         return md == 16 ? launch_shape<TT, WW, SS, 16>(L, stream) : launch_shape<TT, WW, SS, 32>(L, stream)
-#define DOT_CASES(TT) DOT_CASE(TT, 8, 2); DOT_CASE(TT, 7, 2); DOT_CASE(TT, 6, 2); DOT_CASE(TT, 5, 3); DOT_CASE(TT, 4, 4); \
-                      DOT_CASE(TT, 4, 3); DOT_CASE(TT, 4, 2); DOT_CASE(TT, 3, 2); DOT_CASE(TT, 2, 2)
+#define DOT_CASES(TT) DOT_CASE(TT, 8, 2); DOT_CASE(TT, 7, 2); DOT_CASE(TT, 6, 2); DOT_CASE(TT, 4, 3); DOT_CASE(TT, 4, 2); \
+                      DOT_CASE(TT, 3, 2)
     DOT_CASES(1); DOT_CASES(2); DOT_CASES(3); DOT_CASES(4);
 #undef DOT_CASES
 #undef DOT_CASE

@@ -132,11 +132,10 @@ int launch16(const Q4DotLaunch &L, hipStream_t stream) {
 // Waves per workgroup of the sixteen-row shape for this width and token count, or 0 when it should not be used:
 // two workgroups per compute unit where the digit planes leave room, else one of twelve waves.
 int q4_dot16_waves(int cols, int tokens, long long total_blocks32) {
-    static const int want = env_int("SALT_MI355_DOT16", -1);           // 0 forbids the shape, 8 / 12 force it
-    if (want == 0 || tokens > 4 || !q4_dot_takes(cols)) return 0;
-    if (want != 8 && want != 12 && total_blocks32 < 2048) return 0;     // few blocks: the 32-row kernel cuts rows instead
-    if ((want == -1 || want == 8) && 2 * dot16_lds_bytes(cols, tokens, 8) <= DOT_LDS_LIMIT) return 8;
-    if ((want == -1 || want == 12) && dot16_lds_bytes(cols, tokens, 12) <= DOT_LDS_LIMIT) return 12;
+    if (tokens > 4 || !q4_dot_takes(cols)) return 0;
+    if (total_blocks32 < 2048) return 0;                                // few blocks: the 32-row kernel cuts rows instead
+    if (2 * dot16_lds_bytes(cols, tokens, 8) <= DOT_LDS_LIMIT) return 8;
+    if (dot16_lds_bytes(cols, tokens, 12) <= DOT_LDS_LIMIT) return 12;
     return 0;
 }
 

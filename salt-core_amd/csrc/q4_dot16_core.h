@@ -52,18 +52,22 @@ struct Dot16Stream {
     int ngrp, nstage, SG, whole_steps;
     int step_lo, step_hi;
     uint32_t row_bytes;
-    uint8_t *my_lds;                             // WAVE16_LDS bytes
+    uint8_t *my_lds;                             // WAVE16_LDS bytes: the two slots steps alternate between ...
+    uint8_t *slot_lds[2];                        // ... unless the caller places them elsewhere (place_slots)
     // per-lane geometry
     int lane, n, kq, my_strip;
     int src_rowi[LOADS16];
     uint32_t src_col[LOADS16], src_off[LOADS16], rd_off[STAGE_GROUPS];
     int meta_groups, window0, window1, shift0, shift1;
     MetaRegs<MD> scales_r, biases_r;
+    typedef uint32_t MetaVec __attribute__((ext_vector_type(MD)));
+    MetaVec scales_v, biases_v;                  // the same values as one indexable vector, valid after settle()
 
     __device__ __forceinline__ void setup(int lane_, int cols, uint8_t *lds_of_wave) {
         lane = lane_;
         n = lane & 15; kq = lane >> 4; my_strip = kq & 1;
         my_lds = lds_of_wave;
+        slot_lds[0] = lds_of_wave; slot_lds[1] = lds_of_wave + STEP16_BYTES;
         ngrp = cols >> 6;
         nstage = dot_steps(ngrp);
         SG = nstage * STAGE_GROUPS;              // groups of strip 0; strip 1 holds the remaining ngrp - SG
@@ -105,7 +109,7 @@ struct Dot16Stream {
     }
 
     __device__ __forceinline__ void issue_step(int st, int slot) {
-        uint8_t *const stage = my_lds + slot * STEP16_BYTES;
+        uint8_t *const stage = slot_lds[slot];
         const uint8_t *const block_vals = vals + (size_t)row_base * row_bytes;
         const uint32_t advance = (uint32_t)st * (STAGE_GROUPS * 32);
         if (rows_here == ROWS16 && st < whole_steps) {
@@ -127,9 +131,12 @@ struct Dot16Stream {
         }
     }
 
-    // Scales, biases and the first two steps go out: none of them depends on the activations, so the caller builds
-    // the digit planes while they are on their way.
-    __device__ __forceinline__ void start() {
+    __device__ __forceinline__ void place_slots(uint8_t *even_steps, uint8_t *odd_steps) {
+        slot_lds[0] = even_steps; slot_lds[1] = odd_steps;
+    }
+
+    // The scales and biases of the wave's rows go out.
+    __device__ __forceinline__ void issue_meta() {
         const int row = n < rows_here ? n : rows_here - 1;
         const size_t at = ((size_t)(row_base + row) * ngrp + (my_strip ? window1 : window0)) * 2;
         const uint8_t *bias_src = biases ? biases : scales;           // the load happens either way; its result is dropped
@@ -139,6 +146,12 @@ struct Dot16Stream {
             scales_r.q[q] = load_meta16(scales + at + 16 * piece);
             biases_r.q[q] = load_meta16(bias_src + at + 16 * piece);
         }
+    }
+
+    // Scales, biases and the first two steps go out: none of them depends on the activations, so the caller builds
+    // the digit planes while they are on their way.
+    __device__ __forceinline__ void start() {
+        issue_meta();
 #pragma unroll
         for (int g = 0; g < 2; ++g)
             if (step_lo + g < step_hi) issue_step(step_lo + g, g);
@@ -148,9 +161,13 @@ struct Dot16Stream {
     // lane (n, mq) receives row n's sum over the wave's steps of strip mq % 2 for token mq / 2 of pair s.
     template <int SETS>
     __device__ __forceinline__ void run(const Dot16Operand (&operand)[SETS], float (&acc)[SETS]) {
-        typedef uint32_t MetaVec __attribute__((ext_vector_type(MD)));
-        MetaVec scales_v, biases_v;
-        // the scales and biases, the only loads that return to registers, are waited for with everything in flight
+        settle();
+        walk(operand, acc);
+    }
+
+    // Waits for the scales and biases, the only loads that return to registers, together with everything else the
+    // wave has in flight.
+    __device__ __forceinline__ void settle() {
 #pragma unroll
         for (int q = 0; q < MD / 4; ++q) {
             wait_meta(scales_r.q[q]);
@@ -174,6 +191,11 @@ struct Dot16Stream {
                 biases_v[i] = odd ? b_moved : biases_v[i];
             }
         }
+    }
+
+    // The walk over the wave's steps, after settle(); the first two steps have been issued.
+    template <int SETS>
+    __device__ __forceinline__ void walk(const Dot16Operand (&operand)[SETS], float (&acc)[SETS]) {
         const bool no_bias = biases == nullptr;
         const int total_steps = step_hi - step_lo;
         struct StepWeights { u32x4 group[STAGE_GROUPS]; };
@@ -183,12 +205,14 @@ struct Dot16Stream {
             // index per strip (groups past the row's end meet zero digits; they take whatever the clamped index yields)
             float scale[STAGE_GROUPS], bias[STAGE_GROUPS];
             {
-                const int last = MD - 2;
+                // A step's four groups are two dwords; past the registers' end (a step that straddles the row's end:
+                // its real groups are in the last dword, the rest meet zero digits) each index is held back on its own
                 const int at0 = 2 * (st - step_lo) + (shift0 >> 1), at1 = 2 * (st - step_lo) + (shift1 >> 1);
-                const int i0 = at0 < last ? at0 : last, i1 = at1 < last ? at1 : last;
-                uint32_t s_lo = scales_v[i0], s_hi = scales_v[i0 + 1], b_lo = biases_v[i0], b_hi = biases_v[i0 + 1];
-                if (i1 != i0) {                    // uniform
-                    const uint32_t s_lo1 = scales_v[i1], s_hi1 = scales_v[i1 + 1], b_lo1 = biases_v[i1], b_hi1 = biases_v[i1 + 1];
+                const int lo0 = at0 < MD - 1 ? at0 : MD - 1, hi0 = at0 + 1 < MD - 1 ? at0 + 1 : MD - 1;
+                const int lo1 = at1 < MD - 1 ? at1 : MD - 1, hi1 = at1 + 1 < MD - 1 ? at1 + 1 : MD - 1;
+                uint32_t s_lo = scales_v[lo0], s_hi = scales_v[hi0], b_lo = biases_v[lo0], b_hi = biases_v[hi0];
+                if (at1 != at0) {                  // uniform
+                    const uint32_t s_lo1 = scales_v[lo1], s_hi1 = scales_v[hi1], b_lo1 = biases_v[lo1], b_hi1 = biases_v[hi1];
                     s_lo = my_strip ? s_lo1 : s_lo; s_hi = my_strip ? s_hi1 : s_hi;
                     b_lo = my_strip ? b_lo1 : b_lo; b_hi = my_strip ? b_hi1 : b_hi;
                 }
@@ -251,7 +275,7 @@ struct Dot16Stream {
                 if (g >= total_steps) return false;
                 if (g + 1 < total_steps) wait_vm<LOADS16>(); else wait_vm<0>();
                 StepWeights w;
-                const uint8_t *stage = my_lds + r * STEP16_BYTES;
+                const uint8_t *stage = slot_lds[r];
 #pragma unroll
                 for (int u = 0; u < STAGE_GROUPS; ++u) w.group[u] = *(const u32x4 *)(stage + rd_off[u]);
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // the reads have returned before the slot is refilled

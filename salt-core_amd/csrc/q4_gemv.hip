@@ -551,22 +551,14 @@ __global__ __launch_bounds__(256) void q4_generic_kernel(const Q4Launch L) {
     }
 }
 
-// Launches of at most this many tiles use the wide-step variant (tuning: SALT_MI355_Q4_WIDE_TILES).
-int env_wide_limit() {
-    static int cached = -1;
-    if (cached < 0) {
-        const char *e = getenv("SALT_MI355_Q4_WIDE_TILES");
-        cached = e ? atoi(e) : 256;
-        if (cached < 0) cached = 0;
-    }
-    return cached;
-}
+// Launches of at most this many tiles (one per compute unit) use the wide-step variant and two chains per lane.
+constexpr int WIDE_TILE_LIMIT = 256;
 
 template <int S>
 int launch_tiles(const Q4Launch &L, hipStream_t stream) {
     const dim3 grid(L.total_tiles), block((32 / S) * 64);
     // One token with few tiles: a workgroup has its compute unit to itself and stages twice as much per step.
-    if (L.tokens == 1 && S <= 4 && L.total_tiles <= env_wide_limit()) {
+    if (L.tokens == 1 && S <= 4 && L.total_tiles <= WIDE_TILE_LIMIT) {
         note_kernel("q4_tile_kernel<%d,1,32,0>", S);
         hipLaunchKernelGGL((q4_tile_kernel<S, 1, 32>), grid, block, 0, stream, L);
         return hipGetLastError() == hipSuccess ? 0 : -1;
@@ -580,16 +572,6 @@ int launch_tiles(const Q4Launch &L, hipStream_t stream) {
         default: return -1;
     }
     return hipGetLastError() == hipSuccess ? 0 : -1;
-}
-
-int env_chains() {
-    static int cached = -1;
-    if (cached < 0) {
-        const char *e = getenv("SALT_MI355_Q4_CHAINS");
-        const int v = e ? atoi(e) : 0;
-        cached = (v == 8 || v == 4 || v == 2) ? v : 0;
-    }
-    return cached;
 }
 
 }  // namespace
@@ -626,9 +608,9 @@ int q4_moe_gate_up_launch(const Q4Launch &launch, hipStream_t stream) {
     const dim3 grid(L.total_tiles + 1);                         // the extra workgroup publishes the router's outputs
     // measured at 176 tiles (eight experts of 704 rows): 1024-column steps 29.4 us per decode step, 512-column steps 29.1,
     // four chains per lane 30.4 and 33.4; the wide step is kept for launches that leave half the compute units idle
-    if (L.total_tiles <= env_wide_limit() / 2)
+    if (L.total_tiles <= WIDE_TILE_LIMIT / 2)
         hipLaunchKernelGGL((q4_tile_kernel<2, 1, 32, 1>), grid, dim3(1024), 0, stream, L);
-    else if (L.total_tiles <= env_wide_limit())
+    else if (L.total_tiles <= WIDE_TILE_LIMIT)
         hipLaunchKernelGGL((q4_tile_kernel<2, 1, 16, 1>), grid, dim3(1024), 0, stream, L);
     else
         hipLaunchKernelGGL((q4_tile_kernel<4, 1, 16, 1>), grid, dim3(512), 0, stream, L);
@@ -646,7 +628,7 @@ int q4_moe_down_launch(const Q4Launch &launch, hipStream_t stream) {
     const dim3 grid(L.total_tiles);
     // measured at 352 tiles (eight experts of 2816 rows): two chains per lane 31.4 us per decode step, four 29.4,
     // eight 31.4, wide steps 32.7 and 34.5
-    if (L.total_tiles <= env_wide_limit())
+    if (L.total_tiles <= WIDE_TILE_LIMIT)
         hipLaunchKernelGGL((q4_tile_kernel<2, 1, 32, 2>), grid, dim3(1024), 0, stream, L);
     else
         hipLaunchKernelGGL((q4_tile_kernel<4, 1, 16, 2>), grid, dim3(512), 0, stream, L);
@@ -656,7 +638,7 @@ int q4_moe_down_launch(const Q4Launch &launch, hipStream_t stream) {
 int q4_activated_launch(const Q4Launch &L, hipStream_t stream) {
     if (L.total_tiles < 1 || L.tokens != 1 || L.cols < 64 || (L.cols & 63) || L.cols > MOE_FUSE_MAX_ROUTED) return -1;
     const dim3 grid(L.total_tiles);
-    if (L.total_tiles <= env_wide_limit())
+    if (L.total_tiles <= WIDE_TILE_LIMIT)
         hipLaunchKernelGGL((q4_tile_kernel<2, 1, 32, 3>), grid, dim3(1024), 0, stream, L);
     else
         hipLaunchKernelGGL((q4_tile_kernel<4, 1, 16, 3>), grid, dim3(512), 0, stream, L);
@@ -665,12 +647,12 @@ int q4_activated_launch(const Q4Launch &L, hipStream_t stream) {
 
 int q4_launch(const Q4Launch &L, int chains_per_lane, hipStream_t stream) {
     if (L.total_tiles < 1 || L.tokens < 1 || L.tokens > 4 || L.cols < 64 || (L.cols & 63)) return -1;
-    int S = chains_per_lane ? chains_per_lane : env_chains();
+    int S = chains_per_lane;
     if (S == 0) {
         // Up to one tile per compute unit, sixteen waves per tile (two chains per lane) hide more of the LDS and
         // scalar-load latency; beyond that four chains per lane win (one token, 2816 columns: 12.4 against 15.5 us at
         // 256 tiles, 20.7 against 15.2 at 320, 23.3 against 17.6 at 512; eight chains per lane never do).
-        S = L.total_tiles > env_wide_limit() ? 4 : 2;
+        S = L.total_tiles > WIDE_TILE_LIMIT ? 4 : 2;
     }
     switch (S) {
         case 8: return launch_tiles<8>(L, stream);

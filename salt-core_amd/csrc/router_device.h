@@ -156,7 +156,7 @@ constexpr int ROUTER_WAVE_MAX_EXPERTS = 256;
 template <int Q>
 __device__ __forceinline__ int router_select_wave_keys(const float *__restrict__ logits,
                                                        const float *__restrict__ per_expert_scale, int n_experts, int topk,
-                                                       int place) {
+                                                       int place, int second_place, int &second_expert) {
     const int lane = threadIdx.x & 63;
     uint32_t key[Q];
     bool finite = true;
@@ -197,24 +197,38 @@ __device__ __forceinline__ int router_select_wave_keys(const float *__restrict__
         chosen[q] = key[q] > threshold || (key[q] == threshold && my_tie < ties_wanted);
         ties_before += __popcll(equal);
     }
-    // position of every chosen expert in ascending-id order; the one at `place` answers
+    // position of every chosen expert in ascending-id order; the ones at `place` and `second_place` answer
     int expert = -1, before = 0;
+    second_expert = -1;
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
         const uint64_t mask = __ballot(chosen[q]);
-        const uint64_t hit = __ballot(chosen[q] && before + __popcll(mask & below_me) == place);
+        const int position = before + __popcll(mask & below_me);
+        const uint64_t hit = __ballot(chosen[q] && position == place);
         if (hit != 0ull) expert = q * 64 + (int)__builtin_ctzll(hit);
+        const uint64_t second_hit = __ballot(chosen[q] && position == second_place);
+        if (second_hit != 0ull) second_expert = q * 64 + (int)__builtin_ctzll(second_hit);
         before += __popcll(mask);
     }
     return expert;
 }
 
+// Experts at two positions of the selection at once (second_place < 0: none asked for).
+__device__ __forceinline__ int router_select_wave_pair(const float *__restrict__ logits,
+                                                       const float *__restrict__ per_expert_scale, int n_experts, int topk,
+                                                       int place, int second_place, int &second_expert) {
+    if (n_experts <= 64)
+        return router_select_wave_keys<1>(logits, per_expert_scale, n_experts, topk, place, second_place, second_expert);
+    if (n_experts <= 128)
+        return router_select_wave_keys<2>(logits, per_expert_scale, n_experts, topk, place, second_place, second_expert);
+    return router_select_wave_keys<4>(logits, per_expert_scale, n_experts, topk, place, second_place, second_expert);
+}
+
 __device__ __forceinline__ int router_select_wave(const float *__restrict__ logits,
                                                   const float *__restrict__ per_expert_scale, int n_experts, int topk,
                                                   int place) {
-    if (n_experts <= 64) return router_select_wave_keys<1>(logits, per_expert_scale, n_experts, topk, place);
-    if (n_experts <= 128) return router_select_wave_keys<2>(logits, per_expert_scale, n_experts, topk, place);
-    return router_select_wave_keys<4>(logits, per_expert_scale, n_experts, topk, place);
+    int unused;
+    return router_select_wave_pair(logits, per_expert_scale, n_experts, topk, place, -1, unused);
 }
 
 }  // namespace mi355

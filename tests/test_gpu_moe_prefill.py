@@ -18,6 +18,7 @@ import numpy as np
 import pytest
 
 from golden import cases
+from moe_bounds import group_term_magnitudes as term_magnitudes
 from oracle_lib import ExpertGeometry, host_threads, ptr
 
 pytestmark = pytest.mark.gpu
@@ -29,32 +30,6 @@ def expected_grouping(sel, E):
     flat = sel.ravel()
     order = np.argsort(flat, kind="stable").astype(np.int32)
     return np.bincount(flat, minlength=E).astype(np.int32), order
-
-
-def dequantised(pool, e, p, H, F):
-    """Expert e's projection p (0 gate, 1 up, 2 down) as float64 [rows][cols]."""
-    proj, n = synth.expert_proj_bytes(H, F), H * F
-    at = (e * 3 + p) * proj
-    vals = pool[at:at + n // 2].view(np.uint32)
-    sc = synth.bf16_bits_to_f32(pool[at + n // 2:at + n // 2 + n // 32].view(np.uint16)).astype(np.float64)
-    bi = synth.bf16_bits_to_f32(pool[at + n // 2 + n // 32:at + proj].view(np.uint16)).astype(np.float64)
-    q = ((vals[:, None] >> (4 * np.arange(8, dtype=np.uint32))) & 15).reshape(-1).astype(np.float64)
-    w = q * np.repeat(sc, 64) + np.repeat(bi, 64)
-    return w.reshape((F, H) if p < 2 else (H, F))
-
-
-def term_magnitudes(pool, sel, w, xs, H, F):
-    """M[token][d] of the module docstring, in float64."""
-    T, K = sel.shape
-    M = np.zeros((T, H))
-    x64 = xs.astype(np.float64)
-    for e in np.unique(sel):
-        tok, rank = np.nonzero(sel == e)
-        gate, up, down = (dequantised(pool, int(e), p, H, F) for p in range(3))
-        g = x64[tok] @ gate.T
-        h = 0.5 * g * (1.0 + np.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3))) * (x64[tok] @ up.T)
-        M[tok] += np.abs(w[tok, rank].astype(np.float64))[:, None] * (np.abs(h) @ np.abs(down).T)
-    return M
 
 
 def check_values(got, want, magnitudes=None):

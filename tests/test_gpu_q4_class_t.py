@@ -14,50 +14,11 @@ import numpy as np
 import pytest
 
 from golden import cases
-from oracle_lib import host_threads, ptr
+from oracle_lib import ptr
+from q4_bounds import check, magnitude_sums, reference
 
 pytestmark = pytest.mark.gpu
 synth = cases.synth
-
-
-def reference(oracle, vals, scales, biases, R, Cc, xs):
-    ys = np.zeros((xs.shape[0], R), np.float32)
-    for t in range(xs.shape[0]):
-        assert oracle.orc_q4_matvec_threads(ptr(vals), ptr(scales), ptr(biases), R, Cc, ptr(xs[t]), ptr(ys[t]),
-                                            host_threads()) == 0
-    return ys
-
-
-def magnitude_sums(vals, scales, biases, R, Cc, xs):
-    """(sum_c |w x|, sum_c (|q s| + 16|s| + |b|) |x|) per (token, row), in float64, row blocks to bound memory."""
-    wx = np.zeros((xs.shape[0], R))
-    terms = np.zeros((xs.shape[0], R))
-    ax = np.abs(xs.astype(np.float64))
-    words = vals.reshape(R, Cc // 8)
-    sc = synth.bf16_bits_to_f32(scales).reshape(R, Cc // 64).astype(np.float64)
-    bi = np.zeros((R, Cc // 64)) if biases is None else synth.bf16_bits_to_f32(biases).reshape(R, Cc // 64).astype(np.float64)
-    for r0 in range(0, R, 1024):
-        r1 = min(R, r0 + 1024)
-        q = ((words[r0:r1, :, None] >> (4 * np.arange(8, dtype=np.uint32))) & 15).reshape(r1 - r0, Cc).astype(np.float64)
-        s = np.repeat(sc[r0:r1], 64, axis=1)
-        b = np.repeat(bi[r0:r1], 64, axis=1)
-        wx[:, r0:r1] = ax @ np.abs(q * s + b).T
-        terms[:, r0:r1] = ax @ (np.abs(q * s) + 16 * np.abs(s) + np.abs(b)).T
-    return wx, terms
-
-
-def check(got, want, vals, scales, biases, R, Cc, xs, outlier_tokens=()):
-    wx, terms = magnitude_sums(vals, scales, biases, R, Cc, xs)
-    err = np.abs(got.astype(np.float64) - want)
-    bound = 2.0 ** -20 * terms + 1e-6
-    assert np.isfinite(got).all()
-    print("max err / bound", float((err / bound).max()), flush=True)
-    assert (err <= bound).all(), float((err / bound).max())
-    plain = 2.0 ** -18 * wx + 1e-6
-    keep = [t for t in range(xs.shape[0]) if t not in outlier_tokens]
-    if keep:
-        print("max err / plain bound", float((err[keep] / plain[keep]).max()), flush=True)
-        assert (err[keep] <= plain[keep]).all()
 
 
 @pytest.mark.parametrize("R,Cc,B", [
@@ -180,3 +141,82 @@ def test_rejections(pkg):
     assert lib.salt_mi355_q4_matvec_t_dev(None, buf.ptr, None, 8, 512, 1, buf.ptr, buf.ptr, None) == -1
     assert lib.salt_mi355_q4_matvec_t_dev(buf.ptr, buf.ptr, None, 0, 512, 1, buf.ptr, buf.ptr, None) == -1
     assert lib.salt_mi355_q4_jobs_t_dev(None, 1, 512, 1, None) == -1
+
+
+def run_jobs(pkg, Cc, tokens, rows, weights, seed):
+    """One salt_mi355_q4_jobs_t_dev launch of len(rows) jobs; job j reads weights[j % len(weights)] (tensors of at
+    least rows[j] rows) and its own activations.  Returns (kernel name, [(tensor, rows, xs, ys)])."""
+    lib = pkg.lib.init()
+    dev = [tuple(pkg.lib.DeviceBuffer.from_host(a) for a in t) for t in weights]
+    xs = [synth.activations(Cc, tokens, seed + j) for j in range(len(rows))]
+    dxs = [pkg.lib.DeviceBuffer.from_host(x) for x in xs]
+    dys = [pkg.lib.DeviceBuffer(tokens * R * 4, fill=0xFF) for R in rows]
+    jobs = (pkg.lib.Q4Job * len(rows))()
+    for j, R in enumerate(rows):
+        dv, ds, db = dev[j % len(dev)]
+        jobs[j] = pkg.lib.Q4Job(dv.ptr, ds.ptr, db.ptr, dxs[j].ptr, dys[j].ptr, R)
+    stream = lib.salt_mi355_stream()
+    pkg.lib.check(lib.salt_mi355_q4_jobs_t_dev(jobs, len(rows), Cc, tokens, stream), "q4_jobs_t_dev")
+    pkg.lib.check(lib.salt_mi355_stream_sync(stream), "sync")
+    name = lib.salt_mi355_last_kernel().decode()
+    return name, [(weights[j % len(weights)], R, xs[j], dys[j].to_host(np.float32).reshape(tokens, R))
+                  for j, R in enumerate(rows)]
+
+
+# (columns, tokens, rows per job, jobs) -> the launch shape it must take.  Between them the cases reach every entry
+# of the 32-row kernel's candidate list, every cut of the rows (1, 2, 4, 8 parts), both register widths, two blocks
+# per wave, and the sixteen-row kernel at eight and at twelve waves.
+SHAPE_CASES = [
+    (2816, 1, 2816, 12, "q4_dot_kernel<1,4,2,16,0,1> ksplit 1"),
+    (2816, 1, 2816, 6, "q4_dot_kernel<1,4,2,16,0,1> ksplit 2"),
+    (2816, 1, 2816, 1, "q4_dot_kernel<1,4,2,16,0,1> ksplit 4"),
+    (4096, 1, 4096, 8, "q4_dot_kernel<1,3,2,16,0,1> ksplit 1"),
+    (4096, 1, 4096, 1, "q4_dot_kernel<1,8,2,16,0,1> ksplit 8"),
+    (8192, 1, 2816, 12, "q4_dot_kernel<1,7,2,32,0,1> ksplit 1"),
+    (8192, 1, 2816, 6, "q4_dot_kernel<1,6,2,16,0,1> ksplit 2"),
+    (8192, 1, 2816, 3, "q4_dot_kernel<1,4,3,16,0,1> ksplit 4"),
+    (8192, 2, 2816, 12, "q4_dot_kernel<2,4,2,32,0,1> ksplit 1"),
+    (4096, 4, 4096, 16, "q4_dot_kernel<4,4,2,16,0,2> ksplit 1"),
+    (2816, 1, 2816, 24, "q4_dot16_kernel<1,8,16>"),
+    (2816, 2, 2816, 24, "q4_dot16_kernel<2,12,16>"),
+    (8192, 1, 2816, 24, "q4_dot16_kernel<1,12,32>"),
+    (2112, 1, 2816, 2, "q4_dot_kernel<1,4,2,16,0,1> ksplit 4"),     # 33 groups: a step that straddles the row's end
+    (6272, 3, 96, 1, None),                                          # 98 groups, three tokens, rows cut in 8
+]
+
+
+@pytest.mark.parametrize("Cc,tokens,R,njobs,kernel", SHAPE_CASES)
+def test_every_launch_shape(pkg, oracle, Cc, tokens, R, njobs, kernel):
+    print(f"class T shape C={Cc} tokens={tokens} R={R} jobs={njobs}", flush=True)
+    weights = [synth.q4_tensor(R, Cc, 900 + k) for k in range(min(njobs, 2))]
+    name, results = run_jobs(pkg, Cc, tokens, [R] * njobs, weights, 950)
+    print("  ", name, flush=True)
+    if kernel is not None:
+        assert name == kernel
+    for j in sorted({0, njobs // 2, njobs - 1}):
+        (vals, scales, biases), rows, xs, got = results[j]
+        check(got, reference(oracle, vals, scales, biases, rows, Cc, xs), vals, scales, biases, rows, Cc, xs)
+
+
+def test_the_shape_cases_cover_the_candidate_list():
+    reached = {k for *_, k in SHAPE_CASES if k}
+    for waves, stages in ((4, 2), (3, 2), (8, 2), (7, 2), (6, 2), (4, 3)):
+        assert any(k.startswith("q4_dot_kernel<") and k.split("<")[1].split(",")[1:3] == [str(waves), str(stages)]
+                   for k in reached), (waves, stages)
+    for cut in (1, 2, 4, 8):
+        assert any(k.endswith(f"ksplit {cut}") for k in reached)
+    assert any(",32,0,1>" in k for k in reached) and any(",0,2>" in k for k in reached)
+
+
+def test_same_launch_gives_the_same_bits(pkg):
+    """The bits of a tolerance-class result depend on the launch (columns, tokens, number of blocks: they choose the
+    kernel shape and with it the order of the fp32 sums) but not on the run: no atomics, no order between
+    workgroups.  The same launch, repeated with other launches in between, returns identical bits."""
+    for Cc, tokens, R, njobs in ((2816, 1, 2816, 24), (4096, 1, 4096, 1), (8192, 2, 704, 5), (2816, 3, 16384, 1)):
+        weights = [synth.q4_tensor(R, Cc, 31)]
+        first = run_jobs(pkg, Cc, tokens, [R] * njobs, weights, 40)
+        run_jobs(pkg, 1024, 2, [100, 33], [synth.q4_tensor(100, 1024, 32)], 41)
+        again = run_jobs(pkg, Cc, tokens, [R] * njobs, weights, 40)
+        assert first[0] == again[0]
+        for (_, _, _, a), (_, _, _, b) in zip(first[1], again[1]):
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))

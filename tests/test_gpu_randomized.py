@@ -8,6 +8,7 @@ import pytest
 
 from golden import cases
 from oracle_lib import ExpertGeometry, bits, host_threads, ptr
+from q4_bounds import check as check_class_t
 
 pytestmark = pytest.mark.gpu
 synth = cases.synth
@@ -126,3 +127,49 @@ def test_random_moe_decode_steps(gpu, oracle):
             assert st == 0 and np.array_equal(sel, osel) and np.array_equal(bits(w), bits(ow))
             assert np.array_equal(bits(eo), bits(oeo)) and np.array_equal(bits(y), bits(oy))
         del layer
+
+
+@pytest.mark.parametrize("stream_seed", [11, 12])
+def test_random_tolerance_class_launches(gpu, oracle, stream_seed):
+    """salt_mi355_q4_jobs_t_dev at random shapes: 512..8192 columns, 1..9 tokens, 1..40 jobs of ragged row counts,
+    tensors at 0 / 4 / 8 bytes past a multiple of 16, with and without biases; every sampled job inside the stated
+    bound against the CPU checker."""
+    lib = gpu.init()
+    rng = np.random.default_rng(stream_seed)
+    kernels = set()
+    for case in range(40):
+        Cc = 64 * int(rng.integers(8, 129))
+        tokens = int(rng.integers(1, 10))
+        njobs = int(rng.choice([1, 1, 2, 3, 7, 17, 40]))
+        budget = 6_000_000 // Cc                                  # rows in the launch: bounds the checker's time
+        rows = [int(rng.integers(1, max(2, min(3000, 2 * budget // njobs)))) for _ in range(njobs)]
+        seed = int(rng.integers(1, 1 << 30))
+        offset = int(rng.choice([0, 4, 8]))
+        with_bias = bool(rng.random() < 0.8)
+        top = max(rows)
+        tensors = [synth.q4_tensor(top, Cc, seed + k) for k in range(min(njobs, 3))]
+        dev = []
+        for vals, scales, biases in tensors:
+            dv = gpu.DeviceBuffer(vals.nbytes + offset + 16, fill=0)
+            dv.upload(vals, offset)
+            dev.append((dv, gpu.DeviceBuffer.from_host(scales), gpu.DeviceBuffer.from_host(biases)))
+        xs = [synth.activations(Cc, tokens, seed + 10 + j) for j in range(njobs)]
+        dxs = [gpu.DeviceBuffer.from_host(x) for x in xs]
+        dys = [gpu.DeviceBuffer(tokens * R * 4, fill=0xFF) for R in rows]
+        jobs = (gpu.Q4Job * njobs)()
+        for j, R in enumerate(rows):
+            dv, ds, db = dev[j % len(dev)]
+            jobs[j] = gpu.Q4Job(dv.at(offset), ds.ptr, db.ptr if with_bias else None, dxs[j].ptr, dys[j].ptr, R)
+        print("class T", Cc, tokens, njobs, sum(rows), offset, with_bias, seed, flush=True)
+        stream = lib.salt_mi355_stream()
+        gpu.check(lib.salt_mi355_q4_jobs_t_dev(jobs, njobs, Cc, tokens, stream), "q4_jobs_t_dev")
+        gpu.check(lib.salt_mi355_stream_sync(stream), "sync")
+        kernels.add(lib.salt_mi355_last_kernel().decode())
+        for j in sorted({0, njobs // 2, njobs - 1}):
+            vals, scales, biases = tensors[j % len(tensors)]
+            R = rows[j]
+            v, s_, b = vals[:R * Cc // 8], scales[:R * Cc // 64], (biases[:R * Cc // 64] if with_bias else None)
+            got = dys[j].to_host(np.float32).reshape(tokens, R)
+            want = q4_want(oracle, v, s_, b, R, Cc, xs[j])
+            check_class_t(got, want, v, s_, b, R, Cc, xs[j])
+    print("kernels reached:", sorted(kernels), flush=True)
