@@ -19,7 +19,7 @@ reference's own C kernel when oracle/_ref is present (else the checker's
 port), and, under "extra", the same sweep on the bit-exact kernel, the MoE
 decode layer-step, the NVFP4 matvec and the batch-4 sweeps.
 
---only NAME runs a single leg (sweep, sweep-exact, moe, nvfp4, nvfp4-t, copy): what the
+--only NAME runs a single leg (sweep, sweep-exact, sweep-b4, moe, moe-t, nvfp4-t, copy): what the
 rocprofv3 commands in profiles/ use.
 """
 from __future__ import annotations
@@ -96,6 +96,21 @@ class Q4Sweep:
             self.keep += [weights, xs, ys]
             self.launches.append((jobs, G, Cc))
             self.bytes_per_step += G * synth.q4_bytes(R, Cc, tokens)
+
+    def single_launches(self, shape: int, stream):
+        """Every instance of one shape as a launch of its own (what the engine's salt_gpu_q4_matvec issues)."""
+        jobs, G, Cc = self.launches[shape]
+        for g in range(G):
+            j = jobs[g]
+            if self.exact:
+                rc = self.lib.salt_mi355_q4_matvec_dev(j.vals, j.scales, j.biases, j.rows, Cc, self.tokens, j.xs, j.ys, 0,
+                                                       stream)
+            else:
+                rc = self.lib.salt_mi355_q4_matvec_t_dev(j.vals, j.scales, j.biases, j.rows, Cc, self.tokens, j.xs, j.ys,
+                                                         stream)
+            if rc != 0:
+                raise RuntimeError(self.lib.salt_mi355_last_error().decode())
+        return G
 
     def step(self, stream):
         for jobs, G, Cc in self.launches:
@@ -215,25 +230,41 @@ def cpu_other_configs(synth, pool, cores: int, budget_s: float = 3.0):
         bytes_per_s, reps = rate(batch4_pass, nbytes4, budget_s)
         out["q4_sweep_batch4_gbps"] = {"value": round(bytes_per_s / 1e9, 3), "kind": "reference", "cores": cores,
                                        "sample": f"{reps} passes of the 3-shape sweep at batch 4 (one call per token)"}
-    # MoE decode layer-step (port of the reference's step, experts run on `cores` threads)
+    # MoE decode layer-step and grouped prefill: the reference's own public functions in the order of its (static)
+    # step, driven by oracle/ref_moe_driver.c; experts on min(cores, 8) threads as gemma4_text.c:8247-8277
     E, K, H, F = 128, 8, 2816, 704
     g = ExpertGeometry(H, F)
+    stride = pool.nbytes // E
     logits, scale = synth.router_logits(E, 900), np.ones(E, np.float32)
     x = synth.activations(H, 1, 950)[0]
     sel, w = np.zeros(K, np.int32), np.zeros(K, np.float32)
     eo, y = np.zeros((K, H), np.float32), np.zeros(H, np.float32)
-    steps_per_s, reps = rate(lambda: oracle.orc_moe_decode_step(C.byref(g), ptr(pool), E, K, ptr(logits), ptr(scale), ptr(x),
-                                                                ptr(sel), ptr(w), ptr(eo), ptr(y), cores), 1, budget_s)
-    out["moe_decode_step_us"] = {"value": round(1e6 / steps_per_s, 1), "kind": "port", "cores": cores,
-                                 "sample": f"{reps} layer-steps"}
-    # MoE prefill, grouped per expert: a 32-token sample of the 2048-token workload
+    driver = ref is not None and hasattr(ref, "refdrv_moe_decode_step")
+    expert_threads = min(cores, 8)
+    if driver:
+        scratch = np.zeros(K * (2 * F + H), np.float32)
+        step = lambda: ref.refdrv_moe_decode_step(ptr(pool), stride, E, K, H, F, ptr(logits), ptr(scale), ptr(x), ptr(sel),
+                                                  ptr(w), ptr(eo), ptr(y), ptr(scratch), expert_threads)
+    else:
+        step = lambda: oracle.orc_moe_decode_step(C.byref(g), ptr(pool), E, K, ptr(logits), ptr(scale), ptr(x), ptr(sel),
+                                                  ptr(w), ptr(eo), ptr(y), expert_threads)
+    steps_per_s, reps = rate(step, 1, budget_s)
+    out["moe_decode_step_us"] = {"value": round(1e6 / steps_per_s, 1), "kind": "reference-constituents" if driver else "port",
+                                 "cores": expert_threads, "sample": f"{reps} layer-steps"}
+    # MoE prefill, grouped per expert: a 32-token sample of the 2048-token workload through salt_moe_group_execute
     T = 32
     psel, pw = synth.zipf_selection(T, E, K, 1.1, 60)
     px, py = synth.activations(H, T, 61), np.zeros((T, H), np.float32)
-    tok_per_s, reps = rate(lambda: oracle.orc_moe_group(C.byref(g), ptr(pool), E, K, T, ptr(psel), ptr(pw), ptr(px), ptr(py),
-                                                        None, cores), T, budget_s)
-    out["moe_prefill_tokens_per_s"] = {"value": round(tok_per_s, 1), "kind": "port", "cores": cores,
-                                       "sample": f"{reps} passes over {T} tokens"}
+    if driver:
+        gscratch = np.zeros(T * (2 * F + 2 * H + K * H), np.float32)
+        group = lambda: ref.refdrv_moe_group(ptr(pool), stride, E, K, H, F, T, ptr(psel), ptr(pw), ptr(px), ptr(py),
+                                             ptr(gscratch))
+    else:
+        group = lambda: oracle.orc_moe_group(C.byref(g), ptr(pool), E, K, T, ptr(psel), ptr(pw), ptr(px), ptr(py), None, cores)
+    tok_per_s, reps = rate(group, T, budget_s)
+    out["moe_prefill_tokens_per_s"] = {"value": round(tok_per_s, 1), "kind": "reference-constituents" if driver else "port",
+                                       "cores": cores, "sample": f"{reps} passes over {T} tokens; the reference's batch "
+                                       "matvec splits rows over the cores"}
     # the whole feed-forward block of a layer (port of feed_forward; matvecs and experts on `cores` threads)
     from oracle_lib import ffn_layer_struct
     weights = synth.ffn_layer(H, 2112, F, E, K, 70, pool=pool)
@@ -392,7 +423,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the MoE / NVFP4 / batch-4 legs")
-    ap.add_argument("--only", default="", help="run one leg: sweep | sweep-exact | sweep-b4 | moe | moe-t | nvfp4 | nvfp4-t | copy")
+    ap.add_argument("--only", default="", help="run one leg: sweep | sweep-exact | sweep-b4 | sweep-b4-exact | moe | moe-t | nvfp4-t | copy")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU mode (run with --gpus 1)")
@@ -414,13 +445,20 @@ def main():
 
     if not args.no_extra:
         extra = {}
-        del sweep
         extra["q4_sweep_class_t_gbps"] = result["value"]
+        # configs[1] one matrix per launch (what salt_gpu_q4_matvec issues), per shape: microseconds per launch
+        for i, (R, Cc) in enumerate(SWEEP):
+            ms_1 = timed(lib, stream, events, lambda st, i=i: sweep.single_launches(i, st), 1, 3) / sweep.launches[i][1]
+            extra[f"q4_{R}x{Cc}_single_launch_class_t_us"] = round(ms_1 * 1e3, 2)
+        del sweep
         # the same sweep on the bit-exact kernel (the reference's 32-chain order and rounding points)
         sx = Q4Sweep(gpu, synth, tokens=1, exact=True)
         ms_x = timed(lib, stream, events, sx.step, args.warmup, args.steps)
         extra["q4_sweep_bit_exact_gbps"] = round(sx.bytes_per_step / (ms_x * 1e-3) / 1e9, 1)
         extra["q4_sweep_bit_exact_kernel"] = lib.salt_mi355_last_kernel().decode()
+        for i, (R, Cc) in enumerate(SWEEP):
+            ms_1 = timed(lib, stream, events, lambda st, i=i: sx.single_launches(i, st), 1, 3) / sx.launches[i][1]
+            extra[f"q4_{R}x{Cc}_single_launch_bit_exact_us"] = round(ms_1 * 1e3, 2)
         del sx
         # batch 4 of the same sweep, both kernels
         for name, exact in (("q4_sweep_batch4_class_t_gbps", False), ("q4_sweep_batch4_bit_exact_gbps", True)):
@@ -440,6 +478,14 @@ def main():
         pool = synth.expert_pool(E, H, F, 7)
         extra.update(moe_leg(gpu, synth, lib, stream, events, pool, False))
         extra.update(moe_leg(gpu, synth, lib, stream, events, pool, True))
+        # what the step's two launches cost with nothing in them: the same grids, workgroup sizes and LDS, empty bodies
+        # (353 x 384 threads x 63 KB, then 176 x 512 threads x 101 KB: the class-T plan at this geometry)
+        shape = (353, 384, 62_848, 176, 512, 100_608)
+        if lib.salt_mi355_launch_skeleton_dev(*shape, stream) == 0:
+            ms_sk = timed(lib, stream, events, lambda st: lib.salt_mi355_launch_skeleton_dev(*shape, st), 5, 200)
+            extra["moe_launch_skeleton_us"] = round(ms_sk * 1e3, 2)
+            ms_sk1 = timed(lib, stream, events, lambda st: lib.salt_mi355_launch_skeleton_dev(128, 512, 0, 0, 0, 0, st), 5, 200)
+            extra["single_launch_skeleton_us"] = round(ms_sk1 * 1e3, 2)
         # the whole feed-forward block of a decoder layer for one token: pre-norms, dense FFN (2112 wide), router input,
         # 8-bit gate, top-8 of 128, routed experts, parallel combine -- bit-exact, device-resident.  32 residuals taken
         # in turn: the routing, hence the experts read, changes from block to block.

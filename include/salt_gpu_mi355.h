@@ -70,13 +70,24 @@ int salt_mi355_event_elapsed_ms(void *start, void *stop, float *ms);
 /* Stream capture for callers that replay a fixed sequence of the device-resident
  * entry points as one HIP graph.  Capturable: every *_dev entry point that takes
  * a status word and neither uploads a job table nor waits (the MoE decode step,
- * the feed-forward block, the cells, single-matrix matvecs).  begin starts a
+ * the feed-forward block, the cells, single-matrix matvecs, *_jobs_* launches
+ * of up to 16 jobs: their records travel in the kernel arguments).  A *_jobs_*
+ * call with more jobs copies a table to the device through a ring of pinned
+ * buffers that it waits on and rewrites: under capture it is refused (-1) with
+ * an error that says so.  begin starts a
  * capture on `stream`; end finishes it and returns an executable graph (NULL on
  * failure); launch replays it on `stream`. */
 int salt_mi355_graph_begin(void *stream);
 void *salt_mi355_graph_end(void *stream);
 int salt_mi355_graph_launch(void *graph_exec, void *stream);
 int salt_mi355_graph_destroy(void *graph_exec);
+/* Measurement aid (no counterpart in the reference): one or two kernels with
+ * empty bodies, launched one after the other on `stream` with the given
+ * numbers of workgroups, threads per workgroup and bytes of dynamic LDS
+ * (workgroups 0: that launch is left out).  What a step's launches cost with
+ * nothing in them: the floor its arithmetic sits on. */
+int salt_mi355_launch_skeleton_dev(int workgroups_a, int threads_a, int lds_bytes_a,
+                                   int workgroups_b, int threads_b, int lds_bytes_b, void *stream);
 
 /* ---- affine Q4 ("mlx4") matvec, device-resident ------------------------
  * Layout as the reference's salt_q4_matvec (kernels.h:117-130): u32 words of

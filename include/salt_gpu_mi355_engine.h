@@ -193,7 +193,10 @@ typedef struct SaltGpuMoeExpert {                 /* reference gpu.h:276-295 */
 
 /* reference gpu.h:320-329: gate, up, gelu*up, down for `count` experts; rows
  * of inputs/outputs grouped by expert in the order given; the weighted
- * reduction stays with the engine. */
+ * reduction stays with the engine.  The _selected form takes its four buffers
+ * as shared buffers and the device reads `inputs` where they lie, without a
+ * snapshot: they must stay unchanged until the call returns or, in deferred
+ * mode (salt_gpu_set_defer), until salt_gpu_sync() has returned. */
 int salt_gpu_q4_moe_chain(const SaltGpuMoeExpert *experts, int count, int hidden, int routed, const float *inputs,
                           float *outputs, float *gate_scratch, float *up_scratch, size_t scratch_float_capacity);
 int salt_gpu_q4_moe_chain_selected(const SaltGpuMoeExpert *experts, int count, int hidden, int routed,

@@ -93,6 +93,15 @@ int verify_converters() {
 
 State::TableSlot *table_acquire(const void *host_table, size_t nbytes, hipStream_t stream) {
     State &s = g_state;
+    // Not under stream capture: the ring waits on events and rewrites pinned memory between calls, and a captured
+    // upload would not have run when the next call compares bytes.  Launches whose jobs travel in the kernel
+    // arguments (up to Q4_INLINE_JOBS) need no table and can be captured.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capture) != hipSuccess) { (void)hipGetLastError(); capture = hipStreamCaptureStatusNone; }
+    if (capture != hipStreamCaptureStatusNone) {
+        set_error("a launch of more than %d jobs uploads a job table and cannot be captured into a graph", Q4_INLINE_JOBS);
+        return nullptr;
+    }
     // A decode loop sends the same tables token after token: a slot that already holds these bytes, uploaded on this
     // stream, is used again without a copy (stream order puts the earlier upload before the new reader).
     for (State::TableSlot &held : s.tables)
@@ -170,6 +179,7 @@ int salt_mi355_init(void) {
         s.fork = s.join = nullptr;
         return -1;
     }
+    if (moe_static_scratch_prepare() != 0) return -1;
     s.ready = 1;
     if (getenv("SALT_GPU_DIAG"))
         fprintf(stderr, "salt-mi355: ready on %s, %d CUs, fp8 code scale %g\n", prop.gcnArchName,

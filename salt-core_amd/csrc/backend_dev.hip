@@ -632,6 +632,41 @@ int salt_mi355_moe_decode_step_t_dev(const void *pool, size_t expert_stride, int
                                           x, selected, weights, expert_out, out, workspace, stream);
 }
 
+// ---------------------------------------------------------------- launch skeleton (measurement aid)
+
+}  // extern "C"
+
+namespace {
+__global__ void skeleton_kernel(int *never) {
+    if (never && threadIdx.x == 0x7fffffff) *never = 1;       // nothing
+}
+}  // namespace
+
+extern "C" {
+
+int salt_mi355_launch_skeleton_dev(int workgroups_a, int threads_a, int lds_bytes_a, int workgroups_b, int threads_b,
+                                   int lds_bytes_b, void *stream) {
+    if (!g_state.ready) { set_error("launch skeleton: library not initialised"); return -1; }
+    const int shapes[2][3] = {{workgroups_a, threads_a, lds_bytes_a}, {workgroups_b, threads_b, lds_bytes_b}};
+    static int raised = 0;
+    for (const int (&shape)[3] : shapes) {
+        if (shape[0] == 0) continue;
+        if (shape[0] < 0 || shape[1] < 1 || shape[1] > 1024 || shape[2] < 0 || shape[2] > DOT_LDS_LIMIT) {
+            set_error("launch skeleton: bad shape");
+            return -1;
+        }
+        if (shape[2] > raised) {
+            if (hip_ok(hipFuncSetAttribute((const void *)skeleton_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, shape[2]),
+                       "hipFuncSetAttribute") != 0)
+                return -1;
+            raised = shape[2];
+        }
+        hipLaunchKernelGGL(skeleton_kernel, dim3(shape[0]), dim3(shape[1]), shape[2], (hipStream_t)stream, (int *)nullptr);
+        if (hip_ok(hipGetLastError(), "skeleton launch") != 0) return -1;
+    }
+    return 0;
+}
+
 // ---------------------------------------------------------------- the same step without a workspace argument
 
 }  // extern "C"
@@ -641,6 +676,14 @@ int salt_mi355_moe_decode_step_t_dev(const void *pool, size_t expert_stride, int
 // device and kept below.
 static __device__ __align__(256) unsigned char moe_static_scratch[SALT_MI355_MOE_STATIC_SCRATCH_BYTES];
 static void *moe_static_scratch_address[16];        // by device ordinal; nullptr = not looked up yet
+
+static void *moe_static_scratch_of_current_device();
+
+namespace mi355 {
+// Called by salt_mi355_init on the device it initialises: the entry point then finds the address without a runtime
+// query (one that could load the code object in the middle of a capture or a serving loop).
+int moe_static_scratch_prepare() { return moe_static_scratch_of_current_device() ? 0 : -1; }
+}  // namespace mi355
 
 static void *moe_static_scratch_of_current_device() {
     int device = -1;

@@ -120,6 +120,7 @@ int q4_dot16_launch(const Q4DotLaunch &launch, int waves, hipStream_t stream);
 // gelu_tanh(gate) * up in the prologue of the second); -1: the geometry is not served.
 // The whole step in two launches (moe_dot16.hip): gate + up + activation, then down + ordered weighted sum; `out`
 // receives the layer output, moe.expert_out (optional) the expert outputs.  -1: the geometry is not served.
+int moe_static_scratch_prepare();      // backend_dev.hip: looks up the static MoE workspace of the current device
 constexpr int MOE16_NOT_SERVED = 1;
 int moe16_step_launch(const MoeFuse &moe, float *out, hipStream_t stream);
 int q4_dot_moe_gate_up_launch(const MoeFuse &moe, hipStream_t stream);

@@ -146,6 +146,9 @@ def load_reference() -> C.CDLL | None:
     _sig(lib.salt_gemma4_residual_postnorm, i, vp, vp, vp, vp, i, f)
     _sig(lib.salt_gemma4_parallel_ffn_combine, i, vp, vp, vp, vp, vp, vp, vp, f, i, f, vp)
     _sig(lib.salt_gemma4_softcap, i, vp, i, f)
+    if hasattr(lib, "refdrv_moe_decode_step"):          # oracle/ref_moe_driver.c, compiled into the same library
+        _sig(lib.refdrv_moe_decode_step, i, vp, C.c_size_t, i, i, i, i, vp, vp, vp, vp, vp, vp, vp, vp, i)
+        _sig(lib.refdrv_moe_group, i, vp, C.c_size_t, i, i, i, i, i, vp, vp, vp, vp, vp)
     return lib
 
 

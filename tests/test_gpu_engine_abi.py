@@ -363,6 +363,18 @@ def test_expert_seats_through_residency_and_selected_chain(eng, oracle, pkg):
     assert rc == 0, err(pkg)
     want = chain_want(oracle, pool, H, F, [chosen[i] for i in order], [1] * K, np.tile(x, (K, 1)))
     assert np.array_equal(bits(aout.reshape(K, H)), bits(want))
+    # deferred mode: the device reads the shared inputs where they lie and the outputs are published by sync, so the
+    # caller leaves the inputs alone until then
+    x2 = synth.activations(H, 1, 54)[0]
+    ain[:] = np.tile(x2, K)
+    aout[:] = -1.0
+    assert eng.salt_gpu_set_defer(1) == 0
+    assert eng.salt_gpu_q4_moe_chain_selected(recs, K, H, F, bin_.contents, bout.contents, bg.contents, bu.contents, K * F) == 0, err(pkg)
+    assert eng.salt_gpu_sync() == 0
+    assert np.array_equal(bits(aout.reshape(K, H)),
+                          bits(chain_want(oracle, pool, H, F, [chosen[i] for i in order], [1] * K, np.tile(x2, (K, 1)))))
+    assert eng.salt_gpu_set_defer(0) == 0
+    ain[:] = np.tile(x, K)
     # plain host memory instead of shared buffers is refused
     plain = np.zeros(K * H, np.float32)
     assert eng.salt_gpu_q4_moe_chain_selected(recs, K, H, F, ptr(plain), bout.contents, bg.contents, bu.contents, K * F) == -1

@@ -238,3 +238,35 @@ def test_router_topk_equals_compiled_reference(oracle, reference, seed):
 def test_mix64_equals_compiled_reference(oracle, reference):
     for v in [0, 1, 2 ** 64 - 1, 0xDEADBEEF, 0x9E3779B97F4A7C15]:
         assert oracle.orc_mix64(v) == reference.salt_mix64(v)
+
+
+def test_decode_step_and_group_equal_the_reference_driven_through_its_public_functions(oracle, reference):
+    """oracle/ref_moe_driver.c calls the reference's own router, matvecs, gelu and grouped executor in the order of
+    its (static) MoE step; the checker's step and group must give the same bits."""
+    if not hasattr(reference, "refdrv_moe_decode_step"):
+        pytest.skip("the reference library was built without the driver")
+    E, K, H, F = 16, 4, 256, 128
+    pool = synth.expert_pool(E, H, F, 71)
+    stride = synth.expert_slot_bytes(H, F)
+    g = ExpertGeometry(H, F)
+    logits, scale = synth.router_logits(E, 72), (1.0 + 0.1 * synth.router_logits(E, 73)).astype(np.float32)
+    x = synth.activations(H, 1, 74)[0]
+    sel, w, eo, y = np.zeros(K, np.int32), np.zeros(K, np.float32), np.zeros((K, H), np.float32), np.zeros(H, np.float32)
+    assert oracle.orc_moe_decode_step(C.byref(g), ptr(pool), E, K, ptr(logits), ptr(scale), ptr(x), ptr(sel), ptr(w),
+                                      ptr(eo), ptr(y), 2) == 0
+    rsel, rw, reo, ry = np.zeros(K, np.int32), np.zeros(K, np.float32), np.zeros((K, H), np.float32), np.zeros(H, np.float32)
+    scratch = np.zeros(K * (2 * F + H), np.float32)
+    for threads in (1, 3):
+        assert reference.refdrv_moe_decode_step(ptr(pool), stride, E, K, H, F, ptr(logits), ptr(scale), ptr(x), ptr(rsel),
+                                                ptr(rw), ptr(reo), ptr(ry), ptr(scratch), threads) == 0
+        assert np.array_equal(rsel, sel) and np.array_equal(bits(rw), bits(w))
+        assert np.array_equal(bits(reo), bits(eo)) and np.array_equal(bits(ry), bits(y))
+    T = 9
+    gsel, gw = synth.zipf_selection(T, E, K, 1.1, 75)
+    xs = synth.activations(H, T, 76)
+    want, got = np.zeros((T, H), np.float32), np.zeros((T, H), np.float32)
+    assert oracle.orc_moe_group(C.byref(g), ptr(pool), E, K, T, ptr(gsel), ptr(gw), ptr(xs), ptr(want), None, 2) == 0
+    gscratch = np.zeros(T * (2 * F + 2 * H + K * H), np.float32)
+    assert reference.refdrv_moe_group(ptr(pool), stride, E, K, H, F, T, ptr(gsel), ptr(gw), ptr(xs), ptr(got),
+                                      ptr(gscratch)) == 0
+    assert np.array_equal(bits(got), bits(want))

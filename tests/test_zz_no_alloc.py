@@ -10,7 +10,15 @@ pytestmark = pytest.mark.gpu
 synth = cases.synth
 
 
-def run_both(pkg, E, K, H, F, pool_seed, logit_seed, x_seed):
+def free_device_bytes():
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    free, total = C.c_size_t(0), C.c_size_t(0)
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
+def run_both(pkg, E, K, H, F, pool_seed, logit_seed, x_seed, status_word=True):
     gpu = pkg.lib
     lib = gpu.init()
     pool = synth.expert_pool(E, H, F, pool_seed)
@@ -22,12 +30,19 @@ def run_both(pkg, E, K, H, F, pool_seed, logit_seed, x_seed):
     eo, out = gpu.DeviceBuffer(K * H * 4, fill=0xEE), gpu.DeviceBuffer(H * 4, fill=0xEE)
     status = gpu.DeviceBuffer(4, fill=0x7F)
     stream = lib.salt_mi355_stream()
-    rc = lib.salt_mi355_moe_decode_step_static_dev(layer.pool.at(0), layer.stride, H, F, E, K, layer.logits.ptr,
-                                                   layer.scale.ptr, layer.x.ptr, sel.ptr, w.ptr, eo.ptr, out.ptr,
-                                                   status.ptr, stream)
-    assert rc == 0, lib.salt_mi355_last_error().decode()
-    gpu.check(lib.salt_mi355_stream_sync(stream), "sync")
-    got = (int(status.to_host(np.int32)[0]), sel.to_host(np.int32), w.to_host(np.float32),
+
+    def call():
+        rc = lib.salt_mi355_moe_decode_step_static_dev(layer.pool.at(0), layer.stride, H, F, E, K, layer.logits.ptr,
+                                                       layer.scale.ptr, layer.x.ptr, sel.ptr, w.ptr, eo.ptr, out.ptr,
+                                                       status.ptr if status_word else None, stream)
+        assert rc == 0, lib.salt_mi355_last_error().decode()
+        gpu.check(lib.salt_mi355_stream_sync(stream), "sync")
+
+    call()                                                                # warm: code objects are loaded
+    before = free_device_bytes()
+    call()
+    assert free_device_bytes() == before, "the static step changed the amount of free device memory"
+    got = (int(status.to_host(np.int32)[0]) if status_word else 0, sel.to_host(np.int32), w.to_host(np.float32),
            eo.to_host(np.float32).reshape(K, H), out.to_host(np.float32))
     assert got[0] == want[0] == 0
     assert np.array_equal(got[1], want[1])
@@ -42,6 +57,8 @@ def test_static_workspace_step_equals_the_workspace_step(pkg):
     run_both(pkg, 8, 3, 256, 128, 13, 615, 616)
     print("static step: five-launch plan (more experts than the router prologue holds)", flush=True)
     run_both(pkg, 520, 4, 128, 64, 14, 617, 618)
+    print("static step: status word inside the static workspace", flush=True)
+    run_both(pkg, 16, 8, 2816, 704, 15, 619, 620, status_word=False)
 
 
 def test_static_workspace_step_refuses_what_does_not_fit(pkg):
