@@ -202,19 +202,27 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
         if (PRO == 1) {
             RouterShared &sh = *reinterpret_cast<RouterShared *>(w_lds);
             const bool publisher = (int)blockIdx.x == L.total_tiles;       // one workgroup past the tiles
-            router_topk_block(m.logits, m.per_expert_scale, m.n_experts, m.topk, true, publisher, sh);
-            const int bad = sh.bad;
-            if (publisher) {
-                if (tid == 0) *m.status = bad ? -1 : 0;
-                if (tid < m.topk && !bad) { m.selected[tid] = sh.out_sel[tid]; m.weights[tid] = sh.out_w[tid]; }
-                return;
-            }
-            if (bad) return;                                               // uniform
             const int up_tiles = (m.routed + TILE_ROWS - 1) / TILE_ROWS;
             const int slot_index = (int)blockIdx.x / up_tiles;             // 2 * place + (0 gate | 1 up)
             const int place = slot_index >> 1, proj = slot_index & 1;
-            const int expert = __builtin_amdgcn_readfirstlane(sh.out_sel[place]);
-            __syncthreads();                                               // the staging memory is free again
+            int expert;
+            if (!publisher && m.n_experts <= ROUTER_WAVE_MAX_EXPERTS) {
+                // every wave finds the workgroup's expert on its own: no LDS, no barrier (the publisher keeps the
+                // whole router: ordered sums, weights, status)
+                expert = router_select_wave(m.logits, m.per_expert_scale, m.n_experts, m.topk, place);
+                if (expert < 0) return;                                    // uniform: every wave sees the same inputs
+            } else {
+                router_topk_block(m.logits, m.per_expert_scale, m.n_experts, m.topk, true, publisher, sh);
+                const int bad = sh.bad;
+                if (publisher) {
+                    if (tid == 0) *m.status = bad ? -1 : 0;
+                    if (tid < m.topk && !bad) { m.selected[tid] = sh.out_sel[tid]; m.weights[tid] = sh.out_w[tid]; }
+                    return;
+                }
+                if (bad) return;                                           // uniform
+                expert = __builtin_amdgcn_readfirstlane(sh.out_sel[place]);
+                __syncthreads();                                           // the staging memory is free again
+            }
             job.vals = m.pool + (size_t)expert * m.expert_stride + (size_t)proj * proj_bytes;
             job.x = m.x;
             job.y = (proj ? m.up : m.gate) + (size_t)place * m.routed;
