@@ -67,6 +67,17 @@ int salt_mi355_event_destroy(void *event);
 int salt_mi355_event_record(void *event, void *stream);
 /* Waits for `stop`, then returns the milliseconds between the two events. */
 int salt_mi355_event_elapsed_ms(void *start, void *stop, float *ms);
+/* Policy, off by default: with it the engine entry points (salt_gpu_q4_matvec,
+ * salt_gpu_q4_batch, salt_gpu_proj_batch*, salt_gpu_q4_moe_chain*,
+ * salt_gpu_nvfp4_matvec / _batch of up to four tokens) run the tolerance-class
+ * kernels of salt_mi355_q4_jobs_t_dev / salt_mi355_nvfp4_matvec_t_dev instead of
+ * the bit-exact ones: results then carry those entry points' stated bounds
+ * and are no longer bit-identical to the reference CPU kernels.  Never read
+ * from the environment: an engine opts in with this call (compare the
+ * reference's own policy setters salt_gpu_set_mapped_only / salt_gpu_set_defer,
+ * gpu.h:96-100, 190-192).  Returns the previous setting. */
+int salt_mi355_set_tolerance_class(int enabled);
+
 /* Stream capture for callers that replay a fixed sequence of the device-resident
  * entry points as one HIP graph.  Capturable: every *_dev entry point that takes
  * a status word and neither uploads a job table nor waits (the MoE decode step,

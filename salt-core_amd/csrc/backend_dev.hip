@@ -632,6 +632,14 @@ int salt_mi355_moe_decode_step_t_dev(const void *pool, size_t expert_stride, int
                                           x, selected, weights, expert_out, out, workspace, stream);
 }
 
+// ---------------------------------------------------------------- policy
+
+int salt_mi355_set_tolerance_class(int enabled) {
+    const int before = g_state.tolerance_class;
+    g_state.tolerance_class = enabled != 0;
+    return before;
+}
+
 // ---------------------------------------------------------------- launch skeleton (measurement aid)
 
 }  // extern "C"

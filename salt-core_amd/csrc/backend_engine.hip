@@ -584,8 +584,12 @@ int run_q4_jobs(std::vector<HostJob> &jobs, int C, std::vector<OutputCopy> *copi
                 group.push_back(q);
             }
             if (group.empty()) continue;
-            // ys of a job is [tokens][rows]: the sub-launch writes rows `first..first+width` of it
-            if (salt_mi355_q4_jobs_dev(group.data(), (int)group.size(), C, width, 0, g_state.stream) != 0) return -1;
+            // ys of a job is [tokens][rows]: the sub-launch writes rows `first..first+width` of it.  Bit-exact kernels
+            // unless the engine has opted into the tolerance class (salt_mi355_set_tolerance_class).
+            const int rc = g_state.tolerance_class
+                ? salt_mi355_q4_jobs_t_dev(group.data(), (int)group.size(), C, width, g_state.stream)
+                : salt_mi355_q4_jobs_dev(group.data(), (int)group.size(), C, width, 0, g_state.stream);
+            if (rc != 0) return -1;
         }
     }
     return 0;
@@ -1123,7 +1127,8 @@ int moe_chain(const SaltGpuMoeExpert *experts, int count, int hidden, int routed
     std::vector<OutputCopy> none;
     if (run_q4_jobs(jobs, hidden, &none) != 0) { (void)salt_gpu_sync(); return -1; }
     // Decode shape (one row per expert): gelu_tanh(gate) * up is computed in the prologue of the down launch.
-    bool one_row_each = (routed & 63) == 0 && routed <= 4096;
+    // (the tolerance-class kernels take the activation as a vector: that policy keeps the activation launch)
+    bool one_row_each = !g_state.tolerance_class && (routed & 63) == 0 && routed <= 4096;
     for (int i = 0; i < count && one_row_each; ++i)
         one_row_each = experts[i].group == 1 && ((uintptr_t)down[(size_t)i].vals & 3) == 0 &&
                        ((uintptr_t)down[(size_t)i].scales & 1) == 0 && ((uintptr_t)down[(size_t)i].biases & 1) == 0;
@@ -1398,7 +1403,12 @@ int run_fp4_jobs(std::vector<Fp4HostJob> &jobs, int C) {
         float *dq_dev = (float *)device_take(xin * 4);
         uint8_t *y_dev = device_take(yout * 4), *y_pin = pinned_take(yout * 4);
         const bool one_launch = !all_single && j.tokens == 1 && C <= FP4_FUSED_MAX_COLS;
-        if (one_launch) {
+        if (g_state.tolerance_class && j.tokens <= 4) {
+            // the tolerance-class kernel quantises the activation inside its launch
+            if (salt_mi355_nvfp4_matvec_t_dev(j.packed, j.scales, j.tensor->stored_divisor, j.tensor->input_global_scale,
+                                              j.rows, C, j.tokens, x_dev, (float *)y_dev, st_dev, g_state.stream) != 0)
+                return -1;
+        } else if (one_launch) {
             if (salt_mi355_nvfp4_matvec_qdq_dev(j.packed, j.scales, j.tensor->stored_divisor,
                                                 j.tensor->input_global_scale, j.rows, C, x_dev, (float *)y_dev, st_dev, 0,
                                                 g_state.stream) != 0)
@@ -1407,7 +1417,7 @@ int run_fp4_jobs(std::vector<Fp4HostJob> &jobs, int C) {
             if (salt_mi355_nvfp4_qdq_dev(x_dev, C, j.tokens, j.tensor->input_global_scale, nullptr, nullptr, dq_dev,
                                          st_dev, g_state.stream) != 0)
                 return -1;
-            if (all_single) {
+            if (all_single && !g_state.tolerance_class) {
                 SaltMi355Fp4Job t;
                 t.packed = j.packed; t.scales = j.scales; t.stored_divisor = j.tensor->stored_divisor;
                 t.xs = dq_dev; t.ys = (float *)y_dev; t.rows = j.rows;
@@ -1426,7 +1436,7 @@ int run_fp4_jobs(std::vector<Fp4HostJob> &jobs, int C) {
         stats.nvfp4_projection_output_bytes += yout * 4;
         stats.nvfp4_kernel_launches += one_launch ? 1 : all_single ? 1 : 2 + (uint64_t)((j.tokens - 1) / 4);
     }
-    if (all_single) {
+    if (all_single && !table.empty()) {
         if (salt_mi355_nvfp4_jobs_dev(table.data(), (int)table.size(), C, 1, 0, g_state.stream) != 0) return -1;
         stats.nvfp4_kernel_launches += 1;
     }

@@ -15,6 +15,7 @@ struct State {
     hipStream_t stream = nullptr;
     hipStream_t side = nullptr;         // second branch of a forked sequence (default priority, like every stream)
     hipEvent_t fork = nullptr, join = nullptr;
+    int tolerance_class = 0;            // policy: the engine entry points may run the tolerance-class kernels
     float code_scale = 0.0f;            // 1 / fp8_table[1]
     int fp8_is_ocp = 0;                 // the converter decodes every byte as OCP E4M3FN
     float fp8_table[256] = {0};

@@ -84,6 +84,7 @@ def load() -> C.CDLL:
     _sig(lib.salt_mi355_graph_end, vp, vp)
     _sig(lib.salt_mi355_graph_launch, i, vp, vp)
     _sig(lib.salt_mi355_graph_destroy, i, vp)
+    _sig(lib.salt_mi355_set_tolerance_class, i, i)
     _sig(lib.salt_mi355_launch_skeleton_dev, i, i, i, i, i, i, i, vp)
     _sig(lib.salt_mi355_event_create, vp)
     _sig(lib.salt_mi355_event_destroy, i, vp)

@@ -258,6 +258,49 @@ def test_moe_chain_from_a_layer_resource(eng, oracle, pkg):
     eng.salt_gpu_set_mapped_only(0)
 
 
+def test_tolerance_class_policy_reaches_the_engine_entry_points(eng, oracle, pkg):
+    """salt_mi355_set_tolerance_class(1): salt_gpu_q4_matvec and the decode-shaped salt_gpu_q4_moe_chain run the
+    tolerance-class kernels (salt_mi355_last_kernel says so) inside their stated bounds; switched off again, the same
+    calls are bit-identical to the CPU checker."""
+    from moe_bounds import down_term_magnitudes, expert_activation
+    from q4_bounds import check as check_class_t
+    lib = pkg.lib.load()
+    trunk = Trunk([(704, 2816)], 21)
+    assert eng.salt_gpu_weight_resource_describe(TRUNK, 17, trunk.base, trunk.blob.nbytes) == 0
+    assert eng.salt_gpu_weight_resource_activate(TRUNK, 17, 2) == 0, err(pkg)
+    R, Cc, _, vals, scales, biases = trunk.views[0]
+    v0, s0, b0 = trunk.pointers(0)
+    x = synth.activations(Cc, 1, 22)[0]
+    want = q4_want(oracle, vals, scales, biases, R, Cc, x)
+    E, H, F = 8, 2816, 704
+    pool = synth.expert_pool(E, H, F, 23)
+    assert eng.salt_gpu_expert_resource_bind(19, pool.ctypes.data, pool.nbytes) == 0, err(pkg)
+    experts = [1, 4, 6]
+    recs = (abi.MoeExpert * 3)(*[expert_record(pool, e, H, F, 1) for e in experts])
+    xin = np.tile(synth.activations(H, 1, 24)[0], (3, 1)); outputs = np.zeros((3, H), np.float32)
+    scratch = np.zeros((2, 3 * F), np.float32)
+    chain = chain_want(oracle, pool, H, F, experts, [1, 1, 1], xin)
+
+    assert lib.salt_mi355_set_tolerance_class(1) == 0
+    y = np.zeros(R, np.float32)
+    assert eng.salt_gpu_q4_matvec(v0, s0, b0, R, Cc, ptr(x), ptr(y)) == 0, err(pkg)
+    assert lib.salt_mi355_last_kernel().decode().startswith("q4_dot")
+    check_class_t(y[None, :], want, vals, scales, biases, R, Cc, x[None, :])
+    assert eng.salt_gpu_q4_moe_chain(recs, 3, H, F, ptr(xin), ptr(outputs), ptr(scratch[0]), ptr(scratch[1]), 3 * F) == 0, err(pkg)
+    assert lib.salt_mi355_last_kernel().decode().startswith("q4_dot")
+    for i, e in enumerate(experts):
+        terms = down_term_magnitudes(pool, e, expert_activation(pool, e, xin[i:i + 1], H, F), H, F)[0]
+        assert (np.abs(outputs[i].astype(np.float64) - chain[i]) <= 2.0 ** -18 * terms + 1e-6).all()
+
+    assert lib.salt_mi355_set_tolerance_class(0) == 1
+    assert eng.salt_gpu_q4_matvec(v0, s0, b0, R, Cc, ptr(x), ptr(y)) == 0, err(pkg)
+    assert np.array_equal(bits(y), bits(want[0]))
+    assert eng.salt_gpu_q4_moe_chain(recs, 3, H, F, ptr(xin), ptr(outputs), ptr(scratch[0]), ptr(scratch[1]), 3 * F) == 0, err(pkg)
+    assert np.array_equal(bits(outputs), bits(chain))
+    assert eng.salt_gpu_expert_resource_unbind(19) == 0
+    assert eng.salt_gpu_weight_resource_deactivate(TRUNK, 17) == 0 and eng.salt_gpu_weight_resource_unbind(TRUNK, 17) == 0
+
+
 def test_moe_chain_from_a_pool_file_image(eng, oracle, pkg):
     """The engine's expert pool file: three 64-bit header words {slot bytes, layers, experts}, then the slots
     (reference gemma4_text.c:73-79, 1618-1623).  The whole image is one resource; every tensor in it sits 8 bytes past a
