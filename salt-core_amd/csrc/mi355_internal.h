@@ -103,6 +103,10 @@ struct Q4DotLaunch {
     int total_wgs;
     int ksplit;               // filled by q4_dot_launch from the shape
     int wgs_per_job;          // > 0 when every job of the table has this many workgroups (workgroup -> job by division)
+    // q4_dot16_launch only.  passes > 1: the launch covers tokens_total tokens in passes of `tokens` each (the last
+    // may hold fewer); every block of rows is walked once per pass by workgroups that the dispatcher places next
+    // to each other, so that all passes but the first find the weights in the cache they share.
+    int passes, tokens_total;
     MoeFuse moe;              // only read by q4_dot_moe_gate_up_launch / q4_dot_moe_down_launch
     // Up to Q4_INLINE_JOBS job records inside the kernel arguments (table == nullptr, njobs > 1): a decode-sized
     // batch then needs no table upload.  Must stay the last member.
@@ -116,6 +120,7 @@ int q4_dot_launch(const Q4DotLaunch &launch, const DotShape &shape, hipStream_t 
 // q4_dot16_waves: waves per workgroup to use (a workgroup owns that many blocks of 16 rows), or 0 = use the 32-row kernel.
 int q4_dot16_waves(int cols, int tokens, long long total_blocks32);
 int q4_dot16_launch(const Q4DotLaunch &launch, int waves, hipStream_t stream);
+bool q4_dot16_takes_passes(int tokens_per_pass, int waves);
 // The MoE decode step's two matvec launches on the streaming kernel (router top-k in the prologue of the first,
 // gelu_tanh(gate) * up in the prologue of the second); -1: the geometry is not served.
 // The whole step in two launches (moe_dot16.hip): gate + up + activation, then down + ordered weighted sum; `out`

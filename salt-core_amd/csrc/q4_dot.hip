@@ -82,13 +82,10 @@ __device__ __forceinline__ Q4Job dot_find_job(const Q4DotLaunch &L, int wg) {
 // workgroup derives its gate or up job from the selection (one workgroup past the jobs publishes selection, weights
 // and status); 2 = the down projection of one selected expert, whose activation gelu_tanh(gate) * up is computed
 // while the digit planes are built.
-//
-// NB = 2 gives every wave two consecutive blocks of 32 rows, walked back to back as one stream of steps (the second
-// block's first loads go out while the first block's last steps are consumed): launches with many blocks, rows not
-// cut, MD = 16.  Both blocks' scales and biases are fetched before the stream starts.
-template <int T, int WAVES, int STAGES, int MD, int PRO = 0, int NB = 1>
+template <int T, int WAVES, int STAGES, int MD, int PRO = 0>
 __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L) {
-    static_assert(NB == 1 || (NB == 2 && MD == 16 && PRO == 0), "two blocks per wave: plain jobs, short rows");
+    constexpr int NB = 1;        // blocks of 32 rows a wave walks back to back (launches with many blocks take the
+                                 // sixteen-row kernel instead of a longer walk here)
     static_assert(T >= 1 && T <= 4 && STAGES >= 2 && STAGES <= 4 && (MD == 16 || MD == 32), "tokens per pass, steps per wave");
     static_assert(PRO == 0 || (T == 1 && sizeof(RouterShared) <= (size_t)WAVES * STAGES * STEP_LDS),
                   "the MoE prologues serve one token; the router borrows the weight staging memory");
@@ -507,19 +504,19 @@ size_t dot_lds_bytes(int cols, int tokens, int waves, int stages) {
     return (size_t)waves * stages * STEP_LDS + ZERO_BYTES + (size_t)tokens * 2 * sg * (GROUP_IMAGE + 8);
 }
 
-template <int T, int WAVES, int STAGES, int MD, int PRO = 0, int NB = 1>
+template <int T, int WAVES, int STAGES, int MD, int PRO = 0>
 int launch_shape(const Q4DotLaunch &L, hipStream_t stream) {
     const size_t lds = dot_lds_bytes(L.cols, T, WAVES, STAGES);
     static size_t raised = 0;                 // per instantiation: the largest dynamic LDS size asked for so far
     if (lds > raised) {
-        if (hipFuncSetAttribute((const void *)q4_dot_kernel<T, WAVES, STAGES, MD, PRO, NB>,
+        if (hipFuncSetAttribute((const void *)q4_dot_kernel<T, WAVES, STAGES, MD, PRO>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
             return -1;
         raised = lds;
     }
-    note_kernel("q4_dot_kernel<%d,%d,%d,%d,%d,%d> ksplit %d", T, WAVES, STAGES, MD, PRO, NB, L.ksplit);
+    note_kernel("q4_dot_kernel<%d,%d,%d,%d,%d> ksplit %d", T, WAVES, STAGES, MD, PRO, L.ksplit);
     // the router prologue has one more workgroup: the one that publishes its outputs
-    hipLaunchKernelGGL((q4_dot_kernel<T, WAVES, STAGES, MD, PRO, NB>), dim3(L.total_wgs + (PRO == 1 ? 1 : 0)),
+    hipLaunchKernelGGL((q4_dot_kernel<T, WAVES, STAGES, MD, PRO>), dim3(L.total_wgs + (PRO == 1 ? 1 : 0)),
                        dim3(WAVES * 64), lds, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
@@ -552,11 +549,7 @@ DotShape q4_dot_shape(int cols, int tokens, long long total_blocks) {
     for (const Candidate &c : CANDIDATES)
         if (c.waves % ksplit == 0 && (ksplit == 1 || c.waves >= 4) &&
             dot_lds_bytes(cols, tokens, c.waves, c.stages) * c.resident <= DOT_LDS_LIMIT) {
-            // Two blocks per wave (a stream twice as long) where the launch has plenty of blocks, the rows are not
-            // cut and a lane's registers hold both blocks' scales (rows of up to 4096 columns, four waves).
-            const bool can = ksplit == 1 && nstage * STAGE_GROUPS <= 32 && c.waves == 4 && c.stages == 2;
-            const int nb = can && total_blocks >= 2048 ? 2 : 1;
-            return DotShape{c.waves, c.stages, ksplit, nb};
+            return DotShape{c.waves, c.stages, ksplit, 1};
         }
     return DotShape{4, 2, ksplit <= 4 ? ksplit : 4, 1};
 }
@@ -570,13 +563,7 @@ int q4_dot_launch(const Q4DotLaunch &launch, const DotShape &shape, hipStream_t 
     // groups of a strip that one wave walks: its registers hold 32 (MD = 16) or 64 (MD = 32)
     const int steps = dot_steps(L.cols >> 6);
     const int md = ((steps + shape.ksplit - 1) / shape.ksplit) * STAGE_GROUPS <= 32 ? 16 : 32;
-    if (shape.blocks_per_wave == 2) {
-        if (md != 16 || shape.ksplit != 1 || shape.stages != 2) return -1;
-#define DOT_NB2(TT, WW) if (L.tokens == TT && shape.waves == WW) return launch_shape<TT, WW, 2, 16, 0, 2>(L, stream)
-        DOT_NB2(1, 4); DOT_NB2(2, 4); DOT_NB2(3, 4); DOT_NB2(4, 4);
-#undef DOT_NB2
-        return -1;
-    }
+    if (shape.blocks_per_wave != 1) return -1;
 #define DOT_CASE(TT, WW, SS) \
     if (L.tokens == TT && shape.waves == WW && shape.stages == SS) \
         return md == 16 ? launch_shape<TT, WW, SS, 16>(L, stream) : launch_shape<TT, WW, SS, 32>(L, stream)

@@ -52,7 +52,13 @@ __device__ __forceinline__ Q4Job dot16_find_job(const Q4DotLaunch &L, int wg) {
 // T tokens (1..4), WAVES waves of 16 rows per workgroup, MD dwords of scales per lane.  The M side of one matrix
 // instruction holds two tokens; three or four tokens take a second pair of instructions per group on the same
 // weight registers.
-template <int T, int WAVES, int MD>
+//
+// PASSES: more tokens than fit beside the weight steps in LDS run as passes of T tokens inside ONE launch.
+// Workgroups are numbered so that the passes over one block of rows are eight apart: the dispatcher deals
+// consecutive workgroups round the device's eight partitions, so those land on one partition at about the same time
+// and every pass after the first finds its weights in that partition's cache (the loads then carry the default
+// cache policy instead of the non-temporal one).  The last pass may hold fewer than T tokens.
+template <int T, int WAVES, int MD, bool PASSES = false>
 __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch L) {
     static_assert(T >= 1 && T <= 4 && (MD == 16 || MD == 32), "tokens per pass, scale registers");
     constexpr int SETS = (T + 1) / 2;                // pairs of tokens
@@ -62,22 +68,33 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const Q4Job job = dot16_find_job(L, blockIdx.x);
+    int wg = blockIdx.x, pass = 0;
+    if (PASSES) {
+        const int round = 8 * L.passes, within = wg % round;
+        pass = within >> 3;
+        wg = (wg / round) * 8 + (within & 7);
+        if (wg >= L.total_wgs) return;               // the padding of the last round
+    }
+    const int tokens_here = PASSES ? (L.tokens_total - pass * T < T ? L.tokens_total - pass * T : T) : T;
+    const Q4Job job = dot16_find_job(L, wg);
+    const float *const xs = job.x + (size_t)pass * T * job.x_stride;
+    float *const ys = job.y + (size_t)pass * T * job.y_stride;
 
-    Dot16Stream<MD> stream;
+    Dot16Stream<MD, PASSES ? 0 : STREAMING> stream;
     stream.setup(lane, L.cols, lds + (size_t)wave * WAVE16_LDS);
     const int SG = stream.SG;
     uint8_t *const zero_lds = lds + WAVES * WAVE16_LDS;
     uint8_t *const img_lds = zero_lds + ZERO_BYTES;                        // [T][2 * SG][GROUP_IMAGE]
     float *const xm_lds = (float *)(img_lds + (size_t)T * 2 * SG * GROUP_IMAGE);
 
-    const int row_base = (((int)blockIdx.x - job.tile0) * WAVES + wave) * ROWS16;
+    const int row_base = ((wg - job.tile0) * WAVES + wave) * ROWS16;
     const bool has_rows = row_base < job.rows;       // a wave without rows still helps with the activations
     stream.bind(job.vals, job.scales, job.biases, job.rows, has_rows ? row_base : 0, 0, has_rows ? stream.nstage : 0);
     if (has_rows) stream.start();
 
     build_q4_image<T, THREADS>(tid, stream.ngrp, SG, zero_lds, img_lds, xm_lds, T, [&](int t, size_t column, float (&xv)[8]) {
-        const float *src = job.x + (size_t)t * job.x_stride + column;
+        // a token past the last pass's end repeats the last real one (its results are not stored)
+        const float *src = xs + (size_t)(t < tokens_here ? t : tokens_here - 1) * job.x_stride + column;
 #pragma unroll
         for (int k = 0; k < 8; ++k) xv[k] = src[k];
     });
@@ -102,8 +119,8 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch 
     for (int s = 0; s < SETS; ++s) {
         const float other = __shfl_xor(acc[s], 16, 64);
         const int token = 2 * s + my_token;
-        if (token < T && stream.my_strip == 0 && stream.n < stream.rows_here)
-            job.y[(size_t)token * job.y_stride + row_base + stream.n] = acc[s] + other;
+        if (token < tokens_here && stream.my_strip == 0 && stream.n < stream.rows_here)
+            ys[(size_t)token * job.y_stride + row_base + stream.n] = acc[s] + other;
     }
 }
 
@@ -112,18 +129,24 @@ size_t dot16_lds_bytes(int cols, int tokens, int waves) {
     return (size_t)waves * WAVE16_LDS + ZERO_BYTES + (size_t)tokens * 2 * sg * (GROUP_IMAGE + 8);
 }
 
-template <int T, int WAVES, int MD>
+template <int T, int WAVES, int MD, bool PASSES>
 int launch16(const Q4DotLaunch &L, hipStream_t stream) {
     const size_t lds = dot16_lds_bytes(L.cols, T, WAVES);
     static size_t raised = 0;
     if (lds > raised) {
-        if (hipFuncSetAttribute((const void *)q4_dot16_kernel<T, WAVES, MD>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        if (hipFuncSetAttribute((const void *)q4_dot16_kernel<T, WAVES, MD, PASSES>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)lds) != hipSuccess)
             return -1;
         raised = lds;
     }
-    note_kernel("q4_dot16_kernel<%d,%d,%d>", T, WAVES, MD);
-    hipLaunchKernelGGL((q4_dot16_kernel<T, WAVES, MD>), dim3(L.total_wgs), dim3(WAVES * 64), lds, stream, L);
+    unsigned grid = (unsigned)L.total_wgs;
+    if (PASSES) {
+        note_kernel("q4_dot16_kernel<%d,%d,%d> x %d passes", T, WAVES, MD, L.passes);
+        grid = (unsigned)((L.total_wgs + 7) / 8) * 8u * (unsigned)L.passes;
+    } else {
+        note_kernel("q4_dot16_kernel<%d,%d,%d>", T, WAVES, MD);
+    }
+    hipLaunchKernelGGL((q4_dot16_kernel<T, WAVES, MD, PASSES>), dim3(grid), dim3(WAVES * 64), lds, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -136,6 +159,7 @@ int q4_dot16_waves(int cols, int tokens, long long total_blocks32) {
     if (total_blocks32 < 2048) return 0;                                // few blocks: the 32-row kernel cuts rows instead
     if (2 * dot16_lds_bytes(cols, tokens, 8) <= DOT_LDS_LIMIT) return 8;
     if (dot16_lds_bytes(cols, tokens, 12) <= DOT_LDS_LIMIT) return 12;
+    if (dot16_lds_bytes(cols, tokens, 8) <= DOT_LDS_LIMIT) return 8;    // much activation image: one workgroup of eight
     return 0;
 }
 
@@ -143,12 +167,27 @@ int q4_dot16_launch(const Q4DotLaunch &L, int waves, hipStream_t stream) {
     if (L.total_wgs < 1 || L.tokens < 1 || L.tokens > 4 || !q4_dot_takes(L.cols)) return -1;
     if (dot16_lds_bytes(L.cols, L.tokens, waves) > DOT_LDS_LIMIT) return -1;
     const int md = dot_steps(L.cols >> 6) * STAGE_GROUPS <= 32 ? 16 : 32;
+    if (L.passes > 1) {
+        if (L.tokens_total <= (L.passes - 1) * L.tokens || L.tokens_total > L.passes * L.tokens) return -1;
+#define DOT16_PASSES(TT, WW) \
+        if (L.tokens == TT && waves == WW) \
+            return md == 16 ? launch16<TT, WW, 16, true>(L, stream) : launch16<TT, WW, 32, true>(L, stream)
+        DOT16_PASSES(2, 8); DOT16_PASSES(4, 8); DOT16_PASSES(4, 12);
+#undef DOT16_PASSES
+        return -1;
+    }
 #define DOT16_CASE(TT, WW) \
-    if (L.tokens == TT && waves == WW) return md == 16 ? launch16<TT, WW, 16>(L, stream) : launch16<TT, WW, 32>(L, stream)
+    if (L.tokens == TT && waves == WW) \
+        return md == 16 ? launch16<TT, WW, 16, false>(L, stream) : launch16<TT, WW, 32, false>(L, stream)
     DOT16_CASE(1, 8); DOT16_CASE(2, 8); DOT16_CASE(3, 8); DOT16_CASE(4, 8);
     DOT16_CASE(1, 12); DOT16_CASE(2, 12); DOT16_CASE(3, 12); DOT16_CASE(4, 12);
 #undef DOT16_CASE
     return -1;
+}
+
+// Whether q4_dot16_launch serves `passes` passes of `tokens` tokens with `waves` waves per workgroup.
+bool q4_dot16_takes_passes(int tokens, int waves) {
+    return (tokens == 2 && waves == 8) || (tokens == 4 && (waves == 8 || waves == 12));
 }
 
 }  // namespace mi355

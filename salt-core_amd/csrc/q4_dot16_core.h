@@ -44,7 +44,8 @@ __device__ __forceinline__ Dot16Operand dot16_operand(int lane, int token_of_pai
     return op;
 }
 
-template <int MD>
+// POLICY: cache policy of the weight loads (STREAMING = non-temporal: every byte is read once by this launch).
+template <int MD, int POLICY = STREAMING>
 struct Dot16Stream {
     // what the wave walks
     const uint8_t *vals, *scales, *biases;       // biases may be null
@@ -117,7 +118,7 @@ struct Dot16Stream {
 #pragma unroll
             for (int k = 0; k < LOADS16; ++k)
                 __builtin_amdgcn_global_load_lds((global_u128_ptr)(uintptr_t)(block_vals + advance + src_off[k]),
-                                                 (lds_void_ptr)(stage + k * 1024), 16, 0, STREAMING);
+                                                 (lds_void_ptr)(stage + k * 1024), 16, 0, POLICY);
         } else {
             // the matrix ends inside this block, or strip 1 ends inside this step or before it: stay inside
 #pragma unroll
@@ -126,7 +127,7 @@ struct Dot16Stream {
                 uint32_t col = src_col[k] + advance;
                 col = col <= row_bytes - 16 ? col : row_bytes - 16;
                 __builtin_amdgcn_global_load_lds((global_u128_ptr)(uintptr_t)(block_vals + ((uint32_t)row * row_bytes + col)),
-                                                 (lds_void_ptr)(stage + k * 1024), 16, 0, STREAMING);
+                                                 (lds_void_ptr)(stage + k * 1024), 16, 0, POLICY);
             }
         }
     }

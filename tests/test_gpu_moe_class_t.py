@@ -56,7 +56,7 @@ def error_ratios(pool, H, F, x, sel, w, eo, y, want_eo, want_y):
 PLAN = {(128, 8, 2816, 704): "moe16_gate_up_kernel<3,4> + moe16_down_sum_kernel<4>",
         (16, 8, 2816, 704): "moe16_gate_up_kernel<3,4> + moe16_down_sum_kernel<4>",
         (8, 3, 512, 512): "moe16_gate_up_kernel<1,4> + moe16_down_sum_kernel<4>",
-        (200, 1, 1024, 640): "q4_dot_kernel<1,4,2,16,2,1> ksplit 2",
+        (200, 1, 1024, 640): "q4_dot_kernel<1,4,2,16,2> ksplit 2",
         (64, 4, 4096, 2048): "moe16_gate_up_kernel<3,8> + moe16_down_sum_kernel<8>",
         (32, 2, 1536, 2560): "moe16_gate_up_kernel<3,4> + moe16_down_sum_kernel<16>",
         (8, 2, 6272, 512): "moe16_gate_up_kernel<3,16> + moe16_down_sum_kernel<4>"}

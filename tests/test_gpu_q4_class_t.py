@@ -164,23 +164,26 @@ def run_jobs(pkg, Cc, tokens, rows, weights, seed):
 
 
 # (columns, tokens, rows per job, jobs) -> the launch shape it must take.  Between them the cases reach every entry
-# of the 32-row kernel's candidate list, every cut of the rows (1, 2, 4, 8 parts), both register widths, two blocks
-# per wave, and the sixteen-row kernel at eight and at twelve waves.
+# of the 32-row kernel's candidate list, every cut of the rows (1, 2, 4, 8 parts), both register widths, and the
+# sixteen-row kernel at eight and at twelve waves, in one pass and in several.
 SHAPE_CASES = [
-    (2816, 1, 2816, 12, "q4_dot_kernel<1,4,2,16,0,1> ksplit 1"),
-    (2816, 1, 2816, 6, "q4_dot_kernel<1,4,2,16,0,1> ksplit 2"),
-    (2816, 1, 2816, 1, "q4_dot_kernel<1,4,2,16,0,1> ksplit 4"),
-    (4096, 1, 4096, 8, "q4_dot_kernel<1,3,2,16,0,1> ksplit 1"),
-    (4096, 1, 4096, 1, "q4_dot_kernel<1,8,2,16,0,1> ksplit 8"),
-    (8192, 1, 2816, 12, "q4_dot_kernel<1,7,2,32,0,1> ksplit 1"),
-    (8192, 1, 2816, 6, "q4_dot_kernel<1,6,2,16,0,1> ksplit 2"),
-    (8192, 1, 2816, 3, "q4_dot_kernel<1,4,3,16,0,1> ksplit 4"),
-    (8192, 2, 2816, 12, "q4_dot_kernel<2,4,2,32,0,1> ksplit 1"),
-    (4096, 4, 4096, 16, "q4_dot_kernel<4,4,2,16,0,2> ksplit 1"),
+    (2816, 1, 2816, 12, "q4_dot_kernel<1,4,2,16,0> ksplit 1"),
+    (2816, 1, 2816, 6, "q4_dot_kernel<1,4,2,16,0> ksplit 2"),
+    (2816, 1, 2816, 1, "q4_dot_kernel<1,4,2,16,0> ksplit 4"),
+    (4096, 1, 4096, 8, "q4_dot_kernel<1,3,2,16,0> ksplit 1"),
+    (4096, 1, 4096, 1, "q4_dot_kernel<1,8,2,16,0> ksplit 8"),
+    (8192, 1, 2816, 12, "q4_dot_kernel<1,7,2,32,0> ksplit 1"),
+    (8192, 1, 2816, 6, "q4_dot_kernel<1,6,2,16,0> ksplit 2"),
+    (8192, 1, 2816, 3, "q4_dot_kernel<1,4,3,16,0> ksplit 4"),
+    (8192, 2, 2816, 12, "q4_dot_kernel<2,4,2,32,0> ksplit 1"),
+    (4096, 4, 4096, 16, "q4_dot16_kernel<4,8,16>"),
     (2816, 1, 2816, 24, "q4_dot16_kernel<1,8,16>"),
     (2816, 2, 2816, 24, "q4_dot16_kernel<2,12,16>"),
     (8192, 1, 2816, 24, "q4_dot16_kernel<1,12,32>"),
-    (2112, 1, 2816, 2, "q4_dot_kernel<1,4,2,16,0,1> ksplit 4"),     # 33 groups: a step that straddles the row's end
+    (8192, 4, 2816, 24, "q4_dot16_kernel<2,8,32> x 2 passes"),      # more tokens than one pass holds: one launch
+    (8192, 3, 2816, 24, "q4_dot16_kernel<2,8,32> x 2 passes"),      # ... whose last pass is short
+    (2816, 7, 2816, 24, "q4_dot16_kernel<4,12,16> x 2 passes"),
+    (2112, 1, 2816, 2, "q4_dot_kernel<1,4,2,16,0> ksplit 4"),     # 33 groups: a step that straddles the row's end
     (6272, 3, 96, 1, None),                                          # 98 groups, three tokens, rows cut in 8
 ]
 
@@ -205,7 +208,7 @@ def test_the_shape_cases_cover_the_candidate_list():
                    for k in reached), (waves, stages)
     for cut in (1, 2, 4, 8):
         assert any(k.endswith(f"ksplit {cut}") for k in reached)
-    assert any(",32,0,1>" in k for k in reached) and any(",0,2>" in k for k in reached)
+    assert any(",32,0>" in k for k in reached) and any("passes" in k for k in reached)
 
 
 def test_same_launch_gives_the_same_bits(pkg):
