@@ -674,8 +674,9 @@ def main():
         extra["moe_prefill_2048_us"] = round(ms_pf * 1e3, 1)
         extra["moe_prefill_tokens_per_s"] = round(T / (ms_pf * 1e-3), 0)
         extra["moe_prefill_useful_tflops"] = round(flops / (ms_pf * 1e-3) / 1e12, 1)
-        # the activation travels as three exact bf16 planes, so the matrix cores execute three times the useful flops
-        extra["moe_prefill_mfma_frac"] = round(3 * flops / (ms_pf * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
+        # the activation travels as two exact fp16 planes, so the matrix cores execute twice the useful flops (fp16 and
+        # bf16 share the dense peak)
+        extra["moe_prefill_mfma_frac"] = round(2 * flops / (ms_pf * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
         del prefill
         # the bf16 head (262144 x 2816, the largest matrix a decode step streams) and the 8-bit router gate
         # (128 x 2816, one unsplittable 2816-step chain per row), both bit-exact

@@ -10,18 +10,22 @@
 //  * per 64-column scale group,  sum_c (q s + b) x = s * sum_c q x + b * sum_c x.
 //    The integer codes are exact in bf16, so only sum_c q x goes through MFMA
 //    per group; the scale is applied per group in fp32 on the VALU.
-//  * a nibble becomes the bf16 value 16 + q with two bit operations per pair
-//    ((w >> n) & 0x00780078 | 0x41804180); the surplus 16 * s * sum_c x joins
+//  * a nibble becomes the fp16 value 16 + q with two bit operations per pair
+//    ((w shifted) & 0x03C003C0 | 0x4C004C00); the surplus 16 * s * sum_c x joins
 //    the bias term.
+//  * the activation row is scaled by a power of two that puts its largest
+//    magnitude in [2^13, 2^14) and split into two fp16 planes, x * 2^k = hi + lo
+//    (each rounded to nearest: 23 significant bits, |x 2^k - hi - lo| <= 2^-22
+//    of the element's own magnitude, or 2^-25 of the scaled row for elements so
+//    small that lo is subnormal); each plane is an exact MFMA operand,
+//    accumulation is fp32, and the power of two leaves with the store.
 //  * the bias term sum_g (b_g - 16 s_g) * X_g (X_g = the group sums of x) is
 //    itself a small contraction over the groups; b and s are bf16, so it runs
-//    on the matrix cores once per tile before the main loop.
-//  * every fp32 operand (x, X_g) is split into three bf16 planes
-//    (v = hi + mid + lo to 2^-24), each an exact MFMA operand; accumulation is
-//    fp32.
+//    on the matrix cores once per tile before the main loop, with X_g split
+//    into three bf16 planes (v = hi + mid + lo to 2^-24).
 //
 // Tiling: a workgroup of four waves computes 64 tokens x 128 weight rows, each
-// wave 32 tokens x 64 rows as two 32 x 32 blocks of v_mfma_f32_32x32x16_bf16
+// wave 32 tokens x 64 rows as two 32 x 32 blocks of v_mfma_f32_32x32x16_f16
 // that share the token operand (tokens are the M rows, weight rows the N
 // columns, so a lane owns one weight row per block and needs one scale per
 // group).  Per group the planes, the packed codes and the scales are staged in
@@ -39,6 +43,8 @@ namespace mi355 {
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+constexpr int X_PLANES = 2;                // fp16 planes of the scaled activation
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef const uint64_t __attribute__((address_space(4))) *uniform_u64_ptr;
@@ -47,9 +53,9 @@ typedef const uint16_t __attribute__((address_space(1))) *global_u16_ptr;
 typedef const float __attribute__((address_space(1))) *global_f32_ptr;
 
 constexpr int TM = MFMA_TM;                 // tokens per workgroup; weight rows per workgroup: 64 * NBW
-constexpr int X_PITCH = 144;               // bytes per staged token row of one plane: 64 bf16 + 16 pad
+constexpr int X_PITCH = 144;               // bytes per staged token row of one plane: 64 halves + 16 pad
 constexpr int W_PITCH = 36;                // bytes per staged weight row of one group: 32 + 4 pad
-constexpr int XS_BYTES = 3 * TM * X_PITCH;
+constexpr int XS_BYTES = X_PLANES * TM * X_PITCH;
 constexpr int G_PITCH = 48;                // bias pass: bytes per staged row of 16 bf16: 32 + 16 pad
 constexpr int XG_BYTES = 3 * TM * G_PITCH;
 
@@ -89,7 +95,7 @@ __device__ __forceinline__ MfmaJob find_job(const MfmaLaunch &L, int tile) {
 
 __device__ __forceinline__ float bf16_to_f32(uint32_t half) { return __uint_as_float(half << 16); }
 
-// Eight nibbles -> eight bf16 values 16 + q, in the column order 0,4,1,5,2,6,3,7.
+// Eight nibbles -> eight fp16 values 16 + q, in the column order 0,4,1,5,2,6,3,7.
 // (a & mask) | bits in one instruction; the three-operand form takes no
 // literals, so the mask travels in a scalar register and the bits in a vector one.
 __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t bits) {
@@ -98,13 +104,18 @@ __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t b
     return r;
 }
 
-__device__ __forceinline__ bf16x8 codes_to_bf16(uint32_t w, uint32_t mask, uint32_t sixteen) {
-    u32x4 r;
-    r.x = and_or((w << 3), mask, sixteen);               // columns 0 and 4
-    r.y = and_or((w >> 1), mask, sixteen);               // 1 and 5
-    r.z = and_or((w >> 5), mask, sixteen);               // 2 and 6
-    r.w = and_or((w >> 9), mask, sixteen);               // 3 and 7
-    return __builtin_bit_cast(bf16x8, r);
+__device__ __forceinline__ f16x8 codes_to_f16(uint32_t w, uint32_t mask, uint32_t sixteen) {
+    u32x4 r;                                             // a code's four bits land on mantissa bits 6..9 of 16.0
+    r.x = and_or((w << 6), mask, sixteen);               // columns 0 and 4
+    r.y = and_or((w << 2), mask, sixteen);               // 1 and 5
+    r.z = and_or((w >> 2), mask, sixteen);               // 2 and 6
+    r.w = and_or((w >> 6), mask, sixteen);               // 3 and 7
+    return __builtin_bit_cast(f16x8, r);
+}
+
+// 2^-k <-> 2^k for a float that is a power of two (normal range)
+__device__ __forceinline__ float reciprocal_power_of_two(float p) {
+    return __uint_as_float((254u - ((__float_as_uint(p) >> 23) & 0xffu)) << 23);
 }
 
 __device__ __forceinline__ uint32_t f32_to_bf16_rne(float v) {
@@ -127,20 +138,20 @@ __device__ __forceinline__ void group_product(const uint8_t *cur, int wm, int wn
                                               f32x16 (&acc)[NBW]) {
     using S = Stage<64 * NBW>;
     const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    uint32_t sixteen;                                   // two bf16 values 16.0, kept in a vector register
-    asm("v_mov_b32 %0, 0x41804180" : "=v"(sixteen));
+    uint32_t sixteen;                                   // two fp16 values 16.0, kept in a vector register
+    asm("v_mov_b32 %0, 0x4C004C00" : "=v"(sixteen));
     const uint8_t *wrow = cur + S::WS_OFF + (wn * 32 * NBW + l32) * W_PITCH + half * 4;
     const uint8_t *xrow = cur + (wm * 32 + l32) * X_PITCH + half * 16;
     const float *sc = reinterpret_cast<const float *>(cur + S::SC_OFF) + wn * 32 * NBW + l32;
     // The token operand of the whole group stays in registers; the row blocks
     // then run two at a time so that only two partial products are live.
-    bf16x8 a[4][3];
+    f16x8 a[4][X_PLANES];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-        for (int plane = 0; plane < 3; ++plane)
+        for (int plane = 0; plane < X_PLANES; ++plane)
             a[ks][plane] = __builtin_bit_cast(
-                bf16x8, *reinterpret_cast<const u32x4 *>(xrow + plane * (TM * X_PITCH) + ks * 32));
+                f16x8, *reinterpret_cast<const u32x4 *>(xrow + plane * (TM * X_PITCH) + ks * 32));
 #pragma unroll
     for (int nb0 = 0; nb0 < NB; nb0 += 2) {
         constexpr int PAIR_MAX = 2;
@@ -148,19 +159,19 @@ __device__ __forceinline__ void group_product(const uint8_t *cur, int wm, int wn
         f32x16 part[PAIR_MAX];
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-            bf16x8 b[PAIR_MAX];
+            f16x8 b[PAIR_MAX];
 #pragma unroll
             for (int k = 0; k < PAIR_MAX; ++k)
                 if (k < pair)
-                    b[k] = codes_to_bf16(*reinterpret_cast<const uint32_t *>(wrow + (nb0 + k) * 32 * W_PITCH + ks * 8),
-                                         0x00780078u, sixteen);
+                    b[k] = codes_to_f16(*reinterpret_cast<const uint32_t *>(wrow + (nb0 + k) * 32 * W_PITCH + ks * 8),
+                                        0x03C003C0u, sixteen);
 #pragma unroll
-            for (int plane = 0; plane < 3; ++plane)
+            for (int plane = 0; plane < X_PLANES; ++plane)
 #pragma unroll
                 for (int k = 0; k < PAIR_MAX; ++k)
                     if (k < pair)
-                        part[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks][plane], b[k],
-                                                                          (ks | plane) ? part[k] : zero, 0, 0, 0);
+                        part[k] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ks][plane], b[k],
+                                                                         (ks | plane) ? part[k] : zero, 0, 0, 0);
         }
 #pragma unroll
         for (int k = 0; k < PAIR_MAX; ++k)
@@ -179,7 +190,7 @@ void q4_mfma_kernel(const MfmaLaunch L) {
     constexpr int TN = 64 * NBW;
     using S = Stage<TN>;
     constexpr int STAGE_BYTES = S::BYTES;
-    // two stages of { planes [3][64 tokens], codes [TN rows], scales [TN] }
+    // two stages of { planes [2][64 tokens], codes [TN rows], scales [TN] }
     __shared__ __attribute__((aligned(16))) uint8_t stage[2 * STAGE_BYTES];
 
     const int tid = threadIdx.x;
@@ -208,11 +219,12 @@ void q4_mfma_kernel(const MfmaLaunch L) {
     };
 
     // staging geometry of this thread
-    // planes: 3 * 64 tokens * 8 segments of 16 bytes = 1536 pieces, 6 per thread
+    // planes: 2 * 64 tokens * 8 segments of 16 bytes = 1024 pieces, 4 per thread
+    constexpr int XP = X_PLANES * TM * 8 / 256;
     const global_u16_ptr planes = (global_u16_ptr)(uintptr_t)job.planes;
-    uint32_t x_src[6], x_dst[6];                    // element offsets: the planes of one launch stay below 2^32 elements
+    uint32_t x_src[XP], x_dst[XP];                  // element offsets: the planes of one launch stay below 2^32 elements
 #pragma unroll
-    for (int i = 0; i < 6; ++i) {
+    for (int i = 0; i < XP; ++i) {
         const int p = tid + i * 256;
         const int plane = p >> 9, tok = (p >> 3) & 63, seg = p & 7;
         x_src[i] = (uint32_t)plane * (uint32_t)L.plane_stride + source_row(tok) * (uint32_t)C + seg * 8;
@@ -237,17 +249,17 @@ void q4_mfma_kernel(const MfmaLaunch L) {
 
     // Loads travel through registers; two sets are in flight so that a load has
     // two groups of matrix work (of both workgroups on the compute unit) to land.
-    struct Loads { u32x4 x[6], w[WP]; uint32_t s; };
+    struct Loads { u32x4 x[XP], w[WP]; uint32_t s; };
     auto issue = [&](int g, Loads &r) {
 #pragma unroll
-        for (int i = 0; i < 6; ++i) r.x[i] = *(global_u128_ptr)(planes + x_src[i] + (uint32_t)g * 64u);
+        for (int i = 0; i < XP; ++i) r.x[i] = *(global_u128_ptr)(planes + x_src[i] + (uint32_t)g * 64u);
 #pragma unroll
         for (int i = 0; i < WP; ++i) r.w[i] = w_src[i][g * 2];
         if (tid < TN) r.s = scales[g];
     };
     auto commit = [&](uint8_t *base, const Loads &r) {
 #pragma unroll
-        for (int i = 0; i < 6; ++i) *reinterpret_cast<u32x4 *>(base + x_dst[i]) = r.x[i];
+        for (int i = 0; i < XP; ++i) *reinterpret_cast<u32x4 *>(base + x_dst[i]) = r.x[i];
 #pragma unroll
         for (int i = 0; i < WP; ++i) {
             uint32_t *dst = reinterpret_cast<uint32_t *>(base + w_dst[i]);
@@ -329,7 +341,21 @@ void q4_mfma_kernel(const MfmaLaunch L) {
         __syncthreads();
     }
 
-    // ---- main loop: acc += s[row][g] * sum_{c in g} (16 + q[row][c]) * x[tok][c]
+    // The main loop works on x * 2^k (k per token, chosen by the split): the bias term joins it at that scale and
+    // the power of two leaves at the store.  A token's 2^-k lies at the head of its row of the third plane.
+    auto token_scale = [&](int i) -> float {
+        const int tok = wm * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
+        return *(const float __attribute__((address_space(1))) *)(uintptr_t)(
+            job.planes + 2 * (size_t)L.plane_stride + (size_t)source_row(tok) * (size_t)C);
+    };
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const float up = reciprocal_power_of_two(token_scale(i));
+#pragma unroll
+        for (int nb = 0; nb < NBW; ++nb) acc[nb][i] = acc[nb][i] * up;
+    }
+
+    // ---- main loop: acc += s[row][g] * sum_{c in g} (16 + q[row][c]) * x[tok][c] * 2^k
     // Row blocks past the end of the matrix are computed on clamped rows and
     // dropped at the store: one instantiation of the loop keeps the
     // accumulators in place and the register count inside the budget.
@@ -355,6 +381,9 @@ void q4_mfma_kernel(const MfmaLaunch L) {
     }
 
     float __attribute__((address_space(1))) *y = (float __attribute__((address_space(1))) *)(uintptr_t)job.y;
+    float down[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) down[i] = token_scale(i);
 #pragma unroll
     for (int nb = 0; nb < NBW; ++nb) {
         const int row = wn * 32 * NBW + nb * 32 + l32;
@@ -362,62 +391,97 @@ void q4_mfma_kernel(const MfmaLaunch L) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int tok = wm * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
-                if (tok < toks_here) y[(size_t)(tok0 + tok) * job.rows + row0 + row] = acc[nb][i];
+                if (tok < toks_here) y[(size_t)(tok0 + tok) * job.rows + row0 + row] = acc[nb][i] * down[i];
             }
         }
     }
 }
 
-// fp32 rows -> three bf16 planes (columns permuted inside every run of eight,
-// see the top of the file) and per-64-column sums.  Row r of the output is row
-// row_map[r] / map_divisor of the input when a map is given (the grouped MoE
-// gather).
-// With GATED the value split is gelu_tanh(gate) * x (the expert activation,
-// reference gemma4_text.c:8749-9137 "down input"), so the activations never
-// make a round trip through memory in fp32.
+// fp32 rows -> two fp16 planes of the row scaled by a power of two (columns permuted inside every run of eight, see
+// the top of the file), the row's 2^-k at the head of its row of a third plane, and the per-64-column sums of the
+// unscaled values.  Row r of the output is row row_map[r] / map_divisor of the input when a map is given (the
+// grouped MoE gather).  One workgroup per row: the scale needs the row's largest magnitude.
+// With GATED the value split is gelu_tanh(gate) * x (the expert activation, reference gemma4_text.c:8749-9137
+// "down input"), so the activations never make a round trip through memory in fp32.
+constexpr int SPLIT_MAX_ITEMS = 4;          // eight columns per item and thread: rows of up to 8192 columns
+
 template <bool GATED>
 __global__ __launch_bounds__(256) void x_split_kernel(const float *__restrict__ x, const float *__restrict__ gate,
                                                       const int *__restrict__ row_map, int map_divisor, int x_stride,
                                                       int rows, int cols, uint16_t *__restrict__ planes,
                                                       size_t plane_stride, float *__restrict__ xsum) {
+    __shared__ uint32_t wave_top[4];
     const int row = blockIdx.x;
-    const int c0 = (blockIdx.y * 256 + threadIdx.x) * 8;
-    const bool live = c0 < cols;
-    float v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (live) {
-        const int src_row = row_map ? row_map[row] / map_divisor : row;
-        const float4 *src = reinterpret_cast<const float4 *>(x + (size_t)src_row * x_stride + c0);
-        const float4 a = src[0], b = src[1];
-        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-        if (GATED) {
-            const float4 *gsrc = reinterpret_cast<const float4 *>(gate + (size_t)src_row * x_stride + c0);
-            const float4 ga = gsrc[0], gb = gsrc[1];
-            const float gv[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
+    const int src_row = row_map ? row_map[row] / map_divisor : row;
+    float v[SPLIT_MAX_ITEMS][8];
+    uint32_t top = 0u;                              // largest magnitude as a bit pattern: a NaN or an infinity wins it
 #pragma unroll
-            for (int j = 0; j < 8; ++j) v[j] = det_gelu_tanh(gv[j]) * v[j];
+    for (int it = 0; it < SPLIT_MAX_ITEMS; ++it) {
+        const int c0 = (it * 256 + (int)threadIdx.x) * 8;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[it][j] = 0.0f;
+        if (c0 < cols) {
+            const float4 *src = reinterpret_cast<const float4 *>(x + (size_t)src_row * x_stride + c0);
+            const float4 a = src[0], b = src[1];
+            v[it][0] = a.x; v[it][1] = a.y; v[it][2] = a.z; v[it][3] = a.w;
+            v[it][4] = b.x; v[it][5] = b.y; v[it][6] = b.z; v[it][7] = b.w;
+            if (GATED) {
+                const float4 *gsrc = reinterpret_cast<const float4 *>(gate + (size_t)src_row * x_stride + c0);
+                const float4 ga = gsrc[0], gb = gsrc[1];
+                const float gv[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[it][j] = det_gelu_tanh(gv[j]) * v[it][j];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const uint32_t mag = __float_as_uint(v[it][j]) & 0x7fffffffu;
+                top = top > mag ? top : mag;
+            }
         }
     }
-    uint32_t hi[4], mid[4], lo[4];
-    float sum = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        uint32_t h, m, l;
-        split3(v[j], h, m, l);
-        const int k = j & 3;                           // dword k holds columns k (low half) and k + 4 (high half)
-        if (j & 4) { hi[k] |= h << 16; mid[k] |= m << 16; lo[k] |= l << 16; }
-        else { hi[k] = h; mid[k] = m; lo[k] = l; }
-        sum += v[j];
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t other = (uint32_t)__shfl_xor((int)top, d, 64);
+        top = top > other ? top : other;
     }
-    // eight lanes cover one 64-column group
-    sum += __shfl_xor(sum, 1, 64);
-    sum += __shfl_xor(sum, 2, 64);
-    sum += __shfl_xor(sum, 4, 64);
-    if (live) {
-        uint16_t *dst = planes + (size_t)row * cols + c0;
-        *reinterpret_cast<uint4 *>(dst) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-        *reinterpret_cast<uint4 *>(dst + plane_stride) = make_uint4(mid[0], mid[1], mid[2], mid[3]);
-        *reinterpret_cast<uint4 *>(dst + 2 * plane_stride) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-        if ((threadIdx.x & 7) == 0) xsum[(size_t)row * (cols >> 6) + (c0 >> 6)] = sum;
+    if ((threadIdx.x & 63) == 0) wave_top[threadIdx.x >> 6] = top;
+    __syncthreads();
+    top = wave_top[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) top = top > wave_top[w] ? top : wave_top[w];
+    // top in [2^E, 2^(E+1)) -> x * 2^(13 - E) in [2^13, 2^14); rows of zeros or tiny values are pinned
+    int eb = (int)(top >> 23);
+    eb = eb < 14 ? 14 : (eb > 253 ? 253 : eb);
+    const float up = __uint_as_float((uint32_t)(267 - eb) << 23);          // 2^(13 - E)
+    const float down = __uint_as_float((uint32_t)(eb - 13) << 23);         // 2^(E - 13)
+    if (threadIdx.x == 0) *reinterpret_cast<float *>(planes + 2 * plane_stride + (size_t)row * cols) = down;
+#pragma unroll
+    for (int it = 0; it < SPLIT_MAX_ITEMS; ++it) {
+        const int c0 = (it * 256 + (int)threadIdx.x) * 8;
+        const bool live = c0 < cols;
+        uint32_t hi[4], lo[4];
+        float sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float scaled = v[it][j] * up;
+            const _Float16 h = (_Float16)scaled;
+            const _Float16 l = (_Float16)(scaled - (float)h);
+            const uint32_t hb = __builtin_bit_cast(uint16_t, h), lb = __builtin_bit_cast(uint16_t, l);
+            const int k = j & 3;                           // dword k holds columns k (low half) and k + 4 (high half)
+            if (j & 4) { hi[k] |= hb << 16; lo[k] |= lb << 16; }
+            else { hi[k] = hb; lo[k] = lb; }
+            sum += v[it][j];
+        }
+        // eight lanes cover one 64-column group
+        sum += __shfl_xor(sum, 1, 64);
+        sum += __shfl_xor(sum, 2, 64);
+        sum += __shfl_xor(sum, 4, 64);
+        if (live) {
+            uint16_t *dst = planes + (size_t)row * cols + c0;
+            *reinterpret_cast<uint4 *>(dst) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+            *reinterpret_cast<uint4 *>(dst + plane_stride) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+            if ((threadIdx.x & 7) == 0) xsum[(size_t)row * (cols >> 6) + (c0 >> 6)] = sum;
+        }
     }
 }
 
@@ -456,8 +520,8 @@ int q4_mfma_launch(const MfmaLaunch &launch, hipStream_t stream) {
 
 int x_split_launch(const float *x, const float *gate, const int *row_map, int map_divisor, int x_stride, int rows,
                    int cols, uint16_t *planes, size_t plane_stride, float *xsum, hipStream_t stream) {
-    if (rows < 1 || cols < 64 || (cols & 63)) return -1;
-    const dim3 grid(rows, (cols / 8 + 255) / 256);
+    if (rows < 1 || cols < 64 || (cols & 63) || cols > SPLIT_MAX_ITEMS * 256 * 8) return -1;
+    const dim3 grid(rows);
     if (gate)
         hipLaunchKernelGGL(x_split_kernel<true>, grid, dim3(256), 0, stream, x, gate, row_map, map_divisor, x_stride,
                            rows, cols, planes, plane_stride, xsum);
