@@ -19,7 +19,7 @@ reference's own C kernel when oracle/_ref is present (else the checker's
 port), and, under "extra", the same sweep on the bit-exact kernel, the MoE
 decode layer-step, the NVFP4 matvec and the batch-4 sweeps.
 
---only NAME runs a single leg (sweep, sweep-exact, sweep-b4, moe, moe-t, nvfp4-t, copy): what the
+--only NAME runs a single leg (sweep, sweep-exact, sweep-b4, single, single-exact, moe, moe-t, prefill, nvfp4-t, copy): what the
 rocprofv3 commands in profiles/ use.
 """
 from __future__ import annotations
@@ -358,6 +358,18 @@ def moe_leg(gpu, synth, lib, stream, events, pool, tolerance_class):
            tag + "_gbps": round(step_bytes / (ms_moe * 1e-3) / 1e9, 1),
            tag + "_hbm_frac": round(step_bytes / (ms_moe * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     out["moe_layer_tokens_per_s_class_t" if tolerance_class else "moe_layer_tokens_per_s"] = round(1e3 / ms_moe, 1)
+    # the same 64 steps (32 logit vectors x 2 layers) captured once and replayed as one HIP graph: what an engine that
+    # captures a token's layers would see of the launch boundaries
+    if lib.salt_mi355_graph_begin(stream) == 0:
+        turn[0] = 0
+        for _ in range(len(logit_sets[0])):
+            moe_step(stream)
+        graph = lib.salt_mi355_graph_end(stream)
+        if graph:
+            steps_in_graph = len(logit_sets[0]) * len(layers)
+            ms_g = timed(lib, stream, events, lambda st: lib.salt_mi355_graph_launch(graph, st), 2, 10) / steps_in_graph
+            out[tag + "_graph_us"] = round(ms_g * 1e3, 2)
+            lib.salt_mi355_graph_destroy(graph)
     return out
 
 
@@ -390,6 +402,27 @@ def nvfp4_class_t_leg(gpu, synth, lib, stream, events, w, per, packed_bytes, x, 
             "nvfp4_class_t_kernel": lib.salt_mi355_last_kernel().decode()}
 
 
+def prefill_leg(gpu, synth, lib, stream, events, pool):
+    """MoE prefill, 2048 tokens through one layer (E = 128, top-8, Zipf 1.1), grouped per expert, matrix cores."""
+    E, K, H, F, T = 128, 8, 2816, 704, 2048
+    sel, wts = synth.zipf_selection(T, E, K, 1.1, 60)
+    prefill = gpu.MoePrefill(pool, E, H, F, K, T)
+    prefill.sel.upload(sel); prefill.w.upload(wts); prefill.x.upload(synth.activations(H, T, 61))
+
+    def prefill_step(s):
+        if prefill.enqueue(s) != 0:
+            raise RuntimeError(lib.salt_mi355_last_error().decode())
+
+    ms_pf = timed(lib, stream, events, prefill_step, 2, 10)
+    flops = 2.0 * T * K * 3 * H * F                       # useful: one pass over the weights per routed row
+    # the activation travels as two exact fp16 planes, so the matrix cores execute twice the useful flops (fp16 and
+    # bf16 share the dense peak)
+    return {"moe_prefill_2048_us": round(ms_pf * 1e3, 1),
+            "moe_prefill_tokens_per_s": round(T / (ms_pf * 1e-3), 0),
+            "moe_prefill_useful_tflops": round(flops / (ms_pf * 1e-3) / 1e12, 1),
+            "moe_prefill_mfma_frac": round(2 * flops / (ms_pf * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+
+
 def run_only(args, gpu, synth, lib, stream, events):
     """One leg on its own, for profiler runs: the kernels of that leg are the only matvec kernels in the trace."""
     if args.only == "copy":
@@ -401,6 +434,17 @@ def run_only(args, gpu, synth, lib, stream, events):
     if args.only in ("moe", "moe-t"):
         pool = synth.expert_pool(128, 2816, 704, 7)
         return moe_leg(gpu, synth, lib, stream, events, pool, args.only == "moe-t")
+    if args.only == "prefill":
+        return prefill_leg(gpu, synth, lib, stream, events, synth.expert_pool(128, 2816, 704, 7))
+    if args.only in ("single", "single-exact"):
+        # every matrix of the decode sweep as a launch of its own (what the engine's salt_gpu_q4_matvec issues)
+        sweep = Q4Sweep(gpu, synth, tokens=1, exact=args.only.endswith("exact"))
+        out = {}
+        for i, (R, Cc) in enumerate(SWEEP):
+            ms_1 = timed(lib, stream, events, lambda st, i=i: sweep.single_launches(i, st), 1, 3) / sweep.launches[i][1]
+            out[f"q4_{R}x{Cc}_single_launch_us"] = round(ms_1 * 1e3, 2)
+            out[f"q4_{R}x{Cc}_kernel"] = lib.salt_mi355_last_kernel().decode()
+        return out
     if args.only == "nvfp4-t":
         R = Cc = 8192
         packed, fscales = synth.nvfp4_tensor(R, Cc, 40)
@@ -423,7 +467,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the MoE / NVFP4 / batch-4 legs")
-    ap.add_argument("--only", default="", help="run one leg: sweep | sweep-exact | sweep-b4 | sweep-b4-exact | moe | moe-t | nvfp4-t | copy")
+    ap.add_argument("--only", default="", help="run one leg: sweep | sweep-exact | sweep-b4 | sweep-b4-exact | single | single-exact | moe | moe-t | prefill | nvfp4-t | copy")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU mode (run with --gpus 1)")
@@ -659,25 +703,7 @@ def main():
                     chain_call()
                 extra["abi_q4_moe_chain_8_experts_us"] = round((time.perf_counter() - t0) / 200 * 1e6, 1)
                 eabi.salt_gpu_expert_resource_unbind(901)
-        # MoE prefill, 2048 tokens through one layer (E = 128, top-8, Zipf 1.1), grouped per expert, matrix cores
-        T = 2048
-        sel, wts = synth.zipf_selection(T, E, K, 1.1, 60)
-        prefill = gpu.MoePrefill(pool, E, H, F, K, T)
-        prefill.sel.upload(sel); prefill.w.upload(wts); prefill.x.upload(synth.activations(H, T, 61))
-
-        def prefill_step(s):
-            if prefill.enqueue(s) != 0:
-                raise RuntimeError(lib.salt_mi355_last_error().decode())
-
-        ms_pf = timed(lib, stream, events, prefill_step, 2, 10)
-        flops = 2.0 * T * K * 3 * H * F                       # useful: one pass over the weights per routed row
-        extra["moe_prefill_2048_us"] = round(ms_pf * 1e3, 1)
-        extra["moe_prefill_tokens_per_s"] = round(T / (ms_pf * 1e-3), 0)
-        extra["moe_prefill_useful_tflops"] = round(flops / (ms_pf * 1e-3) / 1e12, 1)
-        # the activation travels as two exact fp16 planes, so the matrix cores execute twice the useful flops (fp16 and
-        # bf16 share the dense peak)
-        extra["moe_prefill_mfma_frac"] = round(2 * flops / (ms_pf * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
-        del prefill
+        extra.update(prefill_leg(gpu, synth, lib, stream, events, pool))
         # the bf16 head (262144 x 2816, the largest matrix a decode step streams) and the 8-bit router gate
         # (128 x 2816, one unsplittable 2816-step chain per row), both bit-exact
         RH, CH = 262144, 2816
