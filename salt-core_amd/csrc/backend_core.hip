@@ -363,22 +363,33 @@ int salt_mi355_q4_jobs_t_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int t
                      (uint64_t)DOT_BLOCK_ROWS * (uint64_t)C / 2u < (1ull << 31);
     }
     if (!streamable) return q4_jobs_common(jobs, njobs, C, tokens, 0, false, 0, stream);
-    const int per_pass = q4_dot_tokens_per_pass(C);
+    int per_pass = q4_dot_tokens_per_pass(C);
     std::vector<Q4Job> table((size_t)njobs);
     long long blocks = 0;
     for (int j = 0; j < njobs; ++j) blocks += (jobs[j].rows + DOT_BLOCK_ROWS - 1) / DOT_BLOCK_ROWS;
+    // Rows too wide for the digit planes of three or four tokens at once: two column windows per block of rows keep
+    // it at one read of the weights per four tokens.
+    int window_waves = 0;
+    if (tokens > per_pass) {
+        const int want = tokens < 4 ? tokens : 4;
+        window_waves = q4_dot16_window_waves(C, want, blocks);
+        if (window_waves) per_pass = want;
+    }
     // More tokens than one pass holds: one launch of several passes where the sixteen-row kernel serves it (the
     // passes share the weights through the cache), else a launch per pass.
     const int passes_wanted = (tokens + per_pass - 1) / per_pass;
-    const int waves_passes = passes_wanted > 1 ? q4_dot16_waves(C, per_pass, blocks) : 0;
+    const int waves_passes = passes_wanted > 1 && !window_waves ? q4_dot16_waves(C, per_pass, blocks) : 0;
     const bool one_launch = waves_passes != 0 && q4_dot16_takes_passes(per_pass, waves_passes);
     for (int first = 0; first < tokens; first += one_launch ? tokens : per_pass) {
         const int group = one_launch ? per_pass : (tokens - first < per_pass ? tokens - first : per_pass);
         Q4DotLaunch launch;
         memset(&launch, 0, sizeof launch);
         const DotShape shape = q4_dot_shape(C, group, blocks);
-        const int waves16 = one_launch ? waves_passes : q4_dot16_waves(C, group, blocks);
+        // the last launch of a windowed job may hold one or two tokens: those fit in one window
+        const bool windowed = window_waves && group >= 3;
+        const int waves16 = one_launch ? waves_passes : windowed ? q4_dot16_window_waves(C, group, blocks) : q4_dot16_waves(C, group, blocks);
         if (one_launch) { launch.passes = passes_wanted; launch.tokens_total = tokens; }
+        if (windowed) launch.windows = 2;
         const int rows_per_wg = waves16 ? waves16 * 16 : shape.waves / shape.ksplit * shape.blocks_per_wave * DOT_BLOCK_ROWS;
         int wgs = 0;
         bool uniform = true;

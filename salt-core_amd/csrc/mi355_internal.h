@@ -107,6 +107,7 @@ struct Q4DotLaunch {
     // may hold fewer); every block of rows is walked once per pass by workgroups that the dispatcher places next
     // to each other, so that all passes but the first find the weights in the cache they share.
     int passes, tokens_total;
+    int windows;              // q4_dot16_launch only.  2: every row is walked in two column windows (q4_dot16_window_waves)
     MoeFuse moe;              // only read by q4_dot_moe_gate_up_launch / q4_dot_moe_down_launch
     // Up to Q4_INLINE_JOBS job records inside the kernel arguments (table == nullptr, njobs > 1): a decode-sized
     // batch then needs no table upload.  Must stay the last member.
@@ -121,6 +122,9 @@ int q4_dot_launch(const Q4DotLaunch &launch, const DotShape &shape, hipStream_t 
 int q4_dot16_waves(int cols, int tokens, long long total_blocks32);
 int q4_dot16_launch(const Q4DotLaunch &launch, int waves, hipStream_t stream);
 bool q4_dot16_takes_passes(int tokens_per_pass, int waves);
+// Waves per workgroup when rows too wide for all tokens' digit planes are walked in two column windows (launch.windows
+// = 2, three or four tokens), or 0 when that shape does not serve the launch.
+int q4_dot16_window_waves(int cols, int tokens, long long total_blocks32);
 // The MoE decode step's two matvec launches on the streaming kernel (router top-k in the prologue of the first,
 // gelu_tanh(gate) * up in the prologue of the second); -1: the geometry is not served.
 // The whole step in two launches (moe_dot16.hip): gate + up + activation, then down + ordered weighted sum; `out`

@@ -58,9 +58,16 @@ __device__ __forceinline__ Q4Job dot16_find_job(const Q4DotLaunch &L, int wg) {
 // consecutive workgroups round the device's eight partitions, so those land on one partition at about the same time
 // and every pass after the first finds its weights in that partition's cache (the loads then carry the default
 // cache policy instead of the non-temporal one).  The last pass may hold fewer than T tokens.
-template <int T, int WAVES, int MD, bool PASSES = false>
+//
+// WINDOWS == 2: a row too wide for the digit planes of all T tokens beside the weight steps is walked in two column
+// windows (the first dot16_window_steps(steps) steps, then the rest): the workgroup builds the planes of a window,
+// every wave walks the window's steps, and the planes of the next window replace them.  The weights are still read
+// once, by one stream per wave that runs on across the rebuild; the accumulators carry over, so the result is what
+// one window over the whole row would give.
+template <int T, int WAVES, int MD, bool PASSES = false, int WINDOWS = 1>
 __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch L) {
     static_assert(T >= 1 && T <= 4 && (MD == 16 || MD == 32), "tokens per pass, scale registers");
+    static_assert(WINDOWS == 1 || (WINDOWS == 2 && !PASSES), "windows and passes exclude each other");
     constexpr int SETS = (T + 1) / 2;                // pairs of tokens
     constexpr int THREADS = WAVES * 64;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -82,7 +89,8 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch 
 
     Dot16Stream<MD, PASSES ? 0 : STREAMING> stream;
     stream.setup(lane, L.cols, lds + (size_t)wave * WAVE16_LDS);
-    const int SG = stream.SG;
+    const int window_steps = WINDOWS == 2 ? dot16_window_steps(stream.nstage) : stream.nstage;
+    const int SG = window_steps * STAGE_GROUPS;      // group slots per strip in LDS (all of the row's: one window)
     uint8_t *const zero_lds = lds + WAVES * WAVE16_LDS;
     uint8_t *const img_lds = zero_lds + ZERO_BYTES;                        // [T][2 * SG][GROUP_IMAGE]
     float *const xm_lds = (float *)(img_lds + (size_t)T * 2 * SG * GROUP_IMAGE);
@@ -92,14 +100,23 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch 
     stream.bind(job.vals, job.scales, job.biases, job.rows, has_rows ? row_base : 0, 0, has_rows ? stream.nstage : 0);
     if (has_rows) stream.start();
 
-    build_q4_image<T, THREADS>(tid, stream.ngrp, SG, zero_lds, img_lds, xm_lds, T, [&](int t, size_t column, float (&xv)[8]) {
+    auto load_x = [&](int t, size_t column, float (&xv)[8]) {
         // a token past the last pass's end repeats the last real one (its results are not stored)
         const float *src = xs + (size_t)(t < tokens_here ? t : tokens_here - 1) * job.x_stride + column;
 #pragma unroll
         for (int k = 0; k < 8; ++k) xv[k] = src[k];
-    });
+    };
+    if (WINDOWS == 1) {
+        build_q4_image<T, THREADS>(tid, stream.ngrp, SG, zero_lds, img_lds, xm_lds, T, load_x);
+    } else {
+        for (int i = tid; i < ZERO_BYTES / 4; i += THREADS) ((uint32_t *)zero_lds)[i] = 0u;
+        Q4WindowBuilder<T, THREADS> front;
+        front.window(stream.ngrp, stream.SG, 0, SG, SG);
+        front.request(tid, load_x);
+        front.build(tid, img_lds, xm_lds, load_x);
+    }
     __syncthreads();
-    if (!has_rows) return;                           // no barrier below
+    if (WINDOWS == 1 && !has_rows) return;           // no barrier below
 
     const int my_token = lane >> 5;                  // of each pair
     Dot16Operand operand[SETS];
@@ -112,7 +129,34 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch 
         operand[s] = dot16_operand(lane, m_tok, 2 * s + m_tok < T, 2 * s + m_tok, factor_token, SG, zero_lds, img_lds, xm_lds);
         acc[s] = 0.0f;
     }
-    stream.run(operand, acc);
+    if (WINDOWS == 1) {
+        stream.run(operand, acc);
+    } else {
+        // every wave of the workgroup takes part in the rebuild, also one without rows.  Up to three tokens the
+        // second window's activations are fetched before the walk over the first; with four, holding them across
+        // the walk costs the walk more than the fetch costs the rebuild (measured: 173 against 190 us for 49
+        // matrices of 2816 x 8192).
+        constexpr bool AHEAD = T < 4;
+        Q4WindowBuilder<T, THREADS> back;
+        back.window(stream.ngrp, stream.SG, SG, (stream.nstage - window_steps) * STAGE_GROUPS, SG);
+        if (AHEAD) back.request(tid, load_x);
+        if (has_rows) {
+            stream.settle();
+            stream.walk_range(operand, acc, 0, window_steps);
+        }
+        __syncthreads();                             // nobody reads the first window any more
+        if (!AHEAD) back.request(tid, load_x);
+        back.build(tid, img_lds, xm_lds, load_x);
+        __syncthreads();
+        if (!has_rows) return;
+        // the second window's step s lies where the first window's step s - window_steps lay
+#pragma unroll
+        for (int s = 0; s < SETS; ++s) {
+            operand[s].digits -= (size_t)window_steps * operand[s].digits_step;
+            operand[s].factors -= 2 * STAGE_GROUPS * window_steps;
+        }
+        stream.walk_range(operand, acc, window_steps, stream.nstage);
+    }
 
     // the two strips of a row meet: lanes (n, 2t) and (n, 2t + 1)
 #pragma unroll
@@ -124,18 +168,19 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot16_kernel(const Q4DotLaunch 
     }
 }
 
-size_t dot16_lds_bytes(int cols, int tokens, int waves) {
-    const int sg = dot_steps(cols >> 6) * STAGE_GROUPS;
+size_t dot16_lds_bytes(int cols, int tokens, int waves, int windows = 1) {
+    const int steps = dot_steps(cols >> 6);
+    const int sg = (windows == 2 ? dot16_window_steps(steps) : steps) * STAGE_GROUPS;
     return (size_t)waves * WAVE16_LDS + ZERO_BYTES + (size_t)tokens * 2 * sg * (GROUP_IMAGE + 8);
 }
 
-template <int T, int WAVES, int MD, bool PASSES>
+template <int T, int WAVES, int MD, bool PASSES, int WINDOWS = 1>
 int launch16(const Q4DotLaunch &L, hipStream_t stream) {
-    const size_t lds = dot16_lds_bytes(L.cols, T, WAVES);
+    const size_t lds = dot16_lds_bytes(L.cols, T, WAVES, WINDOWS);
     static size_t raised = 0;
     if (lds > raised) {
-        if (hipFuncSetAttribute((const void *)q4_dot16_kernel<T, WAVES, MD, PASSES>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds) != hipSuccess)
+        if (hipFuncSetAttribute((const void *)q4_dot16_kernel<T, WAVES, MD, PASSES, WINDOWS>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
             return -1;
         raised = lds;
     }
@@ -143,10 +188,12 @@ int launch16(const Q4DotLaunch &L, hipStream_t stream) {
     if (PASSES) {
         note_kernel("q4_dot16_kernel<%d,%d,%d> x %d passes", T, WAVES, MD, L.passes);
         grid = (unsigned)((L.total_wgs + 7) / 8) * 8u * (unsigned)L.passes;
+    } else if (WINDOWS == 2) {
+        note_kernel("q4_dot16_kernel<%d,%d,%d> in 2 windows", T, WAVES, MD);
     } else {
         note_kernel("q4_dot16_kernel<%d,%d,%d>", T, WAVES, MD);
     }
-    hipLaunchKernelGGL((q4_dot16_kernel<T, WAVES, MD, PASSES>), dim3(grid), dim3(WAVES * 64), lds, stream, L);
+    hipLaunchKernelGGL((q4_dot16_kernel<T, WAVES, MD, PASSES, WINDOWS>), dim3(grid), dim3(WAVES * 64), lds, stream, L);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -163,8 +210,23 @@ int q4_dot16_waves(int cols, int tokens, long long total_blocks32) {
     return 0;
 }
 
+// Waves per workgroup for rows walked in two column windows, or 0: the digit planes of all `tokens` tokens of half a
+// row must fit beside the weight steps, and the row must have steps enough for two windows.
+int q4_dot16_window_waves(int cols, int tokens, long long total_blocks32) {
+    if (tokens < 3 || tokens > 4 || !q4_dot_takes(cols) || total_blocks32 < 2048) return 0;
+    if (dot_steps(cols >> 6) * STAGE_GROUPS <= 32) return 0;            // only the wide-row instances exist
+    if (dot16_lds_bytes(cols, tokens, 8, 2) <= DOT_LDS_LIMIT) return 8;
+    return 0;
+}
+
 int q4_dot16_launch(const Q4DotLaunch &L, int waves, hipStream_t stream) {
     if (L.total_wgs < 1 || L.tokens < 1 || L.tokens > 4 || !q4_dot_takes(L.cols)) return -1;
+    if (L.windows == 2) {
+        if (L.passes > 1 || waves != q4_dot16_window_waves(L.cols, L.tokens, 1ll << 40)) return -1;
+        if (L.tokens == 3 && waves == 8) return launch16<3, 8, 32, false, 2>(L, stream);
+        if (L.tokens == 4 && waves == 8) return launch16<4, 8, 32, false, 2>(L, stream);
+        return -1;
+    }
     if (dot16_lds_bytes(L.cols, L.tokens, waves) > DOT_LDS_LIMIT) return -1;
     const int md = dot_steps(L.cols >> 6) * STAGE_GROUPS <= 32 ? 16 : 32;
     if (L.passes > 1) {
@@ -172,7 +234,7 @@ int q4_dot16_launch(const Q4DotLaunch &L, int waves, hipStream_t stream) {
 #define DOT16_PASSES(TT, WW) \
         if (L.tokens == TT && waves == WW) \
             return md == 16 ? launch16<TT, WW, 16, true>(L, stream) : launch16<TT, WW, 32, true>(L, stream)
-        DOT16_PASSES(2, 8); DOT16_PASSES(4, 8); DOT16_PASSES(4, 12);
+        DOT16_PASSES(4, 8); DOT16_PASSES(4, 12);
 #undef DOT16_PASSES
         return -1;
     }
@@ -187,7 +249,7 @@ int q4_dot16_launch(const Q4DotLaunch &L, int waves, hipStream_t stream) {
 
 // Whether q4_dot16_launch serves `passes` passes of `tokens` tokens with `waves` waves per workgroup.
 bool q4_dot16_takes_passes(int tokens, int waves) {
-    return (tokens == 2 && waves == 8) || (tokens == 4 && (waves == 8 || waves == 12));
+    return tokens == 4 && (waves == 8 || waves == 12);
 }
 
 }  // namespace mi355

@@ -20,6 +20,10 @@ constexpr int STEP16_BYTES = 4096;           // 2 strips x 16 rows x 128 bytes
 constexpr int LOADS16 = 4;                   // weight loads per step
 constexpr int WAVE16_LDS = 2 * STEP16_BYTES; // two steps per wave
 
+// Steps of the first of two column windows of a row of `steps` steps: at least half of them, and even (a window
+// starts on the first of the two step slots).
+__host__ __device__ constexpr int dot16_window_steps(int steps) { return ((steps + 1) / 2 + 1) & ~1; }
+
 // Where a lane finds the digits and the per-group factors of one pair of tokens.
 struct Dot16Operand {
     const uint8_t *digits;    // the lane's 16-byte piece of step 0, group 0, first quarter (or the zero region)
@@ -197,6 +201,14 @@ struct Dot16Stream {
     // The walk over the wave's steps, after settle(); the first two steps have been issued.
     template <int SETS>
     __device__ __forceinline__ void walk(const Dot16Operand (&operand)[SETS], float (&acc)[SETS]) {
+        walk_range(operand, acc, 0, step_hi - step_lo);
+    }
+
+    // Steps [from, to) of the wave's steps, counted from step_lo; `from` is even.  Steps from and from + 1 have been
+    // issued (by start() or by the range before); the range issues up to two steps past its own end when the wave
+    // has them, so that ranges follow each other without a gap in the stream.
+    template <int SETS>
+    __device__ __forceinline__ void walk_range(const Dot16Operand (&operand)[SETS], float (&acc)[SETS], int from, int to) {
         const bool no_bias = biases == nullptr;
         const int total_steps = step_hi - step_lo;
         struct StepWeights { u32x4 group[STAGE_GROUPS]; };
@@ -269,11 +281,11 @@ struct Dot16Stream {
         // Loads go out in step order, four per step, two steps ahead: a step's slot is refilled as soon as its
         // weights sit in registers.  Direct-to-LDS loads complete in issue order, so when step g is waited for, what
         // may still be in flight is the step behind it.
-        for (int base = 0; base < total_steps; base += 2) {
+        for (int base = from; base < to; base += 2) {
             const bool more = static_steps(std::make_integer_sequence<int, 2>{}, [&](auto step_in_turn) {
                 constexpr int r = decltype(step_in_turn)::value;
                 const int g = base + r;
-                if (g >= total_steps) return false;
+                if (g >= to) return false;
                 if (g + 1 < total_steps) wait_vm<LOADS16>(); else wait_vm<0>();
                 StepWeights w;
                 const uint8_t *stage = slot_lds[r];

@@ -220,5 +220,52 @@ __device__ __forceinline__ void build_q4_image(int tid, int ngrp, int SG, uint8_
     builder.build(tid, items, SG, zero_lds, img_lds, xm_lds, load);
 }
 
+// A window of the row, for kernels that hold only part of a wide row's image at a time.  The slots are
+// [token][strip 0 | strip 1][SGw]; they take the groups first .. first + groups_here of each strip (strip 1 starts at
+// group SG of the row).  Slots whose group lies past the window's or the row's end hold zero digits.  The zero region
+// is not written here.  request() fetches the activations of the thread's first items and may be called well before
+// build() (before the walk over the window in front, so that the walk hides the fetch).
+template <int T, int THREADS>
+struct Q4WindowBuilder {
+    static constexpr int BATCH = 4;
+    float xs[BATCH][8];
+    int ngrp, SG, first, groups_here, SGw;
+
+    __device__ __forceinline__ void window(int ngrp_, int SG_, int first_, int groups_here_, int SGw_) {
+        ngrp = ngrp_; SG = SG_; first = first_; groups_here = groups_here_; SGw = SGw_;
+    }
+    template <class LoadX>
+    __device__ __forceinline__ void fetch(int base, int tid, LoadX load) {
+        const int count = T * 2 * SGw * 8;
+#pragma unroll
+        for (int k = 0; k < BATCH; ++k) {
+            const int item = base + tid + k * THREADS;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) xs[k][c] = 0.0f;
+            if (item < count) {
+                const int slot = item >> 3, t = slot / (2 * SGw), w = slot - t * (2 * SGw);
+                const int strip = w >= SGw ? 1 : 0, gw = w - strip * SGw, g = strip * SG + first + gw;
+                if (gw < groups_here && g < ngrp) load(t, (size_t)g * 64 + 8 * (item & 7), xs[k]);
+            }
+        }
+    }
+    template <class LoadX>
+    __device__ __forceinline__ void request(int tid, LoadX load) { fetch(0, tid, load); }
+
+    template <class LoadX>
+    __device__ __forceinline__ void build(int tid, uint8_t *img_lds, float *xm_lds, LoadX load) {
+        const ImageItems slots(T, 2 * SGw);
+        for (int base = 0; base < slots.count; base += BATCH * THREADS) {
+            if (base > 0) fetch(base, tid, load);
+#pragma unroll
+            for (int k = 0; k < BATCH; ++k) {
+                const int item = base + tid + k * THREADS;
+                if (base + k * THREADS >= slots.count) break;        // uniform
+                image_store_item(item < slots.count ? item : slots.count - 1, item < slots.count, slots, SGw, xs[k], img_lds, xm_lds);
+            }
+        }
+    }
+};
+
 }  // namespace
 }  // namespace mi355

@@ -180,9 +180,12 @@ SHAPE_CASES = [
     (2816, 1, 2816, 24, "q4_dot16_kernel<1,8,16>"),
     (2816, 2, 2816, 24, "q4_dot16_kernel<2,12,16>"),
     (8192, 1, 2816, 24, "q4_dot16_kernel<1,12,32>"),
-    (8192, 4, 2816, 24, "q4_dot16_kernel<2,8,32> x 2 passes"),      # more tokens than one pass holds: one launch
-    (8192, 3, 2816, 24, "q4_dot16_kernel<2,8,32> x 2 passes"),      # ... whose last pass is short
-    (2816, 7, 2816, 24, "q4_dot16_kernel<4,12,16> x 2 passes"),
+    (8192, 4, 2816, 24, "q4_dot16_kernel<4,8,32> in 2 windows"),    # rows too wide for four tokens' planes at once
+    (8192, 3, 2816, 24, "q4_dot16_kernel<3,8,32> in 2 windows"),
+    (6272, 4, 2816, 24, "q4_dot16_kernel<4,8,32> in 2 windows"),    # 98 groups: the second window ends inside the row
+    (8192, 7, 2816, 24, "q4_dot16_kernel<3,8,32> in 2 windows"),   # four tokens, then three
+    (8192, 5, 2800, 24, "q4_dot16_kernel<1,12,32>"),                # four tokens in windows, then one; a ragged last block
+    (2816, 7, 2816, 24, "q4_dot16_kernel<4,12,16> x 2 passes"),     # more tokens than one pass holds: one launch
     (2112, 1, 2816, 2, "q4_dot_kernel<1,4,2,16,0> ksplit 4"),     # 33 groups: a step that straddles the row's end
     (6272, 3, 96, 1, None),                                          # 98 groups, three tokens, rows cut in 8
 ]
@@ -209,6 +212,7 @@ def test_the_shape_cases_cover_the_candidate_list():
     for cut in (1, 2, 4, 8):
         assert any(k.endswith(f"ksplit {cut}") for k in reached)
     assert any(",32,0>" in k for k in reached) and any("passes" in k for k in reached)
+    assert any("<3,8,32> in 2 windows" in k for k in reached) and any("<4,8,32> in 2 windows" in k for k in reached)
 
 
 def test_same_launch_gives_the_same_bits(pkg):
