@@ -19,7 +19,7 @@ reference's own C kernel when oracle/_ref is present (else the checker's
 port), and, under "extra", the same sweep on the bit-exact kernel, the MoE
 decode layer-step, the NVFP4 matvec and the batch-4 sweeps.
 
---only NAME runs a single leg (sweep, sweep-exact, sweep-b4, single, single-exact, moe, moe-t, prefill, nvfp4-t, copy): what the
+--only NAME runs a single leg (sweep, sweep-exact, sweep-b4, single, single-exact, moe, moe-t, prefill, abi, nvfp4-t, copy): what the
 rocprofv3 commands in profiles/ use.
 """
 from __future__ import annotations
@@ -423,6 +423,66 @@ def prefill_leg(gpu, synth, lib, stream, events, pool):
             "moe_prefill_mfma_frac": round(2 * flops / (ms_pf * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
 
 
+def abi_leg(synth, lib, pool, H, F, K):
+    """The engine-facing ABI with host pointers: per-call latency of salt_gpu_q4_matvec and salt_gpu_q4_moe_chain."""
+    out = {}
+    # BASELINE configs[0] through the engine-facing ABI: host pointers in and out (activation upload, launch,
+    # result download and a stream sync per call); a latency figure, never a throughput claim
+    import ctypes as C
+    R0 = C0 = 4096
+    v0, s0, b0 = synth.q4_tensor(R0, C0, 0)
+    blob = np.concatenate([v0.view(np.uint8), s0.view(np.uint8), b0.view(np.uint8)])
+    base = blob.ctypes.data
+    vp = C.c_void_p
+    lib.salt_gpu_weight_resource_describe.argtypes = [C.c_uint32, C.c_uint32, vp, C.c_size_t]
+    lib.salt_gpu_weight_resource_activate.argtypes = [C.c_uint32, C.c_uint32, C.c_int]
+    lib.salt_gpu_weight_resource_deactivate.argtypes = [C.c_uint32, C.c_uint32]
+    lib.salt_gpu_q4_matvec.argtypes = [vp, vp, vp, C.c_int, C.c_int, vp, vp]
+    x0, y0 = synth.activations(C0, 1, 1)[0], np.zeros(R0, np.float32)
+    if (lib.salt_gpu_init() == 0 and lib.salt_gpu_weight_resource_describe(1, 900, base, blob.nbytes) == 0
+            and lib.salt_gpu_weight_resource_activate(1, 900, 2) == 0):
+        def abi_call():
+            if lib.salt_gpu_q4_matvec(base, base + v0.nbytes, base + v0.nbytes + s0.nbytes, R0, C0,
+                                      x0.ctypes.data, y0.ctypes.data) != 0:
+                raise RuntimeError(lib.salt_mi355_last_error().decode())
+        for _ in range(5):
+            abi_call()
+        t0 = time.perf_counter()
+        for _ in range(200):
+            abi_call()
+        out["abi_q4_matvec_4096_host_pointers_us"] = round((time.perf_counter() - t0) / 200 * 1e6, 1)
+        lib.salt_gpu_weight_resource_deactivate(1, 900)
+        # the engine's decode call for the routed experts: salt_gpu_q4_moe_chain over eight experts, one row each
+        import engine_abi
+        eabi = engine_abi.bind(lib)
+        if eabi.salt_gpu_expert_resource_bind(901, pool.ctypes.data, pool.nbytes) == 0:
+            proj, n = synth.expert_proj_bytes(H, F), H * F
+            recs = (engine_abi.MoeExpert * K)()
+            for i, e8 in enumerate(range(3, 3 + 15 * K, 15)):
+                at = pool.ctypes.data + e8 * 3 * proj
+                for p_, name in enumerate(("gate", "up", "down")):
+                    setattr(recs[i], name + "_vals", at + p_ * proj)
+                    setattr(recs[i], name + "_scales", at + p_ * proj + n // 2)
+                    setattr(recs[i], name + "_biases", at + p_ * proj + n // 2 + (n // 64) * 2)
+                    setattr(recs[i], name + "_id", at + p_ * proj)
+                recs[i].group, recs[i].resource_slot, recs[i].logical_resource_id = 1, -1, 0
+            xin = np.tile(synth.activations(H, 1, 7)[0], (K, 1)).astype(np.float32)
+            yout, scr = np.zeros((K, H), np.float32), np.zeros((2, K * F), np.float32)
+
+            def chain_call():
+                if eabi.salt_gpu_q4_moe_chain(recs, K, H, F, xin.ctypes.data, yout.ctypes.data, scr[0].ctypes.data,
+                                              scr[1].ctypes.data, K * F) != 0:
+                    raise RuntimeError(lib.salt_mi355_last_error().decode())
+            for _ in range(20):
+                chain_call()
+            t0 = time.perf_counter()
+            for _ in range(200):
+                chain_call()
+            out["abi_q4_moe_chain_8_experts_us"] = round((time.perf_counter() - t0) / 200 * 1e6, 1)
+            eabi.salt_gpu_expert_resource_unbind(901)
+    return out
+
+
 def run_only(args, gpu, synth, lib, stream, events):
     """One leg on its own, for profiler runs: the kernels of that leg are the only matvec kernels in the trace."""
     if args.only == "copy":
@@ -434,6 +494,8 @@ def run_only(args, gpu, synth, lib, stream, events):
     if args.only in ("moe", "moe-t"):
         pool = synth.expert_pool(128, 2816, 704, 7)
         return moe_leg(gpu, synth, lib, stream, events, pool, args.only == "moe-t")
+    if args.only == "abi":
+        return abi_leg(synth, lib, synth.expert_pool(128, 2816, 704, 7), 2816, 704, 8)
     if args.only == "prefill":
         return prefill_leg(gpu, synth, lib, stream, events, synth.expert_pool(128, 2816, 704, 7))
     if args.only in ("single", "single-exact"):
@@ -467,7 +529,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the MoE / NVFP4 / batch-4 legs")
-    ap.add_argument("--only", default="", help="run one leg: sweep | sweep-exact | sweep-b4 | sweep-b4-exact | single | single-exact | moe | moe-t | prefill | nvfp4-t | copy")
+    ap.add_argument("--only", default="", help="run one leg: sweep | sweep-exact | sweep-b4 | sweep-b4-exact | single | single-exact | moe | moe-t | prefill | abi | nvfp4-t | copy")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU mode (run with --gpus 1)")
@@ -649,60 +711,7 @@ def main():
         extra["nvfp4_8192_b256_tflops"] = round(2.0 * R * Cc * B / (ms_mm * 1e-3) / 1e12, 1)
         extra["nvfp4_8192_b256_mfma_frac"] = round(2.0 * R * Cc * B / (ms_mm * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
         del w, xb, yb, wsb
-        # BASELINE configs[0] through the engine-facing ABI: host pointers in and out (activation upload, launch,
-        # result download and a stream sync per call); a latency figure, never a throughput claim
-        import ctypes as C
-        R0 = C0 = 4096
-        v0, s0, b0 = synth.q4_tensor(R0, C0, 0)
-        blob = np.concatenate([v0.view(np.uint8), s0.view(np.uint8), b0.view(np.uint8)])
-        base = blob.ctypes.data
-        vp = C.c_void_p
-        lib.salt_gpu_weight_resource_describe.argtypes = [C.c_uint32, C.c_uint32, vp, C.c_size_t]
-        lib.salt_gpu_weight_resource_activate.argtypes = [C.c_uint32, C.c_uint32, C.c_int]
-        lib.salt_gpu_weight_resource_deactivate.argtypes = [C.c_uint32, C.c_uint32]
-        lib.salt_gpu_q4_matvec.argtypes = [vp, vp, vp, C.c_int, C.c_int, vp, vp]
-        x0, y0 = synth.activations(C0, 1, 1)[0], np.zeros(R0, np.float32)
-        if (lib.salt_gpu_init() == 0 and lib.salt_gpu_weight_resource_describe(1, 900, base, blob.nbytes) == 0
-                and lib.salt_gpu_weight_resource_activate(1, 900, 2) == 0):
-            def abi_call():
-                if lib.salt_gpu_q4_matvec(base, base + v0.nbytes, base + v0.nbytes + s0.nbytes, R0, C0,
-                                          x0.ctypes.data, y0.ctypes.data) != 0:
-                    raise RuntimeError(lib.salt_mi355_last_error().decode())
-            for _ in range(5):
-                abi_call()
-            t0 = time.perf_counter()
-            for _ in range(200):
-                abi_call()
-            extra["abi_q4_matvec_4096_host_pointers_us"] = round((time.perf_counter() - t0) / 200 * 1e6, 1)
-            lib.salt_gpu_weight_resource_deactivate(1, 900)
-            # the engine's decode call for the routed experts: salt_gpu_q4_moe_chain over eight experts, one row each
-            import engine_abi
-            eabi = engine_abi.bind(lib)
-            if eabi.salt_gpu_expert_resource_bind(901, pool.ctypes.data, pool.nbytes) == 0:
-                proj, n = synth.expert_proj_bytes(H, F), H * F
-                recs = (engine_abi.MoeExpert * K)()
-                for i, e8 in enumerate(range(3, 3 + 15 * K, 15)):
-                    at = pool.ctypes.data + e8 * 3 * proj
-                    for p_, name in enumerate(("gate", "up", "down")):
-                        setattr(recs[i], name + "_vals", at + p_ * proj)
-                        setattr(recs[i], name + "_scales", at + p_ * proj + n // 2)
-                        setattr(recs[i], name + "_biases", at + p_ * proj + n // 2 + (n // 64) * 2)
-                        setattr(recs[i], name + "_id", at + p_ * proj)
-                    recs[i].group, recs[i].resource_slot, recs[i].logical_resource_id = 1, -1, 0
-                xin = np.tile(synth.activations(H, 1, 7)[0], (K, 1)).astype(np.float32)
-                yout, scr = np.zeros((K, H), np.float32), np.zeros((2, K * F), np.float32)
-
-                def chain_call():
-                    if eabi.salt_gpu_q4_moe_chain(recs, K, H, F, xin.ctypes.data, yout.ctypes.data, scr[0].ctypes.data,
-                                                  scr[1].ctypes.data, K * F) != 0:
-                        raise RuntimeError(lib.salt_mi355_last_error().decode())
-                for _ in range(20):
-                    chain_call()
-                t0 = time.perf_counter()
-                for _ in range(200):
-                    chain_call()
-                extra["abi_q4_moe_chain_8_experts_us"] = round((time.perf_counter() - t0) / 200 * 1e6, 1)
-                eabi.salt_gpu_expert_resource_unbind(901)
+        extra.update(abi_leg(synth, lib, pool, H, F, K))
         extra.update(prefill_leg(gpu, synth, lib, stream, events, pool))
         # the bf16 head (262144 x 2816, the largest matrix a decode step streams) and the 8-bit router gate
         # (128 x 2816, one unsplittable 2816-step chain per row), both bit-exact

@@ -192,6 +192,14 @@ uint8_t *pinned_device_view(const uint8_t *pin) { return g_engine.pinned_dev + (
 float *upload_activations(const float *host, size_t count) {
     uint8_t *pin = pinned_take(count * 4), *dev = device_take(count * 4);
     memcpy(pin, host, count * 4);
+    if (zero_copy(count * 4)) {
+        // a few kilobytes: one small kernel reads them across the bus once (a launch costs less than a copy command)
+        if (copy_words_launch(dev, pinned_device_view(pin), count, g_state.stream) != 0) {
+            set_error("activation upload: copy kernel failed to launch");
+            return nullptr;
+        }
+        return (float *)dev;
+    }
     if (hip_ok(hipMemcpyAsync(dev, pin, count * 4, hipMemcpyHostToDevice, g_state.stream), "activation upload") != 0)
         return nullptr;
     return (float *)dev;

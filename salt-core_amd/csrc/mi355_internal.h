@@ -342,6 +342,8 @@ int moe_prefill_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_
 
 // Zero `words` 32-bit words at dst with a kernel on `stream` (safe under graph capture, unlike a memset node).
 int clear_words_launch(void *dst, size_t words, hipStream_t stream);
+// Copy `words` 32-bit words with a kernel; src may be mapped pinned host memory (its device view).
+int copy_words_launch(void *dst, const void *src, size_t words, hipStream_t stream);
 
 // ---------------------------------------------------------------- formats (formats.hip)
 

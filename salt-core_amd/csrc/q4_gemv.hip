@@ -700,7 +700,20 @@ __global__ __launch_bounds__(256) void clear_words_kernel(uint32_t *dst, size_t 
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i < words) dst[i] = 0u;
 }
+__global__ __launch_bounds__(256) void copy_words_kernel(uint32_t *dst, const uint32_t *src, size_t words) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < words) dst[i] = src[i];
+}
 }  // namespace
+
+// Word copy by a kernel, for sources the device can address (mapped pinned host memory included): for a few
+// kilobytes a launch is cheaper than a copy command.
+int copy_words_launch(void *dst, const void *src, size_t words, hipStream_t stream) {
+    if (words == 0) return 0;
+    hipLaunchKernelGGL(copy_words_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream, (uint32_t *)dst,
+                       (const uint32_t *)src, words);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
 
 // Zero fill by a kernel: a memset node recorded into a caller's graph capture is not reliable on replay here.
 int clear_words_launch(void *dst, size_t words, hipStream_t stream) {
