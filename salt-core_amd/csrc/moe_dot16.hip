@@ -98,20 +98,31 @@ __global__ __launch_bounds__(MOE16_MAX_TOPK * 64) void moe16_down_sum_kernel(con
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    Dot16Stream<MD> stream;
+    stream.setup(lane, m.routed, lds + (size_t)wave * WAVE16_LDS);
+    const int SG = stream.SG;
+    // The activations of all selected experts (expert e of the selection is "token" e of the digit planes) are
+    // requested first, together with the status and the selection, and the weight loads go out when they have
+    // arrived: the digit planes are then built while the weights are on their way (weights first, activations
+    // queued behind them, cost the step a microsecond).  A rejected step leaves whatever an earlier step wrote in
+    // the activations; it is fetched and dropped.
+    const int topk = m.topk;
+    const ImageItems items(topk, stream.ngrp);
+    Q4ImageBuilder<THREADS> image;
+    image.request_early(tid, items, [&](int e) { return m.act + (size_t)e * m.routed; });
     // what the first launch left: status, selection and routing weights, fetched in one go as wave-uniform values
     typedef const int __attribute__((address_space(4))) *uniform_int_ptr;
     typedef const float __attribute__((address_space(4))) *uniform_float_ptr;
-    const bool has_expert = wave < m.topk;
+    const bool has_expert = wave < topk;
     const int status = *(uniform_int_ptr)(uintptr_t)m.status;
     const int expert = ((uniform_int_ptr)(uintptr_t)m.selected)[has_expert ? wave : 0];
     float routing[WAVES];
 #pragma unroll
-    for (int e = 0; e < WAVES; ++e) routing[e] = ((uniform_float_ptr)(uintptr_t)m.weights)[e < m.topk ? e : 0];
-    if (status != 0) return;                         // the router rejected its input
-
-    Dot16Stream<MD> stream;
-    stream.setup(lane, m.routed, lds + (size_t)wave * WAVE16_LDS);
-    const int SG = stream.SG;
+    for (int e = 0; e < WAVES; ++e) routing[e] = ((uniform_float_ptr)(uintptr_t)m.weights)[e < topk ? e : 0];
+    if (status != 0) {                               // the router rejected its input
+        image.settle(status, items);                 // nothing of the wave's may be in flight when it ends
+        return;
+    }
     uint8_t *const zero_lds = lds + WAVES * WAVE16_LDS;
     uint8_t *const img_lds = zero_lds + ZERO_BYTES;                        // [expert of the selection][2 * SG][GROUP_IMAGE]
     float *const xm_lds = (float *)(img_lds + (size_t)WAVES * 2 * SG * GROUP_IMAGE);
@@ -119,14 +130,13 @@ __global__ __launch_bounds__(MOE16_MAX_TOPK * 64) void moe16_down_sum_kernel(con
     const int row_base = (int)blockIdx.x * ROWS16;
     const size_t n_weights = (size_t)m.hidden * (size_t)m.routed;
     const size_t vals_bytes = n_weights / 2, meta_bytes = (n_weights / 64) * 2, proj_bytes = vals_bytes + 2 * meta_bytes;
+    image.settle(expert, items);
     if (has_expert) {
         const uint8_t *vals = m.pool + (size_t)expert * m.expert_stride + 2 * proj_bytes;
         stream.bind(vals, vals + vals_bytes, vals + vals_bytes + meta_bytes, m.hidden, row_base, 0, stream.nstage);
         stream.start();
     }
-    // the activations of all selected experts become digit planes: expert e of the selection is "token" e
-    const int topk = m.topk;
-    build_q4_image<0, THREADS>(tid, stream.ngrp, SG, zero_lds, img_lds, xm_lds, topk, [&](int e, size_t column, float (&xv)[8]) {
+    image.build(tid, items, SG, zero_lds, img_lds, xm_lds, [&](int e, size_t column, float (&xv)[8]) {
 #pragma unroll
         for (int k = 0; k < 8; ++k) xv[k] = m.act[(size_t)e * m.routed + column + k];
     });
