@@ -19,7 +19,7 @@ reference's own C kernel when oracle/_ref is present (else the checker's
 port), and, under "extra", the same sweep on the bit-exact kernel, the MoE
 decode layer-step, the NVFP4 matvec and the batch-4 sweeps.
 
---only NAME runs a single leg (sweep, sweep-exact, sweep-b4, single, single-exact, moe, moe-t, prefill, abi, nvfp4-t, copy): what the
+--only NAME runs a single leg (sweep, sweep-exact, sweep-b4, single, single-exact, moe, moe-t, prefill, abi, nvfp4-t, nvfp4-b256, copy): what the
 rocprofv3 commands in profiles/ use.
 """
 from __future__ import annotations
@@ -423,6 +423,24 @@ def prefill_leg(gpu, synth, lib, stream, events, pool):
             "moe_prefill_mfma_frac": round(2 * flops / (ms_pf * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
 
 
+def nvfp4_b256_leg(gpu, synth, lib, stream, events, w, scales_at, st, R, Cc):
+    """NVFP4 R x Cc, batch 256, on the matrix cores (tolerance class); the activation pass is part of the call."""
+    B = 256
+    xb = gpu.DeviceBuffer.from_host(synth.activations(Cc, B, 42))
+    yb = gpu.DeviceBuffer(B * R * 4)
+    wsb = gpu.DeviceBuffer(lib.salt_mi355_nvfp4_matmul_workspace_bytes(R, Cc, B))
+
+    def fp4_matmul_step(s):
+        if lib.salt_mi355_nvfp4_matmul_dev(w.at(0), w.at(scales_at), 2688.0, 64.0, R, Cc, B, xb.ptr, yb.ptr,
+                                           st.ptr, wsb.ptr, s) != 0:
+            raise RuntimeError(lib.salt_mi355_last_error().decode())
+
+    ms_mm = timed(lib, stream, events, fp4_matmul_step, 2, 20)
+    return {"nvfp4_8192_b256_matmul_us": round(ms_mm * 1e3, 2),
+            "nvfp4_8192_b256_tflops": round(2.0 * R * Cc * B / (ms_mm * 1e-3) / 1e12, 1),
+            "nvfp4_8192_b256_mfma_frac": round(2.0 * R * Cc * B / (ms_mm * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+
+
 def abi_leg(synth, lib, pool, H, F, K):
     """The engine-facing ABI with host pointers: per-call latency of salt_gpu_q4_matvec and salt_gpu_q4_moe_chain."""
     out = {}
@@ -507,6 +525,14 @@ def run_only(args, gpu, synth, lib, stream, events):
             out[f"q4_{R}x{Cc}_single_launch_us"] = round(ms_1 * 1e3, 2)
             out[f"q4_{R}x{Cc}_kernel"] = lib.salt_mi355_last_kernel().decode()
         return out
+    if args.only == "nvfp4-b256":
+        R = Cc = 8192
+        packed, fscales = synth.nvfp4_tensor(R, Cc, 40)
+        w = gpu.DeviceBuffer(packed.nbytes + fscales.nbytes)
+        w.upload(packed, 0)
+        w.upload(fscales, packed.nbytes)
+        st = gpu.DeviceBuffer(4, fill=0)
+        return nvfp4_b256_leg(gpu, synth, lib, stream, events, w, packed.nbytes, st, R, Cc)
     if args.only == "nvfp4-t":
         R = Cc = 8192
         packed, fscales = synth.nvfp4_tensor(R, Cc, 40)
@@ -529,7 +555,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the MoE / NVFP4 / batch-4 legs")
-    ap.add_argument("--only", default="", help="run one leg: sweep | sweep-exact | sweep-b4 | sweep-b4-exact | single | single-exact | moe | moe-t | prefill | abi | nvfp4-t | copy")
+    ap.add_argument("--only", default="", help="run one leg: sweep | sweep-exact | sweep-b4 | sweep-b4-exact | single | single-exact | moe | moe-t | prefill | abi | nvfp4-t | nvfp4-b256 | copy")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU mode (run with --gpus 1)")
@@ -695,22 +721,8 @@ def main():
         fp4_t = nvfp4_class_t_leg(gpu, synth, lib, stream, events, w, per, packed.nbytes, x, st, R, Cc, G)
         extra.update(fp4_t)
         del xq, ys16
-        # NVFP4 8192 x 8192, batch 256, on the matrix cores (tolerance class); activation pass included
-        B = 256
-        xb = gpu.DeviceBuffer.from_host(synth.activations(Cc, B, 42))
-        yb = gpu.DeviceBuffer(B * R * 4)
-        wsb = gpu.DeviceBuffer(lib.salt_mi355_nvfp4_matmul_workspace_bytes(R, Cc, B))
-
-        def fp4_matmul_step(s):
-            if lib.salt_mi355_nvfp4_matmul_dev(w.at(0), w.at(packed.nbytes), 2688.0, 64.0, R, Cc, B, xb.ptr, yb.ptr,
-                                               st.ptr, wsb.ptr, s) != 0:
-                raise RuntimeError(lib.salt_mi355_last_error().decode())
-
-        ms_mm = timed(lib, stream, events, fp4_matmul_step, 2, 20)
-        extra["nvfp4_8192_b256_matmul_us"] = round(ms_mm * 1e3, 2)
-        extra["nvfp4_8192_b256_tflops"] = round(2.0 * R * Cc * B / (ms_mm * 1e-3) / 1e12, 1)
-        extra["nvfp4_8192_b256_mfma_frac"] = round(2.0 * R * Cc * B / (ms_mm * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)
-        del w, xb, yb, wsb
+        extra.update(nvfp4_b256_leg(gpu, synth, lib, stream, events, w, packed.nbytes, st, R, Cc))
+        del w
         extra.update(abi_leg(synth, lib, pool, H, F, K))
         extra.update(prefill_leg(gpu, synth, lib, stream, events, pool))
         # the bf16 head (262144 x 2816, the largest matrix a decode step streams) and the 8-bit router gate

@@ -92,12 +92,18 @@ int salt_mi355_nvfp4_matvec_dev(const void *packed, const void *scales, float st
 }
 
 namespace {
-struct Fp4MatmulWorkspace { int *status; uint16_t *plane; float *partials; size_t bytes; };
+// The activation pass reports per workgroup (flags) while the call is small enough for every consumer workgroup to
+// read all of them; beyond that through the status word, cleared by a launch of its own.
+constexpr int FP4_MATMUL_MAX_FLAGS = 4096;
+struct Fp4MatmulWorkspace { int *status; int *flags; int nflags; uint16_t *plane; float *partials; size_t bytes; };
 Fp4MatmulWorkspace fp4_matmul_carve(void *base, int R, int C, int B) {
     Fp4MatmulWorkspace w;
     uint8_t *p = (uint8_t *)base;
     auto take = [&](size_t n) { uint8_t *q = p; p += (n + 255) & ~(size_t)255; return q; };
     w.status = (int *)take(4);
+    w.nflags = fp4_qdq_flag_count(C, B);
+    if (w.nflags > FP4_MATMUL_MAX_FLAGS) w.nflags = 0;
+    w.flags = w.nflags ? (int *)take((size_t)w.nflags * 4) : nullptr;
     w.plane = (uint16_t *)take((size_t)B * C * 2);
     const int splits = fp4_mfma_splits(R, C, B);
     w.partials = splits > 1 ? (float *)take((size_t)splits * B * R * 4) : nullptr;
@@ -125,19 +131,28 @@ int salt_mi355_nvfp4_matmul_dev(const void *packed, const void *scales, float st
     }
     const Fp4MatmulWorkspace w = fp4_matmul_carve(workspace, R, C, B);
     hipStream_t s = (hipStream_t)stream;
-    if (clear_words_launch(w.status, 1, s) != 0) { set_error("nvfp4 matmul: status clear failed to launch"); return -1; }
-    if (fp4_qdq_launch(xs, C, B, input_global_scale, nullptr, nullptr, nullptr, w.plane, w.status, s) != 0) {
-        set_error("nvfp4 matmul: activation pass failed to launch");
-        return -1;
+    if (w.flags) {
+        if (fp4_qdq_flags_launch(xs, C, B, input_global_scale, w.plane, w.flags, s) != 0) {
+            set_error("nvfp4 matmul: activation pass failed to launch");
+            return -1;
+        }
+    } else {
+        if (clear_words_launch(w.status, 1, s) != 0) { set_error("nvfp4 matmul: status clear failed to launch"); return -1; }
+        if (fp4_qdq_launch(xs, C, B, input_global_scale, nullptr, nullptr, nullptr, w.plane, w.status, s) != 0) {
+            set_error("nvfp4 matmul: activation pass failed to launch");
+            return -1;
+        }
     }
     Fp4MfmaLaunch launch;
     memset(&launch, 0, sizeof launch);
     launch.packed = (const uint8_t *)packed; launch.scales = (const uint8_t *)scales;
     launch.plane = w.plane; launch.ys = ys; launch.partials = w.partials; launch.status = w.status;
+    launch.flags = w.flags; launch.nflags = w.nflags; launch.verdict = w.status; launch.verdict_copy = status_dev;
     launch.rows = R; launch.cols = C; launch.tokens = B; launch.ksplit = fp4_mfma_splits(R, C, B);
     launch.out_scale = (1.0f / stored_divisor) / input_global_scale;
     if (fp4_mfma_launch(launch, s) != 0) { set_error("nvfp4 matmul: launch failed"); return -1; }
     if (status_dev) {
+        if (w.flags) return 0;                      // the last launch has written it
         if (hip_ok(hipMemcpyAsync(status_dev, w.status, 4, hipMemcpyDeviceToDevice, s), "nvfp4 matmul status copy") != 0)
             return -1;
         return 0;

@@ -228,6 +228,11 @@ int fp4_dot_launch(const Fp4DotLaunch &launch, const DotShape &shape, hipStream_
 int fp4_qdq_launch(const float *input, int cols, int tokens, float input_global_scale,
                    uint8_t *packed, uint8_t *scales, float *dequant, uint16_t *plane, int *status,
                    hipStream_t stream);
+// The same pass reporting per workgroup instead of through one word that somebody must have cleared: flags[i]
+// receives 0 or -1 from workgroup i, every one of the fp4_qdq_flag_count(cols, tokens) words is written.
+int fp4_qdq_flag_count(int cols, int tokens);
+int fp4_qdq_flags_launch(const float *input, int cols, int tokens, float input_global_scale, uint16_t *plane,
+                         int *flags, hipStream_t stream);
 
 // Prefill-sized NVFP4 matmul on the matrix cores (tolerance class): ys[token][row] =
 // out_scale * sum_c (code * block scale)[row][c] * plane[token][c].
@@ -236,7 +241,12 @@ struct Fp4MfmaLaunch {
     const uint16_t *plane;    // [tokens][cols] bf16
     float *ys;                // [tokens][rows]
     float *partials;          // [ksplit][tokens][rows], used when ksplit > 1
-    const int *status;        // nothing is published unless *status == 0
+    const int *status;        // nothing is published unless *status == 0 ...
+    // ... or, when flags is set, unless all nflags words are 0; the launch then writes the verdict (0 or -1) to
+    // verdict and, when set, verdict_copy, and `status` is not read
+    const int *flags;
+    int nflags;
+    int *verdict, *verdict_copy;
     int rows, cols, tokens, ksplit;
     float out_scale;
 };

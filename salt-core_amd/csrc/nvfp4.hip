@@ -343,24 +343,36 @@ int launch_tiles(const Fp4Launch &L, hipStream_t stream) {
 
 // ---------------------------------------------------------------- activation Q/DQ
 
-// One thread per 16-element block of one token.
+// One thread per 16-element block of one token.  FLAGS: the workgroup reports in flags[blockIdx.x] (0 or -1, always
+// written) instead of setting *status.
+template <bool FLAGS>
 __global__ __launch_bounds__(256) void fp4_qdq_kernel(const float *__restrict__ input, int cols, int tokens,
                                                       float g, uint8_t *__restrict__ packed,
                                                       uint8_t *__restrict__ scales, float *__restrict__ dequant,
                                                       uint16_t *__restrict__ plane, int *__restrict__ status) {
     const int blocks_per_token = cols >> 4;
     const long long item = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (item >= (long long)blocks_per_token * tokens) return;
-    const float4 *src = reinterpret_cast<const float4 *>(input + item * 16);
+    const bool present = item < (long long)blocks_per_token * tokens;
+    if (!FLAGS && !present) return;
     float v[16];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const float4 f = src[q];
-        v[4 * q] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w;
+    for (int q = 0; q < 16; ++q) v[q] = 0.0f;
+    if (present) {
+        const float4 *src = reinterpret_cast<const float4 *>(input + item * 16);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float4 f = src[q];
+            v[4 * q] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w;
+        }
     }
     uint32_t scale_code, bytes[2], halves[8];
     float out[16];
-    if (!qdq_block(v, g, scale_code, bytes, out, halves)) {     // the reference rejects the whole call
+    const bool good = qdq_block(v, g, scale_code, bytes, out, halves);    // the reference rejects the whole call
+    if (FLAGS) {
+        const int any_bad = __syncthreads_or(good ? 0 : 1);
+        if (threadIdx.x == 0) status[blockIdx.x] = any_bad ? -1 : 0;
+        if (!present || !good) return;
+    } else if (!good) {
         *status = -1;
         return;
     }
@@ -399,8 +411,22 @@ int fp4_qdq_launch(const float *input, int cols, int tokens, float input_global_
     const long long items = (long long)(cols >> 4) * tokens;
     if (items < 1 || (cols & 15)) return -1;
     const unsigned grid = (unsigned)((items + 255) / 256);
-    hipLaunchKernelGGL(fp4_qdq_kernel, dim3(grid), dim3(256), 0, stream, input, cols, tokens, input_global_scale,
+    hipLaunchKernelGGL(fp4_qdq_kernel<false>, dim3(grid), dim3(256), 0, stream, input, cols, tokens, input_global_scale,
                        packed, scales, dequant, plane, status);
+    return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+int fp4_qdq_flag_count(int cols, int tokens) {
+    const long long items = (long long)(cols >> 4) * tokens;
+    return items < 1 || items > (1ll << 38) ? 0 : (int)((items + 255) / 256);
+}
+
+int fp4_qdq_flags_launch(const float *input, int cols, int tokens, float input_global_scale, uint16_t *plane,
+                         int *flags, hipStream_t stream) {
+    const int grid = fp4_qdq_flag_count(cols, tokens);
+    if (grid < 1 || (cols & 15) || !flags) return -1;
+    hipLaunchKernelGGL(fp4_qdq_kernel<true>, dim3((unsigned)grid), dim3(256), 0, stream, input, cols, tokens,
+                       input_global_scale, (uint8_t *)nullptr, (uint8_t *)nullptr, (float *)nullptr, plane, flags);
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

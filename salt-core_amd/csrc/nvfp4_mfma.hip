@@ -40,6 +40,20 @@ struct Geometry {
     int m_tiles, n_tiles, chunks, chunks_per_split;
 };
 
+// Whether the activation pass rejected its input: the launch's status word, or the OR of the pass's per-workgroup
+// flags (every thread of the workgroup calls this; workgroup 0 then also publishes the verdict).
+__device__ __forceinline__ bool rejected(const Fp4MfmaLaunch &L) {
+    if (!L.flags) return *(const int __attribute__((address_space(4))) *)(uintptr_t)L.status != 0;
+    int bad = 0;
+    for (int i = threadIdx.x; i < L.nflags; i += blockDim.x) bad |= L.flags[i];
+    const int any_bad = __syncthreads_or(bad);
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        *L.verdict = any_bad ? -1 : 0;
+        if (L.verdict_copy) *L.verdict_copy = any_bad ? -1 : 0;
+    }
+    return any_bad != 0;
+}
+
 __device__ __forceinline__ uint32_t pack_upper_halves(float lo, float hi) {
     return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
 }
@@ -148,7 +162,7 @@ void fp4_mfma_kernel(const Fp4MfmaLaunch L, const Geometry G) {
     }
 
     const bool direct = L.ksplit == 1;
-    if (direct && *(const int __attribute__((address_space(4))) *)(uintptr_t)L.status != 0) return;
+    if (direct && rejected(L)) return;
     float __attribute__((address_space(1))) *out =
         (float __attribute__((address_space(1))) *)(uintptr_t)(direct ? L.ys
                                                                       : L.partials + (size_t)split * L.tokens * L.rows);
@@ -168,10 +182,12 @@ void fp4_mfma_kernel(const Fp4MfmaLaunch L, const Geometry G) {
 }
 
 // ys = out_scale * (partial 0 + partial 1 + ...), added in split order
-__global__ __launch_bounds__(256) void fp4_split_sum_kernel(const float *__restrict__ partials, size_t n, int ksplit,
-                                                            float out_scale, const int *__restrict__ status,
-                                                            float *__restrict__ ys) {
-    if (*status != 0) return;
+__global__ __launch_bounds__(256) void fp4_split_sum_kernel(const Fp4MfmaLaunch L, size_t n) {
+    if (rejected(L)) return;
+    const float *__restrict__ partials = L.partials;
+    float *__restrict__ ys = L.ys;
+    const int ksplit = L.ksplit;
+    const float out_scale = L.out_scale;
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= n) return;
     if ((n & 3) == 0) {
@@ -205,7 +221,8 @@ int fp4_mfma_splits(int rows, int cols, int tokens) {
 }
 
 int fp4_mfma_launch(const Fp4MfmaLaunch &L, hipStream_t stream) {
-    if (L.rows < 1 || L.tokens < 1 || L.cols < KC || (L.cols % KC) || L.ksplit < 1 || !L.status) return -1;
+    if (L.rows < 1 || L.tokens < 1 || L.cols < KC || (L.cols % KC) || L.ksplit < 1) return -1;
+    if (L.flags ? (L.nflags < 1 || !L.verdict) : !L.status) return -1;
     Geometry G;
     G.m_tiles = (L.tokens + TM - 1) / TM;
     G.n_tiles = (L.rows + TN - 1) / TN;
@@ -218,8 +235,7 @@ int fp4_mfma_launch(const Fp4MfmaLaunch &L, hipStream_t stream) {
     hipLaunchKernelGGL(fp4_mfma_kernel, dim3((unsigned)grid), dim3(256), 0, stream, L, G);
     if (L.ksplit > 1) {
         const size_t n = (size_t)L.tokens * L.rows;
-        hipLaunchKernelGGL(fp4_split_sum_kernel, dim3((unsigned)((n / 4 + 256) / 256)), dim3(256), 0, stream,
-                           L.partials, n, L.ksplit, L.out_scale, L.status, L.ys);
+        hipLaunchKernelGGL(fp4_split_sum_kernel, dim3((unsigned)((n / 4 + 256) / 256)), dim3(256), 0, stream, L, n);
     }
     return hipGetLastError() == hipSuccess ? 0 : -1;
 }
