@@ -42,6 +42,11 @@ struct MoeFuse {
     float *weights;               // [topk]
     int *status;                  // 0, or -1 when the router rejected its input (then nothing else is written)
     int n_experts, topk, hidden, routed;
+    // q4_moe_gate_up_launch / q4_moe_down_launch only, both null or both set: the down launch also writes the layer
+    // output.  arrivals holds one counter per 64-row tile of the output; the gate/up launch zeroes them, and the last
+    // of the topk workgroups of the down launch to finish a tile adds that tile's expert outputs in expert order.
+    float *out;                   // [hidden]
+    int *arrivals;                // [ceil(hidden / 64)]
 };
 constexpr int MOE_FUSE_MAX_ROUTED = 4096;      // activations of one expert held in LDS by the down launch
 constexpr int MOE_FUSE_MAX_EXPERTS = 512;      // one thread per expert in the gate/up prologue
@@ -315,6 +320,7 @@ struct MoeWorkspace {
     float *act;               // [topk][routed]
     float *expert_out;        // [topk][hidden]
     int *status;              // 0 ok, -1 router rejected its input
+    int *arrivals;            // one counter per 64 rows of the layer output (MoeFuse::arrivals)
 };
 
 size_t moe_workspace_bytes(const MoeGeometry &g);

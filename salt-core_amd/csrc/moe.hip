@@ -110,7 +110,8 @@ size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 size_t moe_workspace_bytes(const MoeGeometry &g) {
     const size_t k = (size_t)g.topk;
     return align256(256) + align256(2 * k * sizeof(Q4Job)) + align256(k * sizeof(Q4Job)) +
-           3 * align256(k * g.routed * sizeof(float)) + align256(k * g.hidden * sizeof(float));
+           3 * align256(k * g.routed * sizeof(float)) + align256(k * g.hidden * sizeof(float)) +
+           align256((size_t)((g.hidden + 63) / 64) * sizeof(int));
 }
 
 void moe_workspace_carve(const MoeGeometry &g, void *base, MoeWorkspace *ws) {
@@ -122,7 +123,8 @@ void moe_workspace_carve(const MoeGeometry &g, void *base, MoeWorkspace *ws) {
     ws->gate = (float *)p;                  p += align256(k * g.routed * sizeof(float));
     ws->up = (float *)p;                    p += align256(k * g.routed * sizeof(float));
     ws->act = (float *)p;                   p += align256(k * g.routed * sizeof(float));
-    ws->expert_out = (float *)p;
+    ws->expert_out = (float *)p;            p += align256(k * g.hidden * sizeof(float));
+    ws->arrivals = (int *)p;
 }
 
 int router_topk_launch(const float *logits, const float *per_expert_scale, int n_experts, int topk,
@@ -157,7 +159,8 @@ int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t exp
         return -1;
     float *eo = expert_out ? expert_out : ws.expert_out;
     if (g.n_experts <= MOE_FUSE_MAX_EXPERTS && g.routed <= MOE_FUSE_MAX_ROUTED) {
-        // Three launches: router + gate/up, activation + down, ordered reduction.
+        // Two launches: router + gate/up, then activation + down + the ordered reduction (by the last workgroup
+        // to finish each tile of the output).
         Q4Launch fused;
         memset(&fused, 0, sizeof fused);
         fused.code_scale = code_scale;
@@ -165,9 +168,9 @@ int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t exp
         m.logits = logits; m.per_expert_scale = per_expert_scale; m.pool = pool; m.expert_stride = expert_stride;
         m.x = x; m.gate = ws.gate; m.up = ws.up; m.expert_out = eo; m.selected = selected; m.weights = weights;
         m.status = ws.status; m.n_experts = g.n_experts; m.topk = g.topk; m.hidden = g.hidden; m.routed = g.routed;
+        m.out = out; m.arrivals = out ? ws.arrivals : nullptr;
         if (q4_moe_gate_up_launch(fused, stream) != 0) return -1;
-        if (q4_moe_down_launch(fused, stream) != 0) return -1;
-        return out ? moe_reduce_launch(eo, weights, g.topk, g.hidden, out, ws.status, stream) : 0;
+        return q4_moe_down_launch(fused, stream);
     }
     JobEmit emit;
     emit.gate_up_jobs = ws.gate_up_jobs;

@@ -217,6 +217,8 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
                 if (publisher) {
                     if (tid == 0) *m.status = bad ? -1 : 0;
                     if (tid < m.topk && !bad) { m.selected[tid] = sh.out_sel[tid]; m.weights[tid] = sh.out_w[tid]; }
+                    if (m.arrivals)                 // the down launch counts its workgroups per tile of the output
+                        for (int i = tid; i < (m.hidden + TILE_ROWS - 1) / TILE_ROWS; i += THREADS) m.arrivals[i] = 0;
                     return;
                 }
                 if (bad) return;                                           // uniform
@@ -500,7 +502,34 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
             for (int j = 0; j < 4; ++j) part[j] = part[j] + f[4 * a + j];
         const float even = part[0] + part[2];
         const float odd = part[1] + part[3];
-        if (lane < rows_here) y[(size_t)t * job.y_stride + row0 + lane] = even + odd;
+        if (PRO != 2 || !L.moe.arrivals) {
+            if (lane < rows_here) y[(size_t)t * job.y_stride + row0 + lane] = even + odd;
+        } else {                                        // uniform; NB == 1: these are the 64 lanes of wave 0
+            // The layer output (reference gemma4_text.c:8301-8304: out = 0; out += o_i * w_i in ascending expert
+            // order, product and sum rounded separately).  The topk workgroups that own these rows of the topk
+            // experts count themselves in; the one that arrives last finds every expert's rows written and adds
+            // them.  Which workgroup that is varies from run to run, the sum it forms does not.
+            //
+            // The rows travel as device-scope stores and loads (past the partition's cache, which other partitions
+            // do not see), ordered by waiting for the stores before the count and for the count before the loads: a
+            // fence would write the whole cache back, once per workgroup.
+            const MoeFuse &m = L.moe;
+            float *const mine = m.expert_out + (size_t)(job.y - m.expert_out) + row0;
+            if (lane < rows_here) __hip_atomic_store(mine + lane, even + odd, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            int before = 0;
+            if (tid == 0) before = __hip_atomic_fetch_add(m.arrivals + (row0 / TILE_ROWS), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            before = __builtin_amdgcn_readfirstlane(before);    // waits for the count's return
+            if (before == m.topk - 1 && lane < rows_here) {
+                float total = 0.0f;
+                for (int e = 0; e < m.topk; ++e) {
+                    const float o = __hip_atomic_load(m.expert_out + (size_t)e * m.hidden + row0 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    const float term = o * m.weights[e];
+                    total = total + term;
+                }
+                m.out[row0 + lane] = total;
+            }
+        }
     }
 }
 

@@ -284,6 +284,43 @@ def test_moe_decode_step_fresh_logits_and_rejection(gpu, oracle):
         assert np.array_equal(bits(y), bits(acc)), it
 
 
+@pytest.mark.parametrize("tolerance_class", [False, True], ids=["bit-exact", "class-t"])
+def test_moe_decode_step_replayed_as_a_graph(gpu, oracle, tolerance_class):
+    """Four consecutive steps captured once and replayed with fresh inputs (kernels only; the bit-exact plan's tile
+    counters are zeroed by its own first launch, so a replay needs nothing from the host): every replay equals the
+    eager step on the same inputs, with eager work and synchronisations between the replays."""
+    print("moe step graph replay", "class T" if tolerance_class else "bit-exact", flush=True)
+    E, K, H, F = 16, 8, 2816, 704
+    pool = synth.expert_pool(E, H, F, 35)
+    layer = gpu.MoeLayer(pool, E, H, F, K)
+    layer.tolerance_class = tolerance_class
+    lib = gpu.load()
+    stream = lib.salt_mi355_stream()
+    scale = np.ones(E, np.float32)
+    layer.step(synth.router_logits(E, 1000), scale, synth.activations(H, 1, 1001)[0])     # first use outside the capture
+    gpu.check(lib.salt_mi355_graph_begin(stream), "graph_begin")
+    for _ in range(4):
+        gpu.check(layer.enqueue(stream), "captured step")
+    graph = lib.salt_mi355_graph_end(stream)
+    assert graph, lib.salt_mi355_last_error().decode()
+    for it in range(4):
+        logits, x = synth.router_logits(E, 1010 + it), synth.activations(H, 1, 1020 + it)[0]
+        if it == 2:
+            logits = logits.copy(); logits[5] = np.nan                # a rejected step inside a replay
+        want = layer.step(logits, scale, x)                            # eager, also the work between replays
+        layer.out.upload(np.full(H, 7.0, np.float32))
+        gpu.check(lib.salt_mi355_graph_launch(graph, stream), "graph_launch")
+        gpu.check(lib.salt_mi355_stream_sync(stream), "sync")
+        status, out = int(layer.ws.to_host(np.int32, 1)[0]), layer.out.to_host(np.float32)
+        assert status == want[0] == (-1 if it == 2 else 0)
+        if it == 2:
+            assert (out == 7.0).all()
+        else:
+            assert np.array_equal(bits(out), bits(want[4])), it
+            assert np.array_equal(bits(layer.eo.to_host(np.float32).reshape(K, H)), bits(want[3]))
+    assert lib.salt_mi355_graph_destroy(graph) == 0
+
+
 def test_moe_decode_step_behind_a_pool_file_header(gpu, oracle):
     """Expert 0 starts 24 bytes into the allocation, as in the engine's pool file (three 64-bit header words): every
     tensor of every expert is then 8 bytes past a multiple of 16."""
