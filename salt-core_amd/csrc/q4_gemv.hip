@@ -188,13 +188,13 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
     Q4Job job;
+    const float *act_gate = nullptr, *act_up = nullptr;     // PRO >= 2: the activation row is gelu_tanh(gate) * up
     if (PRO == 0) {
         job = find_job(L, blockIdx.x);
     } else if (PRO == 3) {
         // the job's activation row is gelu_tanh(gate) * up of the two rows its x names: x[i] and x[i + act_delta]
         job = find_job(L, blockIdx.x);
-        const float *gate = job.x, *up = job.x + L.act_delta;
-        for (int i = tid; i < L.cols; i += THREADS) x_lds[i] = det_gelu_tanh(gate[i]) * up[i];
+        act_gate = job.x; act_up = job.x + L.act_delta;
     } else {
         const MoeFuse &m = L.moe;
         const size_t n = (size_t)m.hidden * (size_t)m.routed;
@@ -237,8 +237,7 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
             const int down_tiles = (m.hidden + TILE_ROWS - 1) / TILE_ROWS;
             const int place = (int)blockIdx.x / down_tiles;
             const int expert = ((const int __attribute__((address_space(4))) *)(uintptr_t)m.selected)[place];
-            const float *gate = m.gate + (size_t)place * m.routed, *up = m.up + (size_t)place * m.routed;
-            for (int i = tid; i < m.routed; i += THREADS) x_lds[i] = det_gelu_tanh(gate[i]) * up[i];
+            act_gate = m.gate + (size_t)place * m.routed; act_up = m.up + (size_t)place * m.routed;
             job.vals = m.pool + (size_t)expert * m.expert_stride + 2 * proj_bytes;
             job.x = nullptr;
             job.y = m.expert_out + (size_t)place * m.hidden;
@@ -356,6 +355,10 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
 
     if (tid == 0) slow_flag = 0;
     issue(0);
+    if (PRO >= 2) {
+        // after the first weights have been sent for: they are on their way while the activation is computed
+        for (int i = tid; i < L.cols; i += THREADS) x_lds[i] = det_gelu_tanh(act_gate[i]) * act_up[i];
+    }
     __syncthreads();
 
     const int my_row = lane < rows_here ? lane : rows_here - 1;
