@@ -19,7 +19,7 @@ reference's own C kernel when oracle/_ref is present (else the checker's
 port), and, under "extra", the same sweep on the bit-exact kernel, the MoE
 decode layer-step, the NVFP4 matvec and the batch-4 sweeps.
 
---only NAME runs a single leg (sweep, sweep-exact, sweep-b4, single, single-exact, moe, moe-t, prefill, abi, nvfp4-t, nvfp4-b256, copy): what the
+--only NAME runs a single leg (sweep, sweep-exact, sweep-b4, single, single-exact, moe, moe-t, prefill, ffn, abi, nvfp4-t, nvfp4-b256, copy): what the
 rocprofv3 commands in profiles/ use.
 """
 from __future__ import annotations
@@ -41,13 +41,13 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
 SWEEP = [(2816, 2816), (16384, 2816), (2816, 8192)]        # (R, C) = (N, K)
 INSTANCE_BYTES = 640e6                                      # distinct weight bytes per launch
-# HBM bytes one launch of the default workload moves (mean of the three launches), from FETCH_SIZE / WRITE_SIZE counter
-# runs scaled by a copy of known size; taken from the profile summary named beside it, for the default instance
-# counts only.  bench.py does not measure it: it reports it with its source.
+# HBM bytes one launch of the sweep moves (mean of the three launches), from FETCH_SIZE / WRITE_SIZE counter runs scaled
+# by a copy of known size; taken from the profile summary named beside it, for the default instance counts only, keyed
+# by kernel family and tokens per activation batch.  bench.py does not measure it: it reports it with its source.
 TRAFFIC_FROM_PROFILE = {
-    "q4_dot16_kernel": (650_800_000, "profiles/q4_dot_kernel_decode_sweep_b1.md"),
-    "q4_dot_kernel": (657_200_000, "profiles/q4_dot_kernel_decode_sweep_b1.md"),
-    "q4_tile_kernel": (661_320_000, "profiles/q4_tile_kernel_decode_sweep_b1.md"),
+    ("q4_dot16_kernel", 1): (651_200_000, "profiles/q4_dot16_kernel_decode_sweep.md"),
+    ("q4_dot16_kernel", 4): (656_300_000, "profiles/q4_dot16_kernel_decode_sweep.md"),
+    ("q4_tile_kernel", 1): (661_200_000, "profiles/q4_tile_kernel_decode_sweep_b1.md"),
 }
 
 
@@ -306,7 +306,7 @@ def sweep_record(lib, sweep, ms, steps, warmup):
     bytes_per_launch = sweep.bytes_per_step / launches
     launch_us = ms * 1e3 / launches
     kernel = lib.salt_mi355_last_kernel().decode()
-    traffic, source = TRAFFIC_FROM_PROFILE.get(kernel.split("<")[0], (None, None))
+    traffic, source = TRAFFIC_FROM_PROFILE.get((kernel.split("<")[0], sweep.tokens), (None, None))
     klass = ("bit-exact kernel" if sweep.exact else
              "tolerance-class kernel (|err| <= 2^-20 sum (|q s| + 16|s| + |b|)|x| + 1e-6 per output)")
     return {
@@ -441,6 +441,38 @@ def nvfp4_b256_leg(gpu, synth, lib, stream, events, w, scales_at, st, R, Cc):
             "nvfp4_8192_b256_mfma_frac": round(2.0 * R * Cc * B / (ms_mm * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
 
 
+def ffn_leg(gpu, synth, lib, stream, events, pool, E, K, H, F):
+    out = {}
+    # the whole feed-forward block of a decoder layer for one token: pre-norms, dense FFN (2112 wide), router input,
+    # 8-bit gate, top-8 of 128, routed experts, parallel combine -- bit-exact, device-resident.  32 residuals taken
+    # in turn: the routing, hence the experts read, changes from block to block.
+    block = gpu.FfnBlock(synth.ffn_layer(H, 2112, F, E, K, 70, pool=pool))
+    residuals = [gpu.DeviceBuffer.from_host((synth.activations(H, 1, 71 + k)[0] * 3).astype(np.float32))
+                 for k in range(32)]
+    ffn_turn = [0]
+
+    def ffn_step(st):
+        block.residual = residuals[ffn_turn[0] % len(residuals)]
+        ffn_turn[0] += 1
+        if block.enqueue(st) != 0:
+            raise RuntimeError(lib.salt_mi355_last_error().decode())
+
+    ms_ffn = timed(lib, stream, events, ffn_step, 5, 100)
+    if int(block.status.to_host(np.int32)[0]) != 0:
+        raise RuntimeError("the feed-forward block rejected its input")
+    out["ffn_block_us"] = round(ms_ffn * 1e3, 2)
+    out["ffn_block_layer_tokens_per_s"] = round(1e3 / ms_ffn, 1)
+    # the same block captured once and replayed as a HIP graph
+    if lib.salt_mi355_graph_begin(stream) == 0:              # one residual: a graph replays fixed pointers
+        ffn_step(stream)
+        graph = lib.salt_mi355_graph_end(stream)
+        if graph:
+            ms_g = timed(lib, stream, events, lambda st: lib.salt_mi355_graph_launch(graph, st), 5, 100)
+            out["ffn_block_graph_us"] = round(ms_g * 1e3, 2)
+            lib.salt_mi355_graph_destroy(graph)
+    return out
+
+
 def abi_leg(synth, lib, pool, H, F, K):
     """The engine-facing ABI with host pointers: per-call latency of salt_gpu_q4_matvec and salt_gpu_q4_moe_chain."""
     out = {}
@@ -512,6 +544,8 @@ def run_only(args, gpu, synth, lib, stream, events):
     if args.only in ("moe", "moe-t"):
         pool = synth.expert_pool(128, 2816, 704, 7)
         return moe_leg(gpu, synth, lib, stream, events, pool, args.only == "moe-t")
+    if args.only == "ffn":
+        return ffn_leg(gpu, synth, lib, stream, events, synth.expert_pool(128, 2816, 704, 7), 128, 8, 2816, 704)
     if args.only == "abi":
         return abi_leg(synth, lib, synth.expert_pool(128, 2816, 704, 7), 2816, 704, 8)
     if args.only == "prefill":
@@ -555,7 +589,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the MoE / NVFP4 / batch-4 legs")
-    ap.add_argument("--only", default="", help="run one leg: sweep | sweep-exact | sweep-b4 | sweep-b4-exact | single | single-exact | moe | moe-t | prefill | abi | nvfp4-t | nvfp4-b256 | copy")
+    ap.add_argument("--only", default="", help="run one leg: sweep | sweep-exact | sweep-b4 | sweep-b4-exact | single | single-exact | moe | moe-t | prefill | ffn | abi | nvfp4-t | nvfp4-b256 | copy")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU mode (run with --gpus 1)")
@@ -618,34 +652,7 @@ def main():
             extra["moe_launch_skeleton_us"] = round(ms_sk * 1e3, 2)
             ms_sk1 = timed(lib, stream, events, lambda st: lib.salt_mi355_launch_skeleton_dev(128, 512, 0, 0, 0, 0, st), 5, 200)
             extra["single_launch_skeleton_us"] = round(ms_sk1 * 1e3, 2)
-        # the whole feed-forward block of a decoder layer for one token: pre-norms, dense FFN (2112 wide), router input,
-        # 8-bit gate, top-8 of 128, routed experts, parallel combine -- bit-exact, device-resident.  32 residuals taken
-        # in turn: the routing, hence the experts read, changes from block to block.
-        block = gpu.FfnBlock(synth.ffn_layer(H, 2112, F, E, K, 70, pool=pool))
-        residuals = [gpu.DeviceBuffer.from_host((synth.activations(H, 1, 71 + k)[0] * 3).astype(np.float32))
-                     for k in range(32)]
-        ffn_turn = [0]
-
-        def ffn_step(st):
-            block.residual = residuals[ffn_turn[0] % len(residuals)]
-            ffn_turn[0] += 1
-            if block.enqueue(st) != 0:
-                raise RuntimeError(lib.salt_mi355_last_error().decode())
-
-        ms_ffn = timed(lib, stream, events, ffn_step, 5, 100)
-        if int(block.status.to_host(np.int32)[0]) != 0:
-            raise RuntimeError("the feed-forward block rejected its input")
-        extra["ffn_block_us"] = round(ms_ffn * 1e3, 2)
-        extra["ffn_block_layer_tokens_per_s"] = round(1e3 / ms_ffn, 1)
-        # the same block captured once and replayed as a HIP graph
-        if lib.salt_mi355_graph_begin(stream) == 0:              # one residual: a graph replays fixed pointers
-            ffn_step(stream)
-            graph = lib.salt_mi355_graph_end(stream)
-            if graph:
-                ms_g = timed(lib, stream, events, lambda st: lib.salt_mi355_graph_launch(graph, st), 5, 100)
-                extra["ffn_block_graph_us"] = round(ms_g * 1e3, 2)
-                lib.salt_mi355_graph_destroy(graph)
-        del block, residuals
+        extra.update(ffn_leg(gpu, synth, lib, stream, events, pool, E, K, H, F))
         # BASELINE configs[0]: one 4096 x 4096 Q4 matvec per launch, batch 1, rotating through 64 weight instances (606 MB)
         R = Cc = 4096
         vals, scales, biases = synth.q4_tensor(R, Cc, 60)
