@@ -751,7 +751,8 @@ int salt_mi355_moe_decode_step_static_dev(const void *pool, size_t expert_stride
     MoeWorkspace ws;
     moe_workspace_carve(g, scratch, &ws);
     // Every word of the workspace that a launch reads is written earlier in the same step (the status word by the
-    // router, the job tables and the intermediate vectors by their producers): nothing has to start at zero.
+    // router, the job tables and the intermediate vectors by their producers, the tile counters of the ordered sum by
+    // the first launch): nothing has to start at zero.
     if (status_dev) ws.status = status_dev;
     if (moe_decode_step_launch(g, (const uint8_t *)pool, expert_stride, logits, per_expert_scale, x, selected, weights,
                                expert_out, out, ws, g_state.code_scale, (hipStream_t)stream) != 0) {
