@@ -173,3 +173,48 @@ def test_random_tolerance_class_launches(gpu, oracle, stream_seed):
             want = q4_want(oracle, v, s_, b, R, Cc, xs[j])
             check_class_t(got, want, v, s_, b, R, Cc, xs[j])
     print("kernels reached:", sorted(kernels), flush=True)
+
+
+def test_random_tolerance_class_launches_of_many_blocks(gpu, oracle):
+    """The same entry point at launches of at least 2048 blocks, which the sixteen-row kernel serves: 24..70 jobs of
+    ragged row counts, 1..9 tokens (passes inside one launch beyond four, two column windows for wide rows at three or
+    four), three sampled jobs per launch inside the stated bound."""
+    lib = gpu.init()
+    rng = np.random.default_rng(21)
+    kernels = set()
+    for case in range(10):
+        Cc = 64 * int(rng.integers(8, 129))
+        tokens = int(rng.integers(1, 10))
+        njobs = int(rng.choice([24, 33, 40, 70]))
+        lo = 70000 // njobs
+        rows = [int(rng.integers(lo, lo + 1500)) for _ in range(njobs)]
+        seed = int(rng.integers(1, 1 << 30))
+        offset = int(rng.choice([0, 4, 8]))
+        with_bias = bool(rng.random() < 0.8)
+        tensors = [synth.q4_tensor(max(rows), Cc, seed + k) for k in range(2)]
+        dev = []
+        for vals, scales, biases in tensors:
+            dv = gpu.DeviceBuffer(vals.nbytes + offset + 16, fill=0)
+            dv.upload(vals, offset)
+            dev.append((dv, gpu.DeviceBuffer.from_host(scales), gpu.DeviceBuffer.from_host(biases)))
+        xs = [synth.activations(Cc, tokens, seed + 10 + (j % 5)) for j in range(njobs)]
+        dxs = [gpu.DeviceBuffer.from_host(x) for x in xs]
+        dys = [gpu.DeviceBuffer(tokens * R * 4, fill=0xFF) for R in rows]
+        jobs = (gpu.Q4Job * njobs)()
+        for j, R in enumerate(rows):
+            dv, ds, db = dev[j % len(dev)]
+            jobs[j] = gpu.Q4Job(dv.at(offset), ds.ptr, db.ptr if with_bias else None, dxs[j].ptr, dys[j].ptr, R)
+        print("class T, many blocks", Cc, tokens, njobs, sum(rows), offset, with_bias, seed, flush=True)
+        stream = lib.salt_mi355_stream()
+        gpu.check(lib.salt_mi355_q4_jobs_t_dev(jobs, njobs, Cc, tokens, stream), "q4_jobs_t_dev")
+        gpu.check(lib.salt_mi355_stream_sync(stream), "sync")
+        kernels.add(lib.salt_mi355_last_kernel().decode())
+        for j in sorted({0, njobs // 2, njobs - 1}):
+            vals, scales, biases = tensors[j % len(tensors)]
+            R = rows[j]
+            v, s_, b = vals[:R * Cc // 8], scales[:R * Cc // 64], (biases[:R * Cc // 64] if with_bias else None)
+            got = dys[j].to_host(np.float32).reshape(tokens, R)
+            check_class_t(got, q4_want(oracle, v, s_, b, R, Cc, xs[j]), v, s_, b, R, Cc, xs[j])
+        del dev, dxs, dys
+    print("kernels reached:", sorted(kernels), flush=True)
+    assert all(k.startswith("q4_dot16_kernel<") for k in kernels)
