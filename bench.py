@@ -495,12 +495,40 @@ def abi_leg(synth, lib, pool, H, F, K):
             if lib.salt_gpu_q4_matvec(base, base + v0.nbytes, base + v0.nbytes + s0.nbytes, R0, C0,
                                       x0.ctypes.data, y0.ctypes.data) != 0:
                 raise RuntimeError(lib.salt_mi355_last_error().decode())
-        for _ in range(5):
-            abi_call()
-        t0 = time.perf_counter()
-        for _ in range(200):
-            abi_call()
-        out["abi_q4_matvec_4096_host_pointers_us"] = round((time.perf_counter() - t0) / 200 * 1e6, 1)
+        def per_call_us(call, warm, reps=200):
+            for _ in range(warm):
+                call()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                call()
+            return round((time.perf_counter() - t0) / reps * 1e6, 1)
+
+        out["abi_q4_matvec_4096_host_pointers_us"] = per_call_us(abi_call, 5)
+        # the same call after the engine has opted into the tolerance class (salt_mi355_set_tolerance_class)
+        lib.salt_mi355_set_tolerance_class(1)
+        out["abi_q4_matvec_4096_host_pointers_class_t_us"] = per_call_us(abi_call, 5)
+        lib.salt_mi355_set_tolerance_class(0)
+        # defer mode (salt_gpu_set_defer): a hundred calls enqueued, one salt_gpu_sync at the end -- what a call costs when
+        # the engine does not wait for each result
+        lib.salt_gpu_set_defer.argtypes = [C.c_int]
+
+        def deferred_us(reps=100):
+            lib.salt_gpu_set_defer(1)
+            for _ in range(5):
+                abi_call()
+            lib.salt_gpu_sync()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                abi_call()
+            lib.salt_gpu_sync()
+            us = (time.perf_counter() - t0) / reps * 1e6
+            lib.salt_gpu_set_defer(0)
+            return round(us, 1)
+
+        out["abi_q4_matvec_4096_deferred_us"] = deferred_us()
+        lib.salt_mi355_set_tolerance_class(1)
+        out["abi_q4_matvec_4096_deferred_class_t_us"] = deferred_us()
+        lib.salt_mi355_set_tolerance_class(0)
         lib.salt_gpu_weight_resource_deactivate(1, 900)
         # the engine's decode call for the routed experts: salt_gpu_q4_moe_chain over eight experts, one row each
         import engine_abi
@@ -523,12 +551,10 @@ def abi_leg(synth, lib, pool, H, F, K):
                 if eabi.salt_gpu_q4_moe_chain(recs, K, H, F, xin.ctypes.data, yout.ctypes.data, scr[0].ctypes.data,
                                               scr[1].ctypes.data, K * F) != 0:
                     raise RuntimeError(lib.salt_mi355_last_error().decode())
-            for _ in range(20):
-                chain_call()
-            t0 = time.perf_counter()
-            for _ in range(200):
-                chain_call()
-            out["abi_q4_moe_chain_8_experts_us"] = round((time.perf_counter() - t0) / 200 * 1e6, 1)
+            out["abi_q4_moe_chain_8_experts_us"] = per_call_us(chain_call, 20)
+            lib.salt_mi355_set_tolerance_class(1)
+            out["abi_q4_moe_chain_8_experts_class_t_us"] = per_call_us(chain_call, 20)
+            lib.salt_mi355_set_tolerance_class(0)
             eabi.salt_gpu_expert_resource_unbind(901)
     return out
 
