@@ -376,10 +376,16 @@ int salt_mi355_moe_decode_step_dev(const void *pool, size_t expert_stride,
  * are bit-identical to the reference; the three projections of every selected
  * expert run on the kernel of salt_mi355_q4_matvec_t_dev (its bound applies to
  * each projection against its own input), gelu_tanh and the ordered weighted
- * sum are the reference's.  Stated tolerance of the composition (tests):
- * |expert_out - ref| <= 2^-15 * max_d |ref[expert]| + 1e-6, the same for out.
+ * sum are the reference's.  Stated tolerance of the composition (tests), per
+ * output and relative to the magnitudes of the output's own terms, with
+ * h_k = gelu_tanh(gate_k) * up_k and Wd_k the dequantised down projection:
+ *   |expert_out[k][d] - ref| <= 2^-18 * sum_f |Wd_k[d][f] * h_k[f]| + 1e-6,
+ *   |out[d] - ref| <= 2^-18 * sum_k |w_k| * sum_f |Wd_k[d][f] * h_k[f]| + 1e-6.
  * Same arguments and workspace as salt_mi355_moe_decode_step_dev; more than
- * 256 experts or widths outside 512..4096 take the bit-exact plan. */
+ * 256 experts or widths the streaming kernels do not take (fewer than 512
+ * columns, more than 8192) run the bit-exact plan.  As for every
+ * tolerance-class entry point the bits depend on the launch (here: on the
+ * geometry), not on the run. */
 int salt_mi355_moe_decode_step_t_dev(const void *pool, size_t expert_stride,
                                      int hidden, int routed, int n_experts, int topk,
                                      const float *logits, const float *per_expert_scale,

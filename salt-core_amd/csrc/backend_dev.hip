@@ -639,10 +639,14 @@ int salt_mi355_moe_decode_step_t_dev(const void *pool, size_t expert_stride, int
     }
     MoeWorkspace ws;
     moe_workspace_carve(g, workspace, &ws);
-    if (moe_decode_step_t_launch(g, (const uint8_t *)pool, expert_stride, logits, per_expert_scale, x, selected, weights,
-                                 expert_out, out, ws, (hipStream_t)stream) == 0)
-        return 0;
-    (void)hipGetLastError();
+    const int served = moe_decode_step_t_launch(g, (const uint8_t *)pool, expert_stride, logits, per_expert_scale, x,
+                                                selected, weights, expert_out, out, ws, (hipStream_t)stream);
+    if (served == 0) return 0;
+    if (served != MOE16_NOT_SERVED) {
+        set_error("moe step t: a launch failed: %s", hipGetErrorString(hipGetLastError()));
+        return -1;
+    }
+    // a geometry the streaming kernels do not take: the bit-exact plan, whose result is inside any tolerance
     return salt_mi355_moe_decode_step_dev(pool, expert_stride, hidden, routed, n_experts, topk, logits, per_expert_scale,
                                           x, selected, weights, expert_out, out, workspace, stream);
 }

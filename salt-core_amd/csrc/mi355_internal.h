@@ -137,6 +137,7 @@ int q4_dot16_window_waves(int cols, int tokens, long long total_blocks32);
 int moe_static_scratch_prepare();      // backend_dev.hip: looks up the static MoE workspace of the current device
 constexpr int MOE16_NOT_SERVED = 1;
 int moe16_step_launch(const MoeFuse &moe, float *out, hipStream_t stream);
+bool q4_dot_moe_serves(const MoeFuse &moe);
 int q4_dot_moe_gate_up_launch(const MoeFuse &moe, hipStream_t stream);
 int q4_dot_moe_down_launch(const MoeFuse &moe, hipStream_t stream);
 

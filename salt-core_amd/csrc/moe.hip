@@ -213,6 +213,7 @@ int moe_decode_step_launch(const MoeGeometry &g, const uint8_t *pool, size_t exp
 // The same step on the tolerance-class matvec kernels: router top-k (bit-exact), gate and up, gelu_tanh(gate) * up,
 // down, ordered weighted sum.  Two launches where moe_dot16.hip serves the geometry (the activation rides in the
 // first, the weighted sum in the second), else three launches on the 32-row kernel with the sum on its own.
+// Returns 0, MOE16_NOT_SERVED when neither plan takes the geometry (nothing was launched), or -1 when a launch failed.
 int moe_decode_step_t_launch(const MoeGeometry &g, const uint8_t *pool, size_t expert_stride, const float *logits,
                              const float *per_expert_scale, const float *x, int *selected, float *weights,
                              float *expert_out, float *out, const MoeWorkspace &ws, hipStream_t stream) {
@@ -230,6 +231,7 @@ int moe_decode_step_t_launch(const MoeGeometry &g, const uint8_t *pool, size_t e
         if (served == 0) return 0;
         if (served != MOE16_NOT_SERVED) return -1;    // a launch failed: nothing to fall back on
     }
+    if (!q4_dot_moe_serves(m)) return MOE16_NOT_SERVED;   // nothing launched: the caller takes the bit-exact plan
     if (q4_dot_moe_gate_up_launch(m, stream) != 0) return -1;
     if (q4_dot_moe_down_launch(m, stream) != 0) return -1;
     return out ? moe_reduce_launch(m.expert_out, weights, g.topk, g.hidden, out, ws.status, stream) : 0;

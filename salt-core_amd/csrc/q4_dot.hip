@@ -583,6 +583,12 @@ static bool moe_dot_geometry_ok(const MoeFuse &m) {
            q4_dot_takes(m.hidden) && q4_dot_takes(m.routed) && m.hidden <= 4096 && m.routed <= 4096;
 }
 
+// Whether q4_dot_moe_gate_up_launch and q4_dot_moe_down_launch serve this geometry (a refusal there is then a failure).
+bool q4_dot_moe_serves(const MoeFuse &m) {
+    return moe_dot_geometry_ok(m) && dot_lds_bytes(m.hidden, 1, 4, 2) <= DOT_LDS_LIMIT &&
+           dot_lds_bytes(m.routed, 1, 4, 2) <= DOT_LDS_LIMIT;
+}
+
 static int moe_dot_ksplit(long long blocks, int cols) {
     const int nstage = dot_steps(cols >> 6);
     int ksplit = 1;

@@ -517,7 +517,7 @@ __global__ __launch_bounds__((32 / S) * 64) void q4_tile_kernel(const Q4Launch L
             // do not see), ordered by waiting for the stores before the count and for the count before the loads: a
             // fence would write the whole cache back, once per workgroup.
             const MoeFuse &m = L.moe;
-            float *const mine = m.expert_out + (size_t)(job.y - m.expert_out) + row0;
+            float *const mine = job.y + row0;                 // this expert's rows of expert_out
             if (lane < rows_here) __hip_atomic_store(mine + lane, even + odd, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             int before = 0;
@@ -661,7 +661,7 @@ int q4_moe_down_launch(const Q4Launch &launch, hipStream_t stream) {
     Q4Launch L = launch;
     const MoeFuse &m = L.moe;
     if (m.topk < 1 || m.hidden < 64 || (m.hidden & 63) || m.routed < 64 || (m.routed & 63) ||
-        m.routed > MOE_FUSE_MAX_ROUTED)
+        m.routed > MOE_FUSE_MAX_ROUTED || (m.out == nullptr) != (m.arrivals == nullptr))
         return -1;
     L.table = nullptr; L.njobs = 1; L.cols = m.routed; L.tokens = 1;
     L.total_tiles = m.topk * ((m.hidden + TILE_ROWS - 1) / TILE_ROWS);
