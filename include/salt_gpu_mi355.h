@@ -163,7 +163,9 @@ int salt_mi355_q4_jobs_t_dev(const SaltMi355Q4Job *jobs, int njobs, int C, int t
 
 /* Prefill-sized variant on the matrix cores: ys[t*R + r] for B tokens against
  * one matrix, fp32-accurate but NOT bit-identical to the reference (different
- * summation order): |error| <= 2^-18 * sum_c |w*x| + 1e-6 per output.  Needs
+ * summation order): per output
+ *   |error| <= 2^-20 * sum_c (|q_c s| + 16 |s| + |b|) |x_c| + 1e-6
+ * (and <= 2^-18 * sum_c |w*x| + 1e-6 for activations without outliers).  Needs
  * C % 64 == 0 and device scratch of salt_mi355_q4_matmul_workspace_bytes().
  * The reference has no counterpart: its CPU and GPU paths keep the 32-chain
  * order at every batch size (kernels.c:1252-1261). */
