@@ -433,6 +433,15 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
         job.scales = job.vals + vals_bytes;
         job.biases = job.scales + meta_bytes;
     }
+    // Plain launches: the activations are sent for first and the weights when they have arrived, so that the digit
+    // planes are built while the weights are on their way (weights first, activations queued behind them, cost a
+    // launch of one matrix up to a microsecond).
+    const ImageItems items(T, ngrp);
+    Q4ImageBuilder<THREADS> image;
+    if (PRO == 0) {
+        image.request_early(tid, items, [&](int t) { return job.x + (size_t)t * job.x_stride; });
+        image.settle(0, items);
+    }
     if (has_rows) {
 #pragma unroll
         for (int b = 0; b < NB; ++b)
@@ -441,7 +450,15 @@ __global__ __launch_bounds__(WAVES * 64) void q4_dot_kernel(const Q4DotLaunch L)
         for (int g = 0; g < STAGES; ++g)
             if (g < total_steps) issue_step(block_of(g), step_of(g), g);
     }
-    if (PRO != 1) build_image();
+    if (PRO == 0) {
+        image.build(tid, items, SG, zero_lds, img_lds, xm_lds, [&](int t, size_t column, float (&xv)[8]) {
+            const float *src = job.x + (size_t)t * job.x_stride + column;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) xv[k] = src[k];
+        });
+    } else if (PRO != 1) {
+        build_image();
+    }
     __syncthreads();
     if (has_rows) {
 #pragma unroll
