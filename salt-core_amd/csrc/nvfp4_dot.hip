@@ -240,32 +240,56 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_dot_kernel(const Fp4DotLaunch 
     // ---------------------------------------------------------------- activation quantisation (all waves)
     // One thread per 16-column block: the reference's group-16 quantiser with closed-form encoders.  A unit of 32
     // columns is stored twice 16 bytes: block 0's codes followed by zero codes, and zero codes followed by block 1's.
+    //
+    // The first FP4_HELD blocks of every thread are fetched by request_blocks() before the weight loads go out and
+    // waited for there: the weights then queue behind nothing, and the quantiser runs while they are on their way.
+    // (Fetched after the weights, the activations are the youngest loads in flight and waiting for them waits for the
+    // weights as well.)
+    constexpr int FP4_HELD = 2;
+    const int items = T * 2 * units;
+    float held[FP4_HELD][16];
+    auto fetch_block = [&](int item, float (&v)[16]) {
+        const int blk = item % (2 * units);
+        const int t = item / (2 * units);
+#pragma unroll
+        for (int q = 0; q < 16; ++q) v[q] = 0.0f;
+        if (item < items && blk * 16 < C) {
+            const float4 *src = reinterpret_cast<const float4 *>(job.x + (size_t)t * job.x_stride + (size_t)blk * 16);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float4 f = src[q];
+                v[4 * q] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w;
+            }
+        }
+    };
+    auto request_blocks = [&]() {
+#pragma unroll
+        for (int k = 0; k < FP4_HELD; ++k) fetch_block(tid + k * THREADS, held[k]);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    };
+    auto store_block = [&](int item, const float (&v)[16]) {
+        const int blk = item % (2 * units);
+        const int t = item / (2 * units);
+        uint32_t codes[2] = {0u, 0u};
+        float from_code = 0.0f;
+        if (blk * 16 < C && !fp4_quantise_block(v, L.input_global_scale, codes, from_code)) *bad_lds = 1;
+        uint32_t *slot = (uint32_t *)(img_lds + ((size_t)(t * units + (blk >> 1)) * 2 + (blk & 1)) * 16);
+        const bool second = blk & 1;
+        slot[0] = second ? 0u : codes[0]; slot[1] = second ? 0u : codes[1];
+        slot[2] = second ? codes[0] : 0u; slot[3] = second ? codes[1] : 0u;
+        xs_lds[(size_t)t * 2 * units + blk] = from_code;
+    };
     auto build_image = [&]() {
         for (int i = tid; i < FP4_ZERO_BYTES / 4; i += THREADS) ((uint32_t *)zero_lds)[i] = 0u;
         if (tid == 0) *bad_lds = 0;
         __syncthreads();
-        const int items = T * 2 * units;
-        for (int item = tid; item < items; item += THREADS) {
-            const int blk = item % (2 * units);
-            const int t = item / (2 * units);
-            const bool valid = blk * 16 < C;
-            uint32_t codes[2] = {0u, 0u};
-            float from_code = 0.0f;
-            if (valid) {
-                const float4 *src = reinterpret_cast<const float4 *>(job.x + (size_t)t * job.x_stride + (size_t)blk * 16);
-                float v[16];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float4 f = src[q];
-                    v[4 * q] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w;
-                }
-                if (!fp4_quantise_block(v, L.input_global_scale, codes, from_code)) *bad_lds = 1;
-            }
-            uint32_t *slot = (uint32_t *)(img_lds + ((size_t)(t * units + (blk >> 1)) * 2 + (blk & 1)) * 16);
-            const bool second = blk & 1;
-            slot[0] = second ? 0u : codes[0]; slot[1] = second ? 0u : codes[1];
-            slot[2] = second ? codes[0] : 0u; slot[3] = second ? codes[1] : 0u;
-            xs_lds[(size_t)t * 2 * units + blk] = from_code;
+        for (int k = 0; k < FP4_HELD; ++k)
+            if (tid + k * THREADS < items) store_block(tid + k * THREADS, held[k]);
+        for (int item = tid + FP4_HELD * THREADS; item < items; item += THREADS) {
+            float v[16];
+            fetch_block(item, v);
+            store_block(item, v);
         }
     };
 
@@ -298,6 +322,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_dot_kernel(const Fp4DotLaunch 
     // ---------------------------------------------------------------- main loop (as in q4_dot.hip)
     const int first_step = total_steps > 0 ? (int)(((unsigned)blockIdx.x * WAVES + wave) % (unsigned)total_steps) : 0;
     auto step_of = [&](int g) { const int st = g + first_step; return step_lo + (st < total_steps ? st : st - total_steps); };
+    request_blocks();
     if (has_rows) {
         issue_meta();
 #pragma unroll
