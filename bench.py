@@ -45,8 +45,8 @@ INSTANCE_BYTES = 640e6                                      # distinct weight by
 # by a copy of known size; taken from the profile summary named beside it, for the default instance counts only, keyed
 # by kernel family and tokens per activation batch.  bench.py does not measure it: it reports it with its source.
 TRAFFIC_FROM_PROFILE = {
-    ("q4_dot16_kernel", 1): (651_200_000, "profiles/q4_dot16_kernel_decode_sweep.md"),
-    ("q4_dot16_kernel", 4): (656_300_000, "profiles/q4_dot16_kernel_decode_sweep.md"),
+    ("q4_dot16_kernel", 1): (650_600_000, "profiles/q4_dot16_kernel_decode_sweep.md"),
+    ("q4_dot16_kernel", 4): (656_500_000, "profiles/q4_dot16_kernel_decode_sweep.md"),
     ("q4_tile_kernel", 1): (661_200_000, "profiles/q4_tile_kernel_decode_sweep_b1.md"),
 }
 
@@ -655,7 +655,7 @@ def main():
         # batch 4 of the same sweep, both kernels
         for name, exact in (("q4_sweep_batch4_class_t_gbps", False), ("q4_sweep_batch4_bit_exact_gbps", True)):
             s4 = Q4Sweep(gpu, synth, tokens=4, exact=exact)
-            ms4 = timed(lib, stream, events, s4.step, 2, max(5, args.steps // 5))
+            ms4 = timed(lib, stream, events, s4.step, args.warmup, args.steps)
             extra[name] = round(s4.bytes_per_step / (ms4 * 1e-3) / 1e9, 1)
             del s4
         # the same batch-1 launches with every job reading one of two weight instances per shape (87 MB in all):
