@@ -147,7 +147,7 @@ int salt_mi355_nvfp4_matmul_dev(const void *packed, const void *scales, float st
     memset(&launch, 0, sizeof launch);
     launch.packed = (const uint8_t *)packed; launch.scales = (const uint8_t *)scales;
     launch.plane = w.plane; launch.ys = ys; launch.partials = w.partials; launch.status = w.status;
-    launch.flags = w.flags; launch.nflags = w.nflags; launch.verdict = w.status; launch.verdict_copy = status_dev;
+    launch.flags = w.flags; launch.nflags = w.nflags; launch.outcome = w.status; launch.outcome_copy = status_dev;
     launch.rows = R; launch.cols = C; launch.tokens = B; launch.ksplit = fp4_mfma_splits(R, C, B);
     launch.out_scale = (1.0f / stored_divisor) / input_global_scale;
     if (fp4_mfma_launch(launch, s) != 0) { set_error("nvfp4 matmul: launch failed"); return -1; }

@@ -248,11 +248,11 @@ struct Fp4MfmaLaunch {
     float *ys;                // [tokens][rows]
     float *partials;          // [ksplit][tokens][rows], used when ksplit > 1
     const int *status;        // nothing is published unless *status == 0 ...
-    // ... or, when flags is set, unless all nflags words are 0; the launch then writes the verdict (0 or -1) to
-    // verdict and, when set, verdict_copy, and `status` is not read
+    // ... or, when flags is set, unless all nflags words are 0; the launch then writes the outcome (0 or -1) to
+    // outcome and, when set, outcome_copy, and `status` is not read
     const int *flags;
     int nflags;
-    int *verdict, *verdict_copy;
+    int *outcome, *outcome_copy;
     int rows, cols, tokens, ksplit;
     float out_scale;
 };

@@ -41,15 +41,15 @@ struct Geometry {
 };
 
 // Whether the activation pass rejected its input: the launch's status word, or the OR of the pass's per-workgroup
-// flags (every thread of the workgroup calls this; workgroup 0 then also publishes the verdict).
+// flags (every thread of the workgroup calls this; workgroup 0 then also publishes the outcome).
 __device__ __forceinline__ bool rejected(const Fp4MfmaLaunch &L) {
     if (!L.flags) return *(const int __attribute__((address_space(4))) *)(uintptr_t)L.status != 0;
     int bad = 0;
     for (int i = threadIdx.x; i < L.nflags; i += blockDim.x) bad |= L.flags[i];
     const int any_bad = __syncthreads_or(bad);
     if (blockIdx.x == 0 && threadIdx.x == 0) {
-        *L.verdict = any_bad ? -1 : 0;
-        if (L.verdict_copy) *L.verdict_copy = any_bad ? -1 : 0;
+        *L.outcome = any_bad ? -1 : 0;
+        if (L.outcome_copy) *L.outcome_copy = any_bad ? -1 : 0;
     }
     return any_bad != 0;
 }
@@ -222,7 +222,7 @@ int fp4_mfma_splits(int rows, int cols, int tokens) {
 
 int fp4_mfma_launch(const Fp4MfmaLaunch &L, hipStream_t stream) {
     if (L.rows < 1 || L.tokens < 1 || L.cols < KC || (L.cols % KC) || L.ksplit < 1) return -1;
-    if (L.flags ? (L.nflags < 1 || !L.verdict) : !L.status) return -1;
+    if (L.flags ? (L.nflags < 1 || !L.outcome) : !L.status) return -1;
     Geometry G;
     G.m_tiles = (L.tokens + TM - 1) / TM;
     G.n_tiles = (L.rows + TN - 1) / TN;
